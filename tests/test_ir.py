@@ -1,0 +1,142 @@
+"""Host-side IR, builder API, wire format and model zoo."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import ios
+from ios.ir import Conv, Graph, Identity, Pool, Sequential, Value
+
+GOLDEN = os.path.join(os.path.dirname(__file__), 'golden')
+
+
+def test_sample_network_shapes_and_pretty_print():
+    graph = ios.models.sample_network()
+    assert tuple(graph.exit_node.output_shape) == (1875, 15, 15)    # README output shape
+    graph.sequential_schedule()
+    # text printed by the reference README for the sequential schedule of this network
+    assert str(graph) == ("Sequential(\n  [1]Conv2d(0)\n  [2]Conv2d(0)\n  [3]Conv2d(0)\n  [4]Conv2d(1)\n"
+                          "  [5]Concat(4,2,3)\n)")
+    graph.blocks[0].stages = [[['1'], ['2']], [['4'], ['3']], [['5']]]
+    assert str(graph) == ("Sequential(\n  Parallel(\n    [1]Conv2d(0)\n    [2]Conv2d(0)\n  )\n  Parallel(\n"
+                          "    [4]Conv2d(1)\n    [3]Conv2d(0)\n  )\n  [5]Concat(4,2,3)\n)")
+
+
+def test_inception_v3_topology():
+    graph = ios.models.inception_v3()
+    nodes = list(graph.nodes())
+    assert [n.name for n in nodes] == [str(i) for i in range(120)]
+    assert len(graph.blocks) == 13
+    assert len(graph.conv_nodes()) == 94
+    assert sum(isinstance(n, Pool) for n in nodes) == 14
+    assert sum(isinstance(n, Identity) for n in nodes) == 11
+    by_name = {n.name: n for n in nodes}
+    # spatial sizes of the stem: 149, 147, 147, 73, 73, 71, 35
+    assert [by_name[str(i)].output_shape[1] for i in range(1, 8)] == [149, 147, 147, 73, 73, 71, 35]
+    exits = [tuple(b.exit_node.output_shape) for b in graph.blocks]
+    assert exits == [(192, 35, 35), (256, 35, 35), (288, 35, 35), (288, 35, 35), (768, 17, 17), (768, 17, 17),
+                     (768, 17, 17), (768, 17, 17), (768, 17, 17), (1280, 8, 8), (2048, 8, 8), (2048, 8, 8),
+                     (2048, 1, 1)]
+    macs = sum(np.prod(c.output_shape) * c.fan_in for c in graph.conv_nodes())
+    assert macs == pytest.approx(5.711e9, rel=2e-3)
+    weights = sum(np.prod(c.weight_shape) for c in graph.conv_nodes()) * 4
+    assert weights == pytest.approx(87.07e6, rel=2e-3)
+
+
+def test_inception_schedule_fixture_round_trip():
+    # a schedule document of the shape the reference exports for an optimised Inception-v3 (merged convs,
+    # channel-slice inputs, multi-group stages); it was produced by this package's optimizer
+    with open(os.path.join(GOLDEN, 'inception_v3_dp_parallel_merge.json')) as f:
+        config = json.load(f)
+    graph = Graph.from_config(config)
+    assert json.loads(json.dumps(graph.export_config())) == config
+    assert tuple(graph.exit_node.output_shape) == (2048, 1, 1)
+    plain = {n.name: n for n in ios.models.inception_v3().nodes()}
+    seen = set()
+    for node in graph.nodes():
+        seen.update(node.hint_name.split())
+        if ' ' not in node.hint_name and node.name in plain and node.type == 'conv':
+            ref = plain[node.name]
+            assert (node.out_channels, tuple(node.kernel), tuple(node.stride), tuple(node.padding)) == \
+                   (ref.out_channels, tuple(ref.kernel), tuple(ref.stride), tuple(ref.padding))
+    assert seen == {str(i) for i in range(120)}
+
+
+def test_config_round_trip_all_models():
+    for make in (ios.models.sample_network, ios.models.squeezenet_1_1, ios.models.squeezenet,
+                 ios.models.randwire_small, ios.models.nasnet_mobile):
+        graph = make()
+        graph.sequential_schedule()
+        config = json.loads(json.dumps(graph.export_config()))
+        again = Graph.from_config(config)
+        assert json.loads(json.dumps(again.export_config())) == config
+
+
+def test_model_output_shapes():
+    assert tuple(ios.models.squeezenet_1_1().exit_node.output_shape) == (1000, 1, 1)
+    sq = ios.models.squeezenet_1_1()
+    assert [tuple(b.exit_node.output_shape) for b in sq.blocks][:4] == [(64, 55, 55), (128, 55, 55), (128, 55, 55), (128, 27, 27)]
+    rw = ios.models.randwire_small()
+    assert [tuple(b.exit_node.output_shape) for b in rw.blocks] == [(78, 56, 56), (78, 28, 28), (156, 14, 14),
+                                                                     (312, 7, 7), (1280, 1, 1)]
+    nm = ios.models.nasnet_mobile()
+    assert tuple(nm.exit_node.output_shape) == (880, 1, 1)
+    assert sum(len(p) for p in nm.blocks[0].parts) == len(nm.blocks[0].inner_nodes) + 1
+
+
+def test_randwire_graph_generator_is_seeded_and_valid():
+    from ios.models.randwire import watts_strogatz_edges, read_graph, write_graph
+    e1 = watts_strogatz_edges(32, 4, 0.75, seed=3)
+    assert e1 == watts_strogatz_edges(32, 4, 0.75, seed=3)
+    assert e1 != watts_strogatz_edges(32, 4, 0.75, seed=4)
+    assert len(e1) == 64 and all(0 <= u < v < 32 for u, v in e1) and len(set(e1)) == 64
+    assert watts_strogatz_edges(8, 2, 0.0, seed=0) == sorted([(i, i + 1) for i in range(7)] + [(0, 7)])
+
+
+def test_randwire_edge_file_format(tmp_path):
+    from ios.models.randwire import watts_strogatz_edges, read_graph, write_graph
+    edges = watts_strogatz_edges(16, 4, 0.75, seed=2)
+    path = tmp_path / 'ws.txt'
+    write_graph(path, 16, edges)
+    assert read_graph(path) == (16, edges)
+
+
+def test_sequential_and_greedy_schedules_cover_all_operators():
+    graph = ios.models.inception_v3()
+    for schedule in (graph.sequential_schedule, lambda: graph.greedy_schedule(4)):
+        schedule()
+        for block in graph.blocks:
+            names = [n for stage in block.stages for group in stage for n in group]
+            assert sorted(names) == sorted(n.name for n in block.inner_nodes + [block.exit_node])
+            assert all(len(stage) <= 4 or schedule == graph.sequential_schedule for stage in block.stages)
+    graph.greedy_schedule(10)
+    # inception_a block: the four branch heads are ready at once
+    assert graph.blocks[1].stages[0] == [['8'], ['9'], ['11'], ['14']]
+
+
+def test_seeded_he_normal_init():
+    g1 = ios.models.sample_network(init_seed=0, init_scheme='he_normal')
+    g2 = ios.models.sample_network(init_seed=0, init_scheme='he_normal')
+    c1, c2 = g1.conv_nodes()[0], g2.conv_nodes()[0]
+    np.testing.assert_array_equal(c1.weight, c2.weight)
+    assert c1.weight.dtype == np.float32 and c1.weight.shape == (375, 375, 3, 3)
+    assert np.all(c1.bias == 0)
+    assert c1.weight.std() == pytest.approx(np.sqrt(2.0 / (375 * 9)), rel=0.02)
+
+
+def test_value_and_uses():
+    ios.reset_name()
+    v = ios.placeholder((8, 4, 4))
+    block = ios.Block(v.node)
+    a = ios.conv2d(block, [[v]], 8)
+    b = ios.identity(block, [[a, v]], is_exit=True)
+    assert a.node.uses == [(b.node, 0, 0)]
+    assert v.node.uses == [(a.node, 0, 0), (b.node, 0, 1)]
+    assert Value(a.node, 0, 8) == a and a.length == 8
+    assert b.node.input_readable_str() == '(1+0)'
+
+
+def test_unknown_node_type_raises():
+    with pytest.raises(ValueError):
+        ios.ir.Node.from_config({'type': 'softmax', 'name': 'x', 'hint_name': 'x', 'inputs': [], 'output_shape': None}, {})

@@ -1,0 +1,238 @@
+"""
+The schedule search: optimum against brute-force enumeration of every valid schedule under a
+deterministic additive cost model, structural invariants of the result, merge construction.
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+import ios
+from ios.cost_model import AnalyticCostModel, CostModel, RandomCostModel
+from ios.ir import Conv, Graph
+from ios.optimizer import check_merge, graph_chain_decomposition, build_graph, optimize
+
+
+class TableCost(CostModel):
+    """Deterministic pseudo-random price per (group structure); concurrency is rewarded irregularly."""
+
+    def __init__(self, seed=0):
+        self.seed = seed
+        self.calls = 0
+
+    def get_stage_latency(self, stage, batch_size, warmup, number, repeat, profile_stage=False):
+        self.calls += 1
+        key = tuple(sorted(tuple(n.name for n in group) for group in stage))
+        rng = np.random.default_rng(abs(hash((self.seed, key))) % (2 ** 32))
+        longest = max(sum(1.0 + 0.1 * int(n.name) for n in group) for group in stage)
+        return [longest + 0.3 * len(stage) + float(rng.random())] * repeat
+
+
+def stage_key_cost(cost, groups):
+    return cost.get_stage_latency(groups, 1, 1, 1, 1)[0]
+
+
+def brute_force_best(block, cost, max_group_size, max_num_groups):
+    """Enumerate every way to peel admissible parallel stages off the block; return the minimum cost."""
+    members = block.inner_nodes + [block.exit_node]
+    index = {n: i for i, n in enumerate(members)}
+    succ = {i: set() for i in range(len(members))}
+    for n in members:
+        for use in n.uses:
+            if use[0] in index:
+                succ[index[n]].add(index[use[0]])
+
+    def closure(u, alive):
+        out, todo = {u}, [u]
+        while todo:
+            for v in succ[todo.pop()]:
+                if v in alive and v not in out:
+                    out.add(v)
+                    todo.append(v)
+        return frozenset(out)
+
+    memo = {}
+
+    def best(alive):
+        if not alive:
+            return 0.0
+        if alive in memo:
+            return memo[alive]
+        groups_of = {u: closure(u, alive) for u in alive}
+        candidates = [u for u in alive if len(groups_of[u]) <= max_group_size]
+        value = float('inf')
+        for k in range(1, max_num_groups + 1):
+            for heads in itertools.combinations(sorted(candidates), k):
+                groups = [groups_of[h] for h in heads]
+                if any(a & b for a, b in itertools.combinations(groups, 2)):
+                    continue
+                used = frozenset().union(*groups)
+                stage = [[members[i] for i in sorted(g)] for g in groups]
+                value = min(value, best(alive - used) + stage_key_cost(cost, stage))
+        memo[alive] = value
+        return value
+
+    return best(frozenset(range(len(members))))
+
+
+def small_graphs():
+    def diamond():
+        ios.reset_name()
+        v = ios.placeholder((8, 6, 6))
+        b = ios.Block(v.node)
+        a = ios.conv2d(b, [[v]], 8)
+        c1 = ios.conv2d(b, [[a]], 8, (3, 3), padding=(1, 1))
+        c2 = ios.conv2d(b, [[a]], 8)
+        c3 = ios.conv2d(b, [[c2]], 8)
+        p = ios.pool2d(b, [[v]], 'avg', (3, 3), (1, 1), (1, 1))
+        ios.identity(b, [[c1], [c3], [p]], is_exit=True)
+        return Graph('diamond', v.node, [b])
+
+    def wide():
+        ios.reset_name()
+        v = ios.placeholder((4, 5, 5))
+        b = ios.Block(v.node)
+        heads = [ios.conv2d(b, [[v]], 4) for _ in range(3)]
+        tails = [ios.conv2d(b, [[h]], 4) for h in heads[:2]]
+        ios.identity(b, [[tails[0], tails[1], heads[2]]], is_exit=True)
+        return Graph('wide', v.node, [b])
+
+    return [diamond(), wide(), ios.models.sample_network()]
+
+
+@pytest.mark.parametrize('r,s', [(1, 2), (2, 3), (3, 8)])
+def test_dp_optimum_equals_brute_force(r, s):
+    for graph in small_graphs():
+        cost = TableCost(seed=r * 10 + s)
+        new_graph = optimize(graph, 1, cost, 'dp_parallel', max_group_size=r, max_num_groups=s)
+        want = brute_force_best(graph.blocks[0], cost, r, s)
+        by_name = {n.name: n for n in new_graph.blocks[0].inner_nodes + [new_graph.blocks[0].exit_node]}
+        got = sum(stage_key_cost(cost, [[by_name[n] for n in g] for g in stage]) for stage in new_graph.blocks[0].stages)
+        assert got == pytest.approx(want, rel=1e-12), graph.name
+
+
+def check_schedule_invariants(graph, new_graph, max_group_size, max_num_groups):
+    assert len(new_graph.blocks) == len(graph.blocks)
+    for old, new in zip(graph.blocks, new_graph.blocks):
+        members = new.inner_nodes + [new.exit_node]
+        by_name = {n.name: n for n in members}
+        scheduled = [n for stage in new.stages for group in stage for n in group]
+        assert sorted(scheduled) == sorted(by_name)            # every operator exactly once
+        done = {new.enter_node.name}
+        for stage in new.stages:
+            assert 1 <= len(stage) <= max_num_groups
+            stage_names = {n for group in stage for n in group}
+            for group in stage:
+                assert 1 <= len(group) <= max_group_size
+                local = set()
+                for name in group:
+                    for term in by_name[name].inputs:
+                        for value in term:
+                            dep = value.node.name
+                            # a dependency is finished earlier, or earlier in the same group: groups are independent
+                            assert dep in done or dep in local or dep not in by_name, (name, dep)
+                            assert dep not in stage_names - set(group)
+                    local.add(name)
+            done |= stage_names
+
+
+def test_inception_dp_parallel_invariants_and_never_worse_than_sequential():
+    graph = ios.models.inception_v3()
+    cost = AnalyticCostModel()
+    new_graph = optimize(graph, 1, cost, 'dp_parallel', max_group_size=3, max_num_groups=8)
+    check_schedule_invariants(graph, new_graph, 3, 8)
+    assert new_graph.name == 'inception_v3_dp_parallel'
+    graph.sequential_schedule()
+    seq = cost.get_graph_latency(graph, 1, 0, 1, 1)[0]
+    opt = cost.get_graph_latency(new_graph, 1, 0, 1, 1)[0]
+    assert opt < seq
+    assert [n.name for n in new_graph.nodes()][0] == '0'
+    assert tuple(new_graph.exit_node.output_shape) == (2048, 1, 1)
+
+
+def test_random_cost_model_schedules_are_valid():
+    graph = ios.models.squeezenet_1_1()
+    new_graph = optimize(graph, 1, RandomCostModel(seed=5), 'dp_parallel_merge', max_group_size=2, max_num_groups=3)
+    # merged stages replace several convolutions by one, so only check coverage via hint names
+    hints = set()
+    for node in new_graph.nodes():
+        hints.update(node.hint_name.split())
+    assert hints == {n.name for n in graph.nodes()}
+
+
+def test_stage_measurements_are_memoised():
+    graph = ios.models.sample_network()
+    cost = TableCost()
+    info = {}
+    optimize(graph, 1, cost, 'dp_parallel', debug_dp_info=info)
+    assert cost.calls == len(info['stage_latency'])
+    assert info['#operators'] == [5] and info['#states'][0] >= 5 and info['#schedules'][0] >= 1
+
+
+def test_check_merge_rules():
+    graph = ios.models.inception_v3()
+    block = graph.blocks[1]     # inception_a: 8, 9, 11 are 1x1 convs on the block input
+    members = block.inner_nodes + [block.exit_node]
+    idn = dict(enumerate(members))
+    idx = {n.name: i for i, n in idn.items()}
+    mask = lambda names: sum(1 << idx[n] for n in names)
+    assert check_merge(mask(['8', '9', '11']), idn)
+    assert not check_merge(mask(['8', '10']), idn)            # different inputs
+    assert not check_merge(mask(['8', '14']), idn)            # a pool
+    assert check_merge(mask(['14']), idn)                     # any single operator
+    e = graph.blocks[10]
+    idn_e = dict(enumerate(e.inner_nodes + [e.exit_node]))
+    idx_e = {n.name: i for i, n in idn_e.items()}
+    # 1x3 and 3x1 convolutions on the same input merge into one 3x3
+    assert check_merge(sum(1 << idx_e[n] for n in ['99', '100']), idn_e)
+
+
+def test_merged_graph_weights_reproduce_unmerged_outputs():
+    from oracle import ios_oracle
+    ios.reset_name()
+    v = ios.placeholder((6, 9, 9))
+    b = ios.Block(v.node)
+    a = ios.conv2d(b, [[v]], 5, (1, 1))
+    c = ios.conv2d(b, [[v]], 4, (3, 3), padding=(1, 1))
+    d = ios.conv2d(b, [[v]], 3, (1, 3), padding=(0, 1))
+    e = ios.conv2d(b, [[v]], 2, (3, 1), padding=(1, 0))
+    f = ios.conv2d(b, [[c]], 4, (3, 3), padding=(1, 1))
+    ios.identity(b, [[a], [f], [d], [e]], is_exit=True)
+    graph = Graph('m', v.node, [b])
+    graph.init_weights(seed=3)
+
+    class PreferMerge(CostModel):
+        def get_stage_latency(self, stage, batch_size, warmup, number, repeat, profile_stage=False):
+            return [1.0] * repeat       # every stage costs the same: fewer stages win
+
+    merged = optimize(graph, 1, PreferMerge(), 'dp_merge', compute_weight=True)
+    convs = merged.conv_nodes()
+    assert any(' ' in conv.hint_name for conv in convs)       # something was merged
+    big = max(convs, key=lambda conv: conv.out_channels)
+    assert tuple(big.kernel) == (3, 3) and tuple(big.padding) == (1, 1) and big.out_channels == 14
+    x = np.random.default_rng(0).standard_normal((2, 6, 9, 9)).astype(np.float32)
+    np.testing.assert_allclose(ios_oracle.run(merged, x), ios_oracle.run(graph, x), rtol=1e-5, atol=1e-5)
+    # invariant of the stacked weights: slice i of the merged output equals convolution i alone
+    all_out = ios_oracle.run(merged, x, keep_all=True)
+    plain = ios_oracle.run(graph, x, keep_all=True)
+    first = 0
+    for name in big.hint_name.split():
+        width = plain[name].shape[1]
+        np.testing.assert_allclose(all_out[big.name][:, first:first + width], plain[name], rtol=1e-5, atol=1e-5)
+        first += width
+
+
+def test_chain_decomposition_covers_graph_with_chains():
+    graph = ios.models.inception_v3()
+    block = graph.blocks[6]
+    members = block.inner_nodes + [block.exit_node]
+    nid = {n: i for i, n in enumerate(members)}
+    g = build_graph(members, nid)
+    chains = graph_chain_decomposition(g)
+    flat = [u for chain in chains for u in chain]
+    assert sorted(flat) == sorted(g)
+    from ios.optimizer import graph_transitive_closure
+    tc = graph_transitive_closure(g)
+    for chain in chains:
+        for a, b in zip(chain, chain[1:]):
+            assert b in tc[a]
