@@ -1,0 +1,96 @@
+/*
+ * C ABI of libios_runtime.so -- the MI355X (gfx950) execution engine of the inter-operator scheduler.
+ *
+ * The first four functions are drop-in replacements for the entry points of the reference runtime
+ * (reference src/ios/ios_runtime.cu:1478-1519) that the reference Python glue binds with ctypes
+ * (reference python/ios/contrib/ios_runtime.py:26-135).  Arguments have the same order and meaning.
+ * Differences: they return int (0 = success, non-zero = failure, message via ios_last_error()) where the
+ * reference returns void and terminates the process on errors; a caller that ignores the return value
+ * sees the reference behaviour minus the exit().
+ *
+ * All pointers are owned by the caller and only used during the call.  Host buffers are float32,
+ * C-contiguous, NCHW.  The library is not re-entrant: call it from one thread at a time.
+ * JSON documents are the wire format exported by ios.Graph.export_config() / Block.export_config()
+ * (reference python/ios/ir.py:855-865,1038-1046).
+ */
+#ifndef IOS_RUNTIME_H
+#define IOS_RUNTIME_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Latency of a whole graph under its schedule.  Replaces graph_latency (src/ios/ios_runtime.cu:1480-1484).
+ * results[repeat]: milliseconds per forward pass, each the mean of `number` individually timed passes.
+ * stage_results[repeat * num_stages] (row-major, caller-zeroed): per-stage milliseconds, written only when
+ * profile_stage_latency != 0; num_stages = total number of stages over all blocks.
+ */
+int graph_latency(const char *graph_json, int batch_size, int warmup, int number, int repeat,
+                  int profile_stage_latency, float *results, float *stage_results);
+
+/* Same for a single block document.  Replaces block_latency (src/ios/ios_runtime.cu:1486-1490). */
+int block_latency(const char *block_json, int batch_size, int warmup, int number, int repeat,
+                  int profile_stage_latency, float *results, float *stage_results);
+
+/*
+ * Latency of one candidate stage.  Replaces stage_latency (src/ios/ios_runtime.cu:1492-1498).
+ * stage_json: [[operator config, ...] per group]; input_json: {producer name: [C, H, W]} for every
+ * producer outside the stage.  profile_stage_latency must be 0.  results[repeat]: milliseconds per pass,
+ * `number` passes issued back to back inside one timing bracket.
+ */
+int stage_latency(const char *stage_json, const char *input_json, int batch_size, int warmup, int number,
+                  int repeat, int profile_stage_latency, float *results, float *stage_results);
+
+/*
+ * One inference.  Replaces graph_inference (src/ios/ios_runtime.cu:1500-1517).
+ * input: batch_size x C x H x W; filter_data[i]: OC x IC/groups x KH x KW and bias_data[i]: OC for the
+ * convolution named conv_names[i] (convolutions inside sequential operators included); unknown names are
+ * reported on stdout and skipped, NULL data is an error.  output: batch_size x shape of the last operator;
+ * the last stage of the schedule must have a single group.
+ */
+int graph_inference(const char *graph_json, int batch_size, float *input, int num_convs, char **conv_names,
+                    float **filter_data, float **bias_data, float *output);
+
+/* ---- extensions without a counterpart in the reference ------------------------------------------------ */
+
+/* Message of the most recent failure (valid until the next failing call). */
+const char *ios_last_error(void);
+
+/* Options: "executor" = "streams" | "graph" (hipGraph replay); "autotune" = "0" | "1" (measure convolution
+ * kernel configurations on first use, like the reference's cudnnFind-based selection,
+ * src/ios/ios_runtime.cu:150-205); "clear_tuning" = anything;
+ * "conv_variant" = index or -1 and "conv_split_k" = count or 0 force one convolution kernel configuration (testing). */
+int ios_set_option(const char *key, const char *value);
+
+/* JSON description of device 0 ({"name", "arch", "compute_units", ...}) into buf. */
+int ios_device_info(char *buf, int cap);
+
+/* Host-only planning: writes the JSON list of device operations for a graph into buf and returns its length
+ * (call again with a larger buffer when the return value >= cap); -1 on error.  Touches no device. */
+int ios_plan_describe(const char *graph_json, int batch_size, char *buf, int cap);
+
+/* Persistent session: plan once, keep weights and activations on the device, run many times. */
+typedef struct ios_session ios_session;
+ios_session *ios_session_create(const char *graph_json, int batch_size);   /* NULL on failure */
+void ios_session_destroy(ios_session *session);
+int ios_session_set_conv_weights(ios_session *session, int num_convs, char **conv_names, float **filter_data,
+                                 float **bias_data);
+int ios_session_set_input(ios_session *session, const float *input);
+int ios_session_run(ios_session *session);
+int ios_session_get_output(ios_session *session, float *output);
+/* Dense copy of any operator's output (batch x C x H x W) after a run. */
+int ios_session_get_tensor(ios_session *session, const char *node_name, float *output);
+/* Same protocol and outputs as graph_latency, on the resident session. */
+int ios_session_measure(ios_session *session, int warmup, int number, int repeat, int profile_stage_latency,
+                        float *results, float *stage_results);
+int ios_session_num_ops(ios_session *session);                              /* -1 on failure */
+int ios_session_describe(ios_session *session, char *buf, int cap);         /* like ios_plan_describe */
+/* ms[num_ops]: mean HIP-event time of each device operation launched `repeat` times back to back on one stream. */
+int ios_session_profile_ops(ios_session *session, int warmup, int repeat, float *ms);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* IOS_RUNTIME_H */

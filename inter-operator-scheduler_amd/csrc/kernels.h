@@ -1,0 +1,109 @@
+// Device kernels of the runtime and their host-side launchers (gfx950 / CDNA4 only).
+//
+// All tensors are fp32 NCHW *views*: a base pointer to (n=0, c=0), the extents C/H/W and a batch stride
+// in elements.  The channel stride is always H*W, so a channel slice or a window inside a wider concat
+// buffer is again a view; producers write straight into such windows and consumers read slices without
+// copies.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace ios {
+
+enum Act : int { ACT_NONE = 0, ACT_RELU = 1, ACT_TANH = 2, ACT_SIGMOID = 3 };
+
+struct TensorView {
+    float *ptr = nullptr;  // element (0, 0, 0, 0)
+    int C = 0, H = 0, W = 0;
+    long long bstride = 0;  // elements between images
+};
+
+// ---- convolution ------------------------------------------------------------------------------------
+struct ConvProblem {
+    int B, IC, H, W, OC, KH, KW, sh, sw, ph, pw, groups;
+    int OH, OW;
+    int act;       // Act applied after bias
+    int pre_relu;  // apply max(x, 0) to the input while loading it
+    int ICg() const { return IC / groups; }
+    int OCg() const { return OC / groups; }
+    int K() const { return ICg() * KH * KW; }
+    long long Npix() const { return (long long)B * OH * OW; }
+    int OCgP() const { return (OCg() + 3) & ~3; }  // row length of the packed filter matrix
+    bool is_depthwise() const { return groups > 1 && IC == groups && OC == groups; }
+    bool is_pointwise() const { return KH == 1 && KW == 1 && ph == 0 && pw == 0; }
+    double flops() const { return 2.0 * (double)Npix() * OC * K(); }
+};
+
+// One implicit-GEMM kernel configuration: block tile BM (output channels) x BN (pixels) x BK, a grid of
+// WM x WN x WK wavefronts (WK wavefronts split the block's K tile) built from MT x MT fp32 MFMA tiles.
+struct ConvVariant {
+    const char *name;
+    int BM, BN, BK, WM, WN, WK, MT;
+    int threads() const { return 64 * WM * WN * WK; }
+};
+
+int conv_num_variants();
+const ConvVariant &conv_variant(int index);
+
+struct ConvLaunch {
+    int variant = 0;
+    int split_k = 1;  // number of grid slices along K; > 1 needs workspace and counters
+};
+
+// Bytes of workspace / number of tile counters a launch configuration needs.
+size_t conv_workspace_floats(const ConvProblem &p, const ConvLaunch &l);
+size_t conv_num_counters(const ConvProblem &p, const ConvLaunch &l);
+
+// Default configuration from a closed-form occupancy model (num_cus = compute units of the device).
+ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus);
+
+// Filter packing: w[OC][ICg][KH][KW] -> packed[g][K][OCgP] (K = ICg*KH*KW, zero padded rows), and the
+// per-k gather table {c*H*W + kh*W + kw, kh << 16 | kw} used by the implicit-GEMM input loader.
+size_t conv_packed_floats(const ConvProblem &p);
+void launch_pack_filters(const ConvProblem &p, const float *w, float *packed, hipStream_t stream);
+void launch_build_ktab(const ConvProblem &p, int2 *ktab, hipStream_t stream);
+
+// y = act(conv(x, w) + bias).  `packed` and `ktab` come from the two functions above.  `workspace` holds
+// split_k partial tiles, `counters` must be zero before the first launch and is left zero afterwards.
+void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
+                      const int2 *ktab, const float *bias, const TensorView &y, float *workspace,
+                      unsigned *counters, hipStream_t stream);
+
+// Depth-wise convolution (groups == IC == OC), filters in their original [C][1][KH][KW] layout.
+void launch_dwconv(const ConvProblem &p, const TensorView &x, const float *w, const float *bias,
+                   const TensorView &y, hipStream_t stream);
+
+// Direct convolution for any geometry (one thread per output element); used for grouped convolutions
+// whose groups are too thin for the matrix path.
+void launch_conv_direct(const ConvProblem &p, const TensorView &x, const float *w, const float *bias,
+                        const TensorView &y, hipStream_t stream);
+
+// ---- pooling ----------------------------------------------------------------------------------------
+struct PoolProblem {
+    int B, C, H, W, KH, KW, sh, sw, ph, pw, OH, OW;
+    int is_max;  // 1: max over in-range elements, 0: sum of in-range elements / (KH*KW)
+};
+void launch_pool(const PoolProblem &p, const TensorView &x, const TensorView &y, hipStream_t stream);
+// Window == whole map: one wavefront reduces one (n, c) plane.
+void launch_global_pool(const PoolProblem &p, const TensorView &x, const TensorView &y, hipStream_t stream);
+
+// ---- element-wise -----------------------------------------------------------------------------------
+constexpr int kMaxNaryInputs = 8;
+struct NaryArgs {
+    const float *src[kMaxNaryInputs];
+    long long src_bstride[kMaxNaryInputs];
+    int count;
+};
+// y = act(src0 (+|*) src1 (+|*) ...), left to right; more than kMaxNaryInputs inputs are handled by the
+// caller through accumulation (accumulate != 0 also combines the current contents of y first).
+void launch_nary(const NaryArgs &a, int multiply, int accumulate, int act, int B, long long chw,
+                 const TensorView &y, hipStream_t stream);
+// y = act(x) for views; act == ACT_NONE is a strided copy.
+void launch_unary(const TensorView &x, const TensorView &y, int act, int B, hipStream_t stream);
+// Fill n floats with a deterministic pattern in [-1, 1) (seeded), or with a constant.
+void launch_fill_pattern(float *dst, size_t n, unsigned seed, hipStream_t stream);
+void launch_fill_u32(unsigned *dst, size_t n, unsigned value, hipStream_t stream);
+
+}  // namespace ios

@@ -1,0 +1,662 @@
+// Planner: JSON document -> Plan.  See plan.h for the memory model.  The document layout is the wire
+// format exported by the Python IR (graph = {name, input, blocks}, block = {enter_name, enter_node,
+// inner_nodes, exit_node, stages}, stage document = [[node config, ...] per group]); operator semantics
+// are those the reference runtime gives the same documents (src/ios/ios_runtime.cu:1118-1240 for the
+// three document kinds, :623-812 for the input algebra, :1047-1057 for pooling types).
+#include "plan.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <set>
+#include <sstream>
+#include <stdexcept>
+
+namespace ios {
+
+const char *op_kind_name(OpKind kind) {
+    switch (kind) {
+        case OpKind::ConvMfma: return "conv_mfma";
+        case OpKind::ConvDepthwise: return "conv_depthwise";
+        case OpKind::ConvDirect: return "conv_direct";
+        case OpKind::Pool: return "pool";
+        case OpKind::GlobalPool: return "global_pool";
+        case OpKind::Nary: return "nary";
+        case OpKind::Unary: return "unary";
+    }
+    return "?";
+}
+
+namespace {
+
+struct Val {
+    int node;
+    int begin, end;
+};
+
+enum class NodeType { Placeholder, Conv, Pool, Identity, Relu, Activation, Element, Sequential };
+
+struct PNode {
+    std::string name;
+    NodeType type = NodeType::Placeholder;
+    const Json *cfg = nullptr;
+    int C = 0, H = 0, W = 0;
+    std::vector<std::vector<Val>> inputs;
+    int unit = -1;
+    // storage: either an own region or a channel window of another node's storage
+    bool own = false;
+    size_t own_offset = 0;
+    int parent = -1, parent_begin = 0;
+    bool pre_relu_alias = false;   // elided ReLU: consumers must apply max(x, 0) themselves
+    int fused_into = -1;           // concat (identity) node whose buffer holds this node's output
+    int references = 0;            // number of input values that name this node
+};
+
+int act_code(const std::string &name) {
+    if (name == "identity") return ACT_NONE;
+    if (name == "relu") return ACT_RELU;
+    if (name == "tanh") return ACT_TANH;
+    if (name == "sigmoid") return ACT_SIGMOID;
+    throw std::runtime_error("unsupported activation '" + name + "'");
+}
+
+class Planner {
+public:
+    Planner(int batch, const LaunchChooser &chooser) : batch_(batch), chooser_(chooser) {
+        if (batch < 1) throw std::runtime_error("batch size must be positive");
+        plan_.batch = batch;
+    }
+
+    Plan run(PlanMode mode, const Json &doc, const Json *extra) {
+        std::vector<std::vector<std::vector<std::string>>> stage_names;
+        if (mode == PlanMode::Graph) {
+            add_placeholder(doc["input"]["name"].as_string(), doc["input"]["output_shape"]);
+            plan_.input_name = nodes_[0].name;
+            for (const Json &block : doc["blocks"].items()) add_block(block, stage_names);
+        } else if (mode == PlanMode::Block) {
+            const Json &enter = doc["enter_node"];
+            add_placeholder(enter["name"].as_string(), enter["output_shape"]);
+            plan_.input_name = nodes_[0].name;
+            add_block(doc, stage_names);
+        } else {
+            if (extra == nullptr || !extra->is_object()) throw std::runtime_error("stage document needs an input-shape document");
+            for (const auto &member : extra->members()) add_placeholder(member.first, member.second);
+            if (!doc.is_array() || doc.size() == 0) throw std::runtime_error("stage document must be a non-empty list of groups");
+            std::vector<std::vector<std::string>> groups;
+            for (const Json &group : doc.items()) {
+                std::vector<std::string> names;
+                for (const Json &cfg : group.items()) {
+                    add_unit(cfg);
+                    names.push_back(cfg["name"].as_string());
+                }
+                groups.push_back(names);
+            }
+            stage_names.push_back(groups);
+            if (!nodes_.empty() && nodes_[0].type == NodeType::Placeholder) plan_.input_name = nodes_[0].name;
+        }
+        if (units_.empty()) throw std::runtime_error("document contains no operators");
+        decide_storage();
+        allocate_outputs();
+        for (size_t i = 0; i < nodes_.size(); i++) emit(static_cast<int>(i));
+        assign_stages(stage_names);
+        finish();
+        return std::move(plan_);
+    }
+
+private:
+    // ---- document -> node table ---------------------------------------------------------------------------
+    int lookup(const std::string &name) const {
+        auto it = by_name_.find(name);
+        if (it == by_name_.end()) throw std::runtime_error("operator '" + name + "' is used before it is defined");
+        return it->second;
+    }
+
+    void add_placeholder(const std::string &name, const Json &shape) {
+        if (by_name_.count(name)) throw std::runtime_error("duplicate operator name '" + name + "'");
+        PNode n;
+        n.name = name;
+        n.type = NodeType::Placeholder;
+        n.C = shape[0].as_int();
+        n.H = shape[1].as_int();
+        n.W = shape[2].as_int();
+        n.own = true;
+        by_name_[name] = static_cast<int>(nodes_.size());
+        nodes_.push_back(n);
+    }
+
+    void add_block(const Json &block, std::vector<std::vector<std::vector<std::string>>> &stage_names) {
+        for (const Json &cfg : block["inner_nodes"].items()) add_unit(cfg);
+        add_unit(block["exit_node"]);
+        const Json &stages = block["stages"];
+        if (!stages.is_array()) throw std::runtime_error("block has no schedule (stages is null); call sequential_schedule() first");
+        for (const Json &stage : stages.items()) {
+            std::vector<std::vector<std::string>> groups;
+            for (const Json &group : stage.items()) {
+                std::vector<std::string> names;
+                for (const Json &name : group.items()) names.push_back(name.as_string());
+                groups.push_back(names);
+            }
+            stage_names.push_back(groups);
+        }
+    }
+
+    void add_unit(const Json &cfg) {
+        const int unit = static_cast<int>(units_.size());
+        units_.push_back(cfg["name"].as_string());
+        plan_.unit_names.push_back(units_.back());
+        const int index = add_node(cfg, unit);
+        unit_result_.push_back(index);
+    }
+
+    std::vector<std::vector<Val>> parse_inputs(const Json &inputs) {
+        std::vector<std::vector<Val>> terms;
+        for (const Json &term : inputs.items()) {
+            std::vector<Val> values;
+            for (const Json &value : term.items()) {
+                Val v{lookup(value[0].as_string()), value[1].as_int(), value[2].as_int()};
+                const PNode &src = nodes_[v.node];
+                if (v.begin < 0 || v.end > src.C || v.begin >= v.end)
+                    throw std::runtime_error("bad channel slice of '" + src.name + "'");
+                nodes_[v.node].references++;
+                values.push_back(v);
+            }
+            if (values.empty()) throw std::runtime_error("empty input term");
+            terms.push_back(values);
+        }
+        if (terms.empty()) throw std::runtime_error("operator without inputs");
+        return terms;
+    }
+
+    void input_shape(const PNode &n, int &C, int &H, int &W) const {
+        C = 0;
+        H = nodes_[n.inputs[0][0].node].H;
+        W = nodes_[n.inputs[0][0].node].W;
+        for (const auto &term : n.inputs) {
+            const int len = term[0].end - term[0].begin;
+            for (const Val &v : term) {
+                if (v.end - v.begin != len || nodes_[v.node].H != H || nodes_[v.node].W != W)
+                    throw std::runtime_error("operator '" + n.name + "': input values of different shapes");
+            }
+            C += len;
+        }
+    }
+
+    int add_node(const Json &cfg, int unit) {
+        const std::string type = cfg["type"].as_string();
+        const std::string name = cfg["name"].as_string();
+        if (by_name_.count(name)) throw std::runtime_error("duplicate operator name '" + name + "'");
+        if (type == "sequential") {
+            const Json &children = cfg["nodes"];
+            if (children.size() == 0) throw std::runtime_error("empty sequential operator '" + name + "'");
+            int last = -1;
+            const int first_child = static_cast<int>(nodes_.size());
+            for (const Json &child : children.items()) last = add_node(child, unit);
+            sequentials_.push_back({first_child, last});
+            PNode n;
+            n.name = name;
+            n.type = NodeType::Sequential;
+            n.cfg = &cfg;
+            n.unit = unit;
+            n.C = nodes_[last].C;
+            n.H = nodes_[last].H;
+            n.W = nodes_[last].W;
+            n.parent = last;
+            by_name_[name] = static_cast<int>(nodes_.size());
+            nodes_.push_back(n);
+            return static_cast<int>(nodes_.size()) - 1;
+        }
+        PNode n;
+        n.name = name;
+        n.cfg = &cfg;
+        n.unit = unit;
+        n.inputs = parse_inputs(cfg["inputs"]);
+        int C, H, W;
+        input_shape(n, C, H, W);
+        if (type == "conv") {
+            n.type = NodeType::Conv;
+            const int kh = cfg["kernel"][0].as_int(), kw = cfg["kernel"][1].as_int();
+            const int sh = cfg["stride"][0].as_int(), sw = cfg["stride"][1].as_int();
+            const int ph = cfg["padding"][0].as_int(), pw = cfg["padding"][1].as_int();
+            const int groups = cfg["groups"].as_int();
+            n.C = cfg["out_channels"].as_int();
+            if (groups < 1 || C % groups != 0 || n.C % groups != 0)
+                throw std::runtime_error("conv '" + name + "': channels not divisible by groups");
+            if (sh < 1 || sw < 1 || kh < 1 || kw < 1) throw std::runtime_error("conv '" + name + "': bad geometry");
+            n.H = 1 + (H - kh + 2 * ph) / sh;
+            n.W = 1 + (W - kw + 2 * pw) / sw;
+            act_code(cfg["act"].as_string());
+        } else if (type == "pool") {
+            n.type = NodeType::Pool;
+            n.C = C;
+            const std::string pool_type = cfg["pool_type"].as_string();
+            if (pool_type.find("global") != std::string::npos) {
+                n.H = 1;
+                n.W = 1;
+            } else {
+                const int kh = cfg["kernel"][0].as_int(), kw = cfg["kernel"][1].as_int();
+                const int sh = cfg["stride"][0].as_int(), sw = cfg["stride"][1].as_int();
+                const int ph = cfg["padding"][0].as_int(), pw = cfg["padding"][1].as_int();
+                if (sh < 1 || sw < 1 || kh < 1 || kw < 1) throw std::runtime_error("pool '" + name + "': bad geometry");
+                n.H = 1 + (H - kh + 2 * ph) / sh;
+                n.W = 1 + (W - kw + 2 * pw) / sw;
+            }
+        } else if (type == "identity" || type == "relu" || type == "activation" || type == "element") {
+            n.type = type == "identity" ? NodeType::Identity
+                     : type == "relu"   ? NodeType::Relu
+                     : type == "activation" ? NodeType::Activation
+                                            : NodeType::Element;
+            if (n.type == NodeType::Element) {
+                if (n.inputs.size() != 1) throw std::runtime_error("element '" + name + "' needs exactly one term");
+                const std::string op = cfg["op_type"].as_string();
+                if (op != "add" && op != "mul") throw std::runtime_error("element '" + name + "': unknown op_type " + op);
+            }
+            if (n.type == NodeType::Activation) act_code(cfg["act_type"].as_string());
+            n.C = C;
+            n.H = H;
+            n.W = W;
+        } else {
+            throw std::runtime_error("unsupported type " + type);
+        }
+        if (n.H < 1 || n.W < 1) throw std::runtime_error("operator '" + name + "' has an empty output");
+        by_name_[name] = static_cast<int>(nodes_.size());
+        nodes_.push_back(n);
+        return static_cast<int>(nodes_.size()) - 1;
+    }
+
+    // ---- storage decisions -----------------------------------------------------------------------------------
+    static bool single_value(const PNode &n) { return n.inputs.size() == 1 && n.inputs[0].size() == 1; }
+
+    bool computes_own_output(const PNode &n) const {
+        switch (n.type) {
+            case NodeType::Conv:
+            case NodeType::Pool:
+            case NodeType::Element: return true;
+            case NodeType::Relu:
+            case NodeType::Activation: return !n.pre_relu_alias;
+            case NodeType::Identity: return !single_value(n);
+            default: return false;
+        }
+    }
+
+    void decide_storage() {
+        // ReLU directly in front of a convolution inside one Sequential, read by nobody else: fold it
+        for (const auto &seq : sequentials_) {
+            for (int i = seq.first; i < seq.second; i++) {
+                PNode &r = nodes_[i];
+                const PNode &next = nodes_[i + 1];
+                if (r.type == NodeType::Relu && next.type == NodeType::Conv && single_value(r) && r.references == 1 &&
+                    single_value(next) && next.inputs[0][0].node == i) {
+                    r.pre_relu_alias = true;
+                    r.parent = r.inputs[0][0].node;
+                    r.parent_begin = r.inputs[0][0].begin;
+                }
+            }
+        }
+        for (PNode &n : nodes_) {
+            if (n.type == NodeType::Identity && single_value(n)) {
+                n.parent = n.inputs[0][0].node;
+                n.parent_begin = n.inputs[0][0].begin;
+            }
+        }
+        // concat fusion: a term that is the whole output of a computing operator is produced in place
+        for (size_t i = 0; i < nodes_.size(); i++) {
+            PNode &cat = nodes_[i];
+            if (cat.type != NodeType::Identity || cat.inputs.size() < 2) continue;
+            int offset = 0;
+            for (const auto &term : cat.inputs) {
+                const int len = term[0].end - term[0].begin;
+                if (term.size() == 1) {
+                    const int src = resolve_sequential(term[0].node);
+                    PNode &p = nodes_[src];
+                    if (term[0].begin == 0 && term[0].end == p.C && computes_own_output(p) && p.fused_into < 0 &&
+                        p.parent < 0) {
+                        p.fused_into = static_cast<int>(i);
+                        p.parent = static_cast<int>(i);
+                        p.parent_begin = offset;
+                    }
+                }
+                offset += len;
+            }
+        }
+        for (PNode &n : nodes_)
+            if (n.parent < 0) n.own = true;
+    }
+
+    int resolve_sequential(int index) const {
+        while (nodes_[index].type == NodeType::Sequential) index = nodes_[index].parent;
+        return index;
+    }
+
+    size_t reserve(size_t floats) {
+        const size_t at = plan_.arena_floats;
+        plan_.arena_floats += (floats + 63) & ~size_t(63);
+        return at;
+    }
+
+    void allocate_outputs() {
+        for (PNode &n : nodes_)
+            if (n.own) n.own_offset = reserve((size_t)batch_ * n.C * n.H * n.W);
+    }
+
+    ViewRef view_of(int index) const {
+        const PNode &n = nodes_[index];
+        if (n.own) {
+            ViewRef v;
+            v.offset = n.own_offset;
+            v.C = n.C;
+            v.H = n.H;
+            v.W = n.W;
+            v.bstride = (long long)n.C * n.H * n.W;
+            return v;
+        }
+        return view_of(n.parent).window(n.parent_begin, n.parent_begin + n.C);
+    }
+
+    bool needs_relu(int index) const {
+        // true when the value seen through `index` is an elided ReLU (possibly behind aliases)
+        const PNode &n = nodes_[index];
+        if (n.pre_relu_alias) return true;
+        return false;
+    }
+
+    ViewRef dense_temp(int C, int H, int W) {
+        ViewRef v;
+        v.offset = reserve((size_t)batch_ * C * H * W);
+        v.C = C;
+        v.H = H;
+        v.W = W;
+        v.bstride = (long long)C * H * W;
+        return v;
+    }
+
+    // ---- op emission --------------------------------------------------------------------------------------------
+    PlanOp &push(OpKind kind, const PNode &owner) {
+        PlanOp op;
+        op.kind = kind;
+        op.node = owner.name;
+        op.unit = owner.unit;
+        plan_.ops.push_back(op);
+        return plan_.ops.back();
+    }
+
+    // dst = act(combine(values of term)); dst has the term's channel count
+    void materialise_term(const PNode &owner, const std::vector<Val> &term, const ViewRef &dst, int act, bool multiply) {
+        const double elems = (double)batch_ * dst.image_floats();
+        if (term.size() == 1) {
+            PlanOp &op = push(OpKind::Unary, owner);
+            op.in = view_of(term[0].node).window(term[0].begin, term[0].end);
+            op.out = dst;
+            op.act = act;
+            op.bytes = 8.0 * elems;
+            return;
+        }
+        for (size_t first = 0; first < term.size(); first += kMaxNaryInputs) {
+            const size_t last = std::min(term.size(), first + kMaxNaryInputs);
+            PlanOp &op = push(OpKind::Nary, owner);
+            for (size_t i = first; i < last; i++) op.srcs.push_back(view_of(term[i].node).window(term[i].begin, term[i].end));
+            op.out = dst;
+            op.multiply = multiply ? 1 : 0;
+            op.accumulate = first > 0 ? 1 : 0;
+            op.act = last == term.size() ? act : ACT_NONE;
+            op.flops = elems * (double)(last - first - (first > 0 ? 0 : 1));
+            op.bytes = 4.0 * elems * (double)(last - first + 1 + (first > 0 ? 1 : 0));
+        }
+    }
+
+    // the operator's input as one view; builds it in a temporary when it is a sum or a concatenation
+    ViewRef input_view(const PNode &n, int C, int H, int W, bool *pre_relu) {
+        if (pre_relu) *pre_relu = false;
+        if (single_value(n)) {
+            const Val &v = n.inputs[0][0];
+            if (nodes_[v.node].pre_relu_alias) {
+                if (pre_relu == nullptr) throw std::runtime_error("internal: folded ReLU read by a non-convolution");
+                *pre_relu = true;
+            }
+            return view_of(v.node).window(v.begin, v.end);
+        }
+        ViewRef temp = dense_temp(C, H, W);
+        int offset = 0;
+        for (const auto &term : n.inputs) {
+            const int len = term[0].end - term[0].begin;
+            materialise_term(n, term, temp.window(offset, offset + len), ACT_NONE, false);
+            offset += len;
+        }
+        return temp;
+    }
+
+    void emit(int index) {
+        PNode &n = nodes_[index];
+        if (n.type == NodeType::Placeholder || n.type == NodeType::Sequential) return;
+        int C, H, W;
+        input_shape(n, C, H, W);
+        const Json &cfg = *n.cfg;
+        switch (n.type) {
+            case NodeType::Conv: emit_conv(n, cfg, C, H, W, index); break;
+            case NodeType::Pool: emit_pool(n, cfg, C, H, W, index); break;
+            case NodeType::Identity:
+                if (!single_value(n)) emit_terms(n, index, ACT_NONE, false);
+                break;
+            case NodeType::Relu:
+                if (!n.pre_relu_alias) emit_terms(n, index, ACT_RELU, false);
+                break;
+            case NodeType::Activation: emit_terms(n, index, act_code(cfg["act_type"].as_string()), false); break;
+            case NodeType::Element: emit_terms(n, index, ACT_NONE, cfg["op_type"].as_string() == "mul"); break;
+            default: break;
+        }
+    }
+
+    void emit_terms(const PNode &n, int index, int act, bool multiply) {
+        const ViewRef out = view_of(index);
+        int offset = 0;
+        for (const auto &term : n.inputs) {
+            const int len = term[0].end - term[0].begin;
+            bool in_place = false;
+            if (term.size() == 1 && n.type == NodeType::Identity) {
+                const PNode &p = nodes_[resolve_sequential(term[0].node)];
+                in_place = p.fused_into == index && p.parent_begin == offset;
+            }
+            if (!in_place) materialise_term(n, term, out.window(offset, offset + len), act, multiply);
+            offset += len;
+        }
+    }
+
+    void emit_conv(PNode &n, const Json &cfg, int C, int H, int W, int index) {
+        bool pre_relu = false;
+        const ViewRef in = input_view(n, C, H, W, &pre_relu);
+        PlanConv conv;
+        conv.name = n.name;
+        ConvProblem &p = conv.problem;
+        p.B = batch_;
+        p.IC = C; p.H = H; p.W = W;
+        p.OC = n.C; p.OH = n.H; p.OW = n.W;
+        p.KH = cfg["kernel"][0].as_int(); p.KW = cfg["kernel"][1].as_int();
+        p.sh = cfg["stride"][0].as_int(); p.sw = cfg["stride"][1].as_int();
+        p.ph = cfg["padding"][0].as_int(); p.pw = cfg["padding"][1].as_int();
+        p.groups = cfg["groups"].as_int();
+        p.act = act_code(cfg["act"].as_string());
+        p.pre_relu = pre_relu ? 1 : 0;
+        conv.weight_off = reserve((size_t)p.OC * p.K());
+        conv.bias_off = reserve((size_t)p.OC);
+        OpKind kind;
+        if (p.is_depthwise()) {
+            kind = OpKind::ConvDepthwise;
+        } else if (p.groups > 1 && (p.ICg() < 4 || p.OCg() < 8)) {
+            kind = OpKind::ConvDirect;
+        } else {
+            kind = OpKind::ConvMfma;
+            conv.matrix_path = true;
+            conv.packed_off = reserve(conv_packed_floats(p));
+            conv.ktab_off = reserve((size_t)p.K() * 2);
+            conv.launch = chooser_(p);
+        }
+        if (plan_.conv_index.count(n.name)) throw std::runtime_error("duplicate convolution name '" + n.name + "'");
+        plan_.conv_index[n.name] = static_cast<int>(plan_.convs.size());
+        plan_.convs.push_back(conv);
+        PlanOp &op = push(kind, n);
+        op.in = in;
+        op.out = view_of(index);
+        op.conv = static_cast<int>(plan_.convs.size()) - 1;
+        op.flops = p.flops();
+        op.bytes = 4.0 * ((double)batch_ * C * H * W + (double)p.OC * p.K() + p.OC + (double)batch_ * p.OC * p.OH * p.OW);
+    }
+
+    void emit_pool(PNode &n, const Json &cfg, int C, int H, int W, int index) {
+        const ViewRef in = input_view(n, C, H, W, nullptr);
+        const std::string pool_type = cfg["pool_type"].as_string();
+        const bool global = pool_type.find("global") != std::string::npos;
+        PoolProblem p;
+        p.B = batch_; p.C = C; p.H = H; p.W = W;
+        p.is_max = pool_type.find("max") != std::string::npos ? 1 : 0;
+        if (global) {
+            p.KH = H; p.KW = W; p.sh = 1; p.sw = 1; p.ph = 0; p.pw = 0;
+        } else {
+            p.KH = cfg["kernel"][0].as_int(); p.KW = cfg["kernel"][1].as_int();
+            p.sh = cfg["stride"][0].as_int(); p.sw = cfg["stride"][1].as_int();
+            p.ph = cfg["padding"][0].as_int(); p.pw = cfg["padding"][1].as_int();
+        }
+        p.OH = n.H; p.OW = n.W;
+        PlanOp &op = push(global ? OpKind::GlobalPool : OpKind::Pool, n);
+        op.in = in;
+        op.out = view_of(index);
+        op.pool = p;
+        op.flops = (double)batch_ * C * p.OH * p.OW * p.KH * p.KW;
+        op.bytes = 4.0 * (double)batch_ * C * ((double)H * W + (double)p.OH * p.OW);
+    }
+
+    // ---- schedule -------------------------------------------------------------------------------------------------
+    void assign_stages(const std::vector<std::vector<std::vector<std::string>>> &stage_names) {
+        std::map<std::string, int> unit_of;
+        for (size_t u = 0; u < units_.size(); u++) unit_of[units_[u]] = static_cast<int>(u);
+        std::vector<std::vector<int>> ops_of_unit(units_.size());
+        for (size_t i = 0; i < plan_.ops.size(); i++) ops_of_unit[plan_.ops[i].unit].push_back(static_cast<int>(i));
+        // producers of every unit (as units), for the order check
+        std::vector<std::set<int>> deps(units_.size());
+        for (const PNode &n : nodes_) {
+            if (n.unit < 0) continue;
+            for (const auto &term : n.inputs)
+                for (const Val &v : term) {
+                    const int pu = nodes_[v.node].unit;
+                    if (pu >= 0 && pu != n.unit) deps[n.unit].insert(pu);
+                }
+        }
+        std::vector<int> state(units_.size(), 0);   // 0 pending, 1 in the running stage, 2 finished
+        std::vector<int> group_of(units_.size(), -1);
+        for (size_t s = 0; s < stage_names.size(); s++) {
+            const auto &groups = stage_names[s];
+            if (groups.empty()) throw std::runtime_error("stage without groups");
+            if (groups.size() > (size_t)kMaxGroups)
+                throw std::runtime_error("The number of groups in stage " + std::to_string(s) + " exceeds the number of available streams " +
+                                         std::to_string(kMaxGroups));
+            std::vector<std::vector<int>> stage_ops(groups.size());
+            for (size_t g = 0; g < groups.size(); g++) {
+                for (const std::string &name : groups[g]) {
+                    auto it = unit_of.find(name);
+                    if (it == unit_of.end()) throw std::runtime_error("schedule names unknown operator '" + name + "'");
+                    const int u = it->second;
+                    if (state[u] != 0) throw std::runtime_error("operator '" + name + "' is scheduled twice");
+                    for (int d : deps[u]) {
+                        const bool ok = state[d] == 2 || (state[d] == 1 && group_of[d] == (int)g);
+                        if (!ok)
+                            throw std::runtime_error("schedule is not topological: '" + name + "' runs before or beside its input '" +
+                                                     units_[d] + "'");
+                    }
+                    state[u] = 1;
+                    group_of[u] = static_cast<int>(g);
+                    for (int op : ops_of_unit[u]) {
+                        plan_.ops[op].stage = static_cast<int>(s);
+                        plan_.ops[op].group = static_cast<int>(g);
+                        stage_ops[g].push_back(op);
+                    }
+                }
+            }
+            for (int &st : state)
+                if (st == 1) st = 2;
+            plan_.stages.push_back(stage_ops);
+        }
+        for (size_t u = 0; u < units_.size(); u++)
+            if (state[u] == 0) throw std::runtime_error("operator '" + units_[u] + "' is missing from the schedule");
+        plan_.output_single_group = stage_names.back().size() == 1;
+    }
+
+    void finish() {
+        for (size_t i = 0; i < nodes_.size(); i++) {
+            const PNode &n = nodes_[i];
+            if (n.pre_relu_alias) continue;   // never materialised
+            plan_.tensors[n.name] = view_of(static_cast<int>(i));
+        }
+        plan_.input = view_of(0);
+        // the result is the last operator of the last stage's last group
+        const auto &last_stage_units = unit_result_;
+        int out_node = last_stage_units.back();
+        plan_.output = view_of(out_node);
+        plan_.output_name = nodes_[out_node].name;
+        for (PlanConv &conv : plan_.convs) {
+            if (!conv.matrix_path) continue;
+            conv.ws_floats = conv_workspace_floats(conv.problem, conv.launch);
+            conv.num_counters = conv_num_counters(conv.problem, conv.launch);
+            if (conv.ws_floats > 0) {
+                conv.ws_off = reserve(conv.ws_floats);
+                conv.counter_off = reserve(conv.num_counters);
+            }
+        }
+    }
+
+    int batch_;
+    const LaunchChooser &chooser_;
+    Plan plan_;
+    std::vector<PNode> nodes_;
+    std::map<std::string, int> by_name_;
+    std::vector<std::string> units_;
+    std::vector<int> unit_result_;
+    struct SeqRange { int first, second; };
+    std::vector<SeqRange> sequentials_;
+};
+
+void json_escape(std::ostringstream &os, const std::string &s) {
+    os << '"';
+    for (char c : s) {
+        if (c == '"' || c == '\\') os << '\\' << c;
+        else if ((unsigned char)c < 0x20) os << ' ';
+        else os << c;
+    }
+    os << '"';
+}
+
+}  // namespace
+
+Plan build_plan(PlanMode mode, const Json &doc, const Json *extra, int batch, const LaunchChooser &chooser) {
+    Planner planner(batch, chooser);
+    return planner.run(mode, doc, extra);
+}
+
+std::string describe_plan(const Plan &plan) {
+    std::ostringstream os;
+    os << '[';
+    for (size_t i = 0; i < plan.ops.size(); i++) {
+        const PlanOp &op = plan.ops[i];
+        if (i) os << ',';
+        os << "{\"index\":" << i << ",\"node\":";
+        json_escape(os, op.node);
+        os << ",\"unit\":";
+        json_escape(os, plan.unit_names[op.unit]);
+        os << ",\"kind\":\"" << op_kind_name(op.kind) << "\",\"stage\":" << op.stage << ",\"group\":" << op.group;
+        os << ",\"flops\":" << op.flops << ",\"bytes\":" << op.bytes;
+        os << ",\"out\":[" << op.out.C << ',' << op.out.H << ',' << op.out.W << "],\"out_bstride\":" << op.out.bstride;
+        if (op.conv >= 0) {
+            const PlanConv &c = plan.convs[op.conv];
+            const ConvProblem &p = c.problem;
+            os << ",\"conv\":{\"ic\":" << p.IC << ",\"h\":" << p.H << ",\"w\":" << p.W << ",\"oc\":" << p.OC << ",\"kh\":" << p.KH
+               << ",\"kw\":" << p.KW << ",\"sh\":" << p.sh << ",\"sw\":" << p.sw << ",\"ph\":" << p.ph << ",\"pw\":" << p.pw
+               << ",\"groups\":" << p.groups << ",\"act\":" << p.act << ",\"pre_relu\":" << p.pre_relu << "}";
+            if (c.matrix_path) {
+                os << ",\"variant\":\"" << conv_variant(c.launch.variant).name << "\",\"split_k\":" << c.launch.split_k;
+            }
+        }
+        if (op.kind == OpKind::Nary) os << ",\"inputs\":" << op.srcs.size() << ",\"accumulate\":" << op.accumulate;
+        if (op.kind == OpKind::Nary || op.kind == OpKind::Unary) os << ",\"act\":" << op.act;
+        os << '}';
+    }
+    os << ']';
+    return os.str();
+}
+
+}  // namespace ios

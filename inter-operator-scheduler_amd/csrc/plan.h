@@ -1,0 +1,92 @@
+// Execution plan: the flat list of device operations, tensor views and the memory layout that a graph,
+// block or stage document compiles to.  Planning is pure host code; nothing here touches the device.
+//
+// Memory model: one arena of 4-byte words.  Every operator output, temporary, filter, bias, gather table,
+// split-K workspace and tile counter is a region of it at a 256-byte aligned offset.  Tensor views are
+// (offset, C, H, W, batch stride); a channel slice or a window of a concat buffer is again a view, so
+//   * an identity with one input value is an alias (no memory, no work),
+//   * a producer whose whole output is one term of a concat writes directly into the concat buffer,
+//   * a channel slice of a merged convolution is read in place at any batch size,
+//   * a ReLU that only feeds the next convolution of its Sequential is folded into that convolution's
+//     input loader.
+#pragma once
+
+#include <functional>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "json.h"
+#include "kernels.h"
+
+namespace ios {
+
+constexpr int kMaxGroups = 16;   // concurrent groups (streams) per stage
+
+struct ViewRef {
+    size_t offset = 0;   // in floats from the arena base
+    int C = 0, H = 0, W = 0;
+    long long bstride = 0;
+    ViewRef window(int begin, int end) const {
+        ViewRef v = *this;
+        v.offset += (size_t)begin * H * W;
+        v.C = end - begin;
+        return v;
+    }
+    size_t image_floats() const { return (size_t)C * H * W; }
+};
+
+enum class OpKind { ConvMfma, ConvDepthwise, ConvDirect, Pool, GlobalPool, Nary, Unary };
+const char *op_kind_name(OpKind kind);
+
+struct PlanConv {
+    std::string name;
+    ConvProblem problem;
+    size_t weight_off = 0, bias_off = 0;       // original layouts
+    size_t packed_off = 0, ktab_off = 0;       // matrix path only
+    size_t ws_off = 0, counter_off = 0;        // split-K only
+    size_t ws_floats = 0, num_counters = 0;
+    ConvLaunch launch;
+    bool matrix_path = false;
+};
+
+struct PlanOp {
+    OpKind kind;
+    std::string node;     // operator name in the document
+    int unit = -1;        // schedule unit (top-level operator) this op belongs to
+    int stage = -1, group = -1;
+    ViewRef in, out;
+    int conv = -1;        // index into Plan::convs
+    PoolProblem pool{};
+    std::vector<ViewRef> srcs;   // Nary
+    int multiply = 0, accumulate = 0, act = 0;
+    double flops = 0.0, bytes = 0.0;
+};
+
+struct Plan {
+    int batch = 1;
+    std::vector<PlanOp> ops;
+    std::vector<PlanConv> convs;
+    std::vector<std::vector<std::vector<int>>> stages;   // stage -> group -> op indices in launch order
+    std::vector<std::string> unit_names;
+    std::map<std::string, ViewRef> tensors;              // operator name -> materialised output view
+    std::map<std::string, int> conv_index;               // convolution name -> index into convs
+    ViewRef input, output;
+    std::string input_name, output_name;
+    size_t arena_floats = 0;
+    bool output_single_group = true;                     // the last stage has one group
+};
+
+enum class PlanMode { Graph, Block, Stage };
+
+// Picks the kernel configuration of a matrix-path convolution (closed-form model or measured).
+typedef std::function<ConvLaunch(const ConvProblem &)> LaunchChooser;
+
+// Compile a document.  `extra` is the input-shape document of stage mode ({name: [C, H, W]}).
+// Throws std::runtime_error on malformed documents, unknown operator types, non-topological schedules
+// and stages with too many groups.
+Plan build_plan(PlanMode mode, const Json &doc, const Json *extra, int batch, const LaunchChooser &chooser);
+
+std::string describe_plan(const Plan &plan);   // JSON array, one object per op
+
+}  // namespace ios

@@ -1,0 +1,104 @@
+// Device-side half of the runtime: the process-wide device context (stream pool, reusable arena, options,
+// kernel-configuration cache) and Session, a plan bound to device memory that can be run, timed per
+// stage and profiled per operation.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "plan.h"
+
+namespace ios {
+
+void hip_check(hipError_t status, const char *what, const char *file, int line);
+#define IOS_HIP(call) ::ios::hip_check((call), #call, __FILE__, __LINE__)
+
+enum class ExecMode { Streams, Graph };
+
+class DeviceContext {
+public:
+    static DeviceContext &get();   // initialises the device on first use
+
+    int num_cus() const { return num_cus_; }
+    const std::string &name() const { return name_; }
+    const std::string &arch() const { return arch_; }
+    hipStream_t stream(int group) { return streams_[group]; }
+
+    // a process-wide arena reused by the stateless latency / inference entry points
+    float *shared_arena(size_t floats);
+
+    void set_option(const std::string &key, const std::string &value);
+    ExecMode exec_mode() const { return exec_mode_; }
+    bool autotune() const { return autotune_; }
+    // testing aid: force one kernel configuration for every matrix-path convolution (-1 / 0 = off)
+    int forced_variant() const { return forced_variant_; }
+    int forced_split_k() const { return forced_split_k_; }
+    std::string info_json() const;
+
+    // measured kernel configurations, keyed by problem signature
+    std::map<std::string, ConvLaunch> tuned;
+
+private:
+    DeviceContext();
+    int num_cus_ = 0;
+    std::string name_, arch_;
+    hipStream_t streams_[kMaxGroups];
+    float *arena_ = nullptr;
+    size_t arena_floats_ = 0;
+    ExecMode exec_mode_ = ExecMode::Streams;
+    bool autotune_ = false;
+    int forced_variant_ = -1;
+    int forced_split_k_ = 0;
+};
+
+class Session {
+public:
+    // `shared` sessions live in the context's shared arena (one at a time), others own their memory
+    Session(Plan plan, bool shared);
+    ~Session();
+    Session(const Session &) = delete;
+    Session &operator=(const Session &) = delete;
+
+    const Plan &plan() const { return plan_; }
+
+    void set_input(const float *host);
+    // returns false (and prints like the reference runtime) when no convolution has that name
+    bool set_conv_weights(const char *name, const float *weight, const float *bias);
+    void get_output(float *host);
+    void get_tensor(const std::string &name, float *host);
+
+    void run();   // one forward pass, synchronised
+    // reference timing protocol for graphs / blocks: per repeat the mean of `number` individually
+    // bracketed forward passes; optional per-stage times from events recorded after every stage
+    void measure(int warmup, int number, int repeat, bool profile_stage, float *results, float *stage_results);
+    // reference timing protocol for stage probes: `number` back-to-back passes in one bracket
+    void measure_back_to_back(int warmup, int number, int repeat, float *results);
+    void profile_ops(int warmup, int repeat, float *ms);
+
+private:
+    void setup();
+    void tune_convs();
+    void launch_op(const PlanOp &op, hipStream_t stream);
+    void enqueue(bool stage_events);   // issue one forward pass on the stream pool
+    void forward();                    // enqueue or graph launch according to the execution mode
+    void build_graph();
+    void copy_out(const ViewRef &view, float *host);
+    TensorView tv(const ViewRef &v) const;
+
+    Plan plan_;
+    DeviceContext &ctx_;
+    float *base_ = nullptr;
+    bool owns_memory_ = false;
+    std::vector<hipEvent_t> fork_events_;                 // per stage (multi-group stages only)
+    std::vector<std::vector<hipEvent_t>> join_events_;    // per stage, per extra group
+    std::vector<hipEvent_t> stage_events_;                // per stage, profile mode
+    hipEvent_t start_ = nullptr, stop_ = nullptr;
+    hipGraph_t graph_ = nullptr;
+    hipGraphExec_t graph_exec_ = nullptr;
+};
+
+}  // namespace ios

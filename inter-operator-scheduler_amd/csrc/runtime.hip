@@ -1,0 +1,375 @@
+// Stage executor, timers and device context.
+//
+// A forward pass walks the plan's stages.  Group g of a stage is issued to stream g of a fixed pool;
+// stream 0 is the main stream.  A multi-group stage forks (the extra streams wait on an event recorded on
+// the main stream) and joins (the main stream waits on one event per extra stream), so stage boundaries
+// are device-side dependencies and the host never blocks inside a pass.  In graph mode the same
+// issue sequence is captured once into a hipGraph and replayed.
+//
+// Timing follows the reference runtime (src/ios/ios_runtime.cu:1328-1455): graph / block latency is the
+// mean over `number` individually bracketed passes per repeat, with optional per-stage times from events
+// recorded on the main stream after every stage; stage probes time `number` back-to-back passes inside
+// one event pair.
+#include "runtime.h"
+
+#include <cstdio>
+#include <cstring>
+#include <sstream>
+#include <stdexcept>
+
+namespace ios {
+
+void hip_check(hipError_t status, const char *what, const char *file, int line) {
+    if (status == hipSuccess) return;
+    std::ostringstream os;
+    os << "HIP failure " << hipGetErrorString(status) << " (" << (int)status << ") in " << what << " at " << file << ":" << line;
+    throw std::runtime_error(os.str());
+}
+
+// ---- device context --------------------------------------------------------------------------------------------
+DeviceContext &DeviceContext::get() {
+    static DeviceContext instance;
+    return instance;
+}
+
+DeviceContext::DeviceContext() {
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count < 1) throw std::runtime_error("no HIP device available");
+    IOS_HIP(hipSetDevice(0));
+    hipDeviceProp_t prop;
+    IOS_HIP(hipGetDeviceProperties(&prop, 0));
+    num_cus_ = prop.multiProcessorCount;
+    name_ = prop.name;
+    arch_ = prop.gcnArchName;
+    for (int i = 0; i < kMaxGroups; i++) IOS_HIP(hipStreamCreateWithFlags(&streams_[i], hipStreamNonBlocking));
+    const char *mode = getenv("IOS_EXECUTOR");
+    if (mode != nullptr) set_option("executor", mode);
+    const char *tune = getenv("IOS_AUTOTUNE");
+    if (tune != nullptr) set_option("autotune", tune);
+}
+
+float *DeviceContext::shared_arena(size_t floats) {
+    if (floats > arena_floats_) {
+        IOS_HIP(hipDeviceSynchronize());
+        if (arena_ != nullptr) IOS_HIP(hipFree(arena_));
+        arena_ = nullptr;
+        arena_floats_ = 0;
+        const size_t want = floats + floats / 4 + (1u << 20);
+        IOS_HIP(hipMalloc(reinterpret_cast<void **>(&arena_), want * sizeof(float)));
+        arena_floats_ = want;
+        // latency probes run on whatever the arena holds; start from finite, varied values
+        launch_fill_pattern(arena_, arena_floats_, 0x1234567u, streams_[0]);
+        IOS_HIP(hipStreamSynchronize(streams_[0]));
+    }
+    return arena_;
+}
+
+void DeviceContext::set_option(const std::string &key, const std::string &value) {
+    if (key == "executor") {
+        if (value == "streams") exec_mode_ = ExecMode::Streams;
+        else if (value == "graph") exec_mode_ = ExecMode::Graph;
+        else throw std::runtime_error("option executor: expected 'streams' or 'graph', got '" + value + "'");
+    } else if (key == "autotune") {
+        autotune_ = !(value == "0" || value == "false" || value == "off" || value.empty());
+    } else if (key == "conv_variant") {
+        const int v = atoi(value.c_str());
+        if (v < -1 || v >= conv_num_variants()) throw std::runtime_error("option conv_variant: index out of range");
+        forced_variant_ = v;
+    } else if (key == "conv_split_k") {
+        const int v = atoi(value.c_str());
+        if (v < 0 || v > 64) throw std::runtime_error("option conv_split_k: expected 0..64");
+        forced_split_k_ = v;
+    } else if (key == "clear_tuning") {
+        tuned.clear();
+    } else {
+        throw std::runtime_error("unknown option '" + key + "'");
+    }
+}
+
+std::string DeviceContext::info_json() const {
+    std::ostringstream os;
+    os << "{\"name\":\"" << name_ << "\",\"arch\":\"" << arch_ << "\",\"compute_units\":" << num_cus_
+       << ",\"executor\":\"" << (exec_mode_ == ExecMode::Graph ? "graph" : "streams") << "\",\"autotune\":" << (autotune_ ? "true" : "false")
+       << ",\"max_groups\":" << kMaxGroups << "}";
+    return os.str();
+}
+
+// ---- session ---------------------------------------------------------------------------------------------------------
+Session::Session(Plan plan, bool shared) : plan_(std::move(plan)), ctx_(DeviceContext::get()) {
+    if (shared) {
+        base_ = ctx_.shared_arena(plan_.arena_floats);
+        owns_memory_ = false;
+    } else {
+        IOS_HIP(hipMalloc(reinterpret_cast<void **>(&base_), std::max<size_t>(plan_.arena_floats, 64) * sizeof(float)));
+        owns_memory_ = true;
+    }
+    try {
+        setup();
+    } catch (...) {
+        if (owns_memory_ && base_ != nullptr) (void)hipFree(base_);
+        throw;
+    }
+}
+
+Session::~Session() {
+    (void)hipDeviceSynchronize();
+    if (graph_exec_ != nullptr) (void)hipGraphExecDestroy(graph_exec_);
+    if (graph_ != nullptr) (void)hipGraphDestroy(graph_);
+    for (hipEvent_t e : fork_events_)
+        if (e != nullptr) (void)hipEventDestroy(e);
+    for (auto &per_stage : join_events_)
+        for (hipEvent_t e : per_stage) (void)hipEventDestroy(e);
+    for (hipEvent_t e : stage_events_) (void)hipEventDestroy(e);
+    if (start_ != nullptr) (void)hipEventDestroy(start_);
+    if (stop_ != nullptr) (void)hipEventDestroy(stop_);
+    if (owns_memory_ && base_ != nullptr) (void)hipFree(base_);
+}
+
+TensorView Session::tv(const ViewRef &v) const {
+    TensorView t;
+    t.ptr = base_ + v.offset;
+    t.C = v.C;
+    t.H = v.H;
+    t.W = v.W;
+    t.bstride = v.bstride;
+    return t;
+}
+
+void Session::setup() {
+    hipStream_t main = ctx_.stream(0);
+    if (owns_memory_) launch_fill_pattern(base_, plan_.arena_floats, 0x2468aceu, main);
+    for (const PlanConv &conv : plan_.convs) {
+        if (!conv.matrix_path) continue;
+        launch_build_ktab(conv.problem, reinterpret_cast<int2 *>(base_ + conv.ktab_off), main);
+        if (conv.ws_floats > 0) launch_fill_u32(reinterpret_cast<unsigned *>(base_ + conv.counter_off), conv.num_counters, 0u, main);
+        // the probes never upload filters: pack whatever the filter region holds so that the matrix
+        // path reads initialised memory
+        launch_pack_filters(conv.problem, base_ + conv.weight_off, base_ + conv.packed_off, main);
+    }
+    const size_t num_stages = plan_.stages.size();
+    fork_events_.assign(num_stages, nullptr);
+    join_events_.assign(num_stages, {});
+    for (size_t s = 0; s < num_stages; s++) {
+        const size_t groups = plan_.stages[s].size();
+        if (groups <= 1) continue;
+        IOS_HIP(hipEventCreateWithFlags(&fork_events_[s], hipEventDisableTiming));
+        join_events_[s].resize(groups - 1);
+        for (hipEvent_t &e : join_events_[s]) IOS_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    }
+    IOS_HIP(hipEventCreate(&start_));
+    IOS_HIP(hipEventCreate(&stop_));
+    IOS_HIP(hipStreamSynchronize(main));
+}
+
+void Session::set_input(const float *host) {
+    if (host == nullptr) throw std::runtime_error("input pointer is null");
+    hipStream_t main = ctx_.stream(0);
+    const ViewRef &in = plan_.input;
+    IOS_HIP(hipMemcpyAsync(base_ + in.offset, host, (size_t)plan_.batch * in.image_floats() * sizeof(float), hipMemcpyHostToDevice, main));
+    IOS_HIP(hipStreamSynchronize(main));
+}
+
+bool Session::set_conv_weights(const char *name, const float *weight, const float *bias) {
+    auto it = plan_.conv_index.find(name ? name : "");
+    if (it == plan_.conv_index.end()) {
+        printf("%s not found\n", name ? name : "(null)");
+        return false;
+    }
+    if (weight == nullptr || bias == nullptr) throw std::runtime_error(std::string("convolution '") + name + "': weight or bias pointer is null");
+    const PlanConv &conv = plan_.convs[it->second];
+    const ConvProblem &p = conv.problem;
+    hipStream_t main = ctx_.stream(0);
+    IOS_HIP(hipMemcpyAsync(base_ + conv.weight_off, weight, (size_t)p.OC * p.K() * sizeof(float), hipMemcpyHostToDevice, main));
+    IOS_HIP(hipMemcpyAsync(base_ + conv.bias_off, bias, (size_t)p.OC * sizeof(float), hipMemcpyHostToDevice, main));
+    if (conv.matrix_path) launch_pack_filters(p, base_ + conv.weight_off, base_ + conv.packed_off, main);
+    IOS_HIP(hipStreamSynchronize(main));
+    return true;
+}
+
+void Session::copy_out(const ViewRef &view, float *host) {
+    hipStream_t main = ctx_.stream(0);
+    const size_t image = view.image_floats();
+    if (view.bstride == (long long)image) {
+        IOS_HIP(hipMemcpyAsync(host, base_ + view.offset, (size_t)plan_.batch * image * sizeof(float), hipMemcpyDeviceToHost, main));
+    } else {
+        for (int b = 0; b < plan_.batch; b++)
+            IOS_HIP(hipMemcpyAsync(host + (size_t)b * image, base_ + view.offset + (size_t)b * view.bstride, image * sizeof(float),
+                                   hipMemcpyDeviceToHost, main));
+    }
+    IOS_HIP(hipStreamSynchronize(main));
+}
+
+void Session::get_output(float *host) {
+    if (host == nullptr) throw std::runtime_error("output pointer is null");
+    if (!plan_.output_single_group) throw std::runtime_error("the last stage of the schedule must have a single group");
+    copy_out(plan_.output, host);
+}
+
+void Session::get_tensor(const std::string &name, float *host) {
+    auto it = plan_.tensors.find(name);
+    if (it == plan_.tensors.end()) throw std::runtime_error("operator '" + name + "' has no materialised output");
+    copy_out(it->second, host);
+}
+
+void Session::launch_op(const PlanOp &op, hipStream_t stream) {
+    switch (op.kind) {
+        case OpKind::ConvMfma: {
+            const PlanConv &c = plan_.convs[op.conv];
+            launch_conv_mfma(c.problem, c.launch, tv(op.in), base_ + c.packed_off, reinterpret_cast<const int2 *>(base_ + c.ktab_off),
+                             base_ + c.bias_off, tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr,
+                             c.ws_floats ? reinterpret_cast<unsigned *>(base_ + c.counter_off) : nullptr, stream);
+            break;
+        }
+        case OpKind::ConvDepthwise: {
+            const PlanConv &c = plan_.convs[op.conv];
+            launch_dwconv(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), stream);
+            break;
+        }
+        case OpKind::ConvDirect: {
+            const PlanConv &c = plan_.convs[op.conv];
+            launch_conv_direct(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), stream);
+            break;
+        }
+        case OpKind::Pool: launch_pool(op.pool, tv(op.in), tv(op.out), stream); break;
+        case OpKind::GlobalPool: launch_global_pool(op.pool, tv(op.in), tv(op.out), stream); break;
+        case OpKind::Nary: {
+            NaryArgs a;
+            a.count = (int)op.srcs.size();
+            for (int i = 0; i < a.count; i++) {
+                a.src[i] = base_ + op.srcs[i].offset;
+                a.src_bstride[i] = op.srcs[i].bstride;
+            }
+            launch_nary(a, op.multiply, op.accumulate, op.act, plan_.batch, (long long)op.out.image_floats(), tv(op.out), stream);
+            break;
+        }
+        case OpKind::Unary: launch_unary(tv(op.in), tv(op.out), op.act, plan_.batch, stream); break;
+    }
+}
+
+void Session::enqueue(bool stage_events) {
+    hipStream_t main = ctx_.stream(0);
+    for (size_t s = 0; s < plan_.stages.size(); s++) {
+        const auto &groups = plan_.stages[s];
+        const bool fork = groups.size() > 1;
+        if (fork) {
+            IOS_HIP(hipEventRecord(fork_events_[s], main));
+            for (size_t g = 1; g < groups.size(); g++) IOS_HIP(hipStreamWaitEvent(ctx_.stream((int)g), fork_events_[s], 0));
+        }
+        for (size_t g = 0; g < groups.size(); g++)
+            for (int op : groups[g]) launch_op(plan_.ops[op], ctx_.stream((int)g));
+        if (fork) {
+            for (size_t g = 1; g < groups.size(); g++) {
+                IOS_HIP(hipEventRecord(join_events_[s][g - 1], ctx_.stream((int)g)));
+                IOS_HIP(hipStreamWaitEvent(main, join_events_[s][g - 1], 0));
+            }
+        }
+        if (stage_events) IOS_HIP(hipEventRecord(stage_events_[s], main));
+    }
+}
+
+void Session::build_graph() {
+    hipStream_t main = ctx_.stream(0);
+    IOS_HIP(hipStreamBeginCapture(main, hipStreamCaptureModeRelaxed));
+    try {
+        enqueue(false);
+    } catch (...) {
+        hipGraph_t broken = nullptr;
+        (void)hipStreamEndCapture(main, &broken);
+        if (broken != nullptr) (void)hipGraphDestroy(broken);
+        throw;
+    }
+    IOS_HIP(hipStreamEndCapture(main, &graph_));
+    IOS_HIP(hipGraphInstantiate(&graph_exec_, graph_, nullptr, nullptr, 0));
+}
+
+void Session::forward() {
+    if (ctx_.exec_mode() == ExecMode::Graph) {
+        if (graph_exec_ == nullptr) build_graph();
+        IOS_HIP(hipGraphLaunch(graph_exec_, ctx_.stream(0)));
+    } else {
+        enqueue(false);
+    }
+}
+
+void Session::run() {
+    forward();
+    IOS_HIP(hipStreamSynchronize(ctx_.stream(0)));
+}
+
+void Session::measure(int warmup, int number, int repeat, bool profile_stage, float *results, float *stage_results) {
+    if (number < 1 || repeat < 1 || warmup < 0) throw std::runtime_error("measure: warmup >= 0, number >= 1, repeat >= 1 required");
+    hipStream_t main = ctx_.stream(0);
+    const size_t num_stages = plan_.stages.size();
+    if (profile_stage && stage_events_.empty()) {
+        stage_events_.resize(num_stages);
+        for (hipEvent_t &e : stage_events_) IOS_HIP(hipEventCreate(&e));
+    }
+    auto pass = [&]() {
+        if (profile_stage) enqueue(true);
+        else forward();
+    };
+    for (int i = 0; i < warmup; i++) pass();
+    for (int i = 0; i < repeat; i++) {
+        double total = 0.0;
+        std::vector<double> per_stage(num_stages, 0.0);
+        for (int t = 0; t < number; t++) {
+            IOS_HIP(hipDeviceSynchronize());
+            IOS_HIP(hipEventRecord(start_, main));
+            pass();
+            IOS_HIP(hipEventRecord(stop_, main));
+            IOS_HIP(hipEventSynchronize(stop_));
+            float ms = 0.f;
+            if (profile_stage) {
+                for (size_t s = 0; s < num_stages; s++) {
+                    hipEvent_t from = s == 0 ? start_ : stage_events_[s - 1];
+                    hipEvent_t to = s + 1 == num_stages ? stop_ : stage_events_[s];
+                    IOS_HIP(hipEventElapsedTime(&ms, from, to));
+                    per_stage[s] += ms;
+                }
+            }
+            IOS_HIP(hipEventElapsedTime(&ms, start_, stop_));
+            total += ms;
+        }
+        results[i] = (float)(total / number);
+        if (profile_stage && stage_results != nullptr)
+            for (size_t s = 0; s < num_stages; s++) stage_results[i * num_stages + s] = (float)(per_stage[s] / number);
+    }
+    IOS_HIP(hipDeviceSynchronize());
+}
+
+void Session::measure_back_to_back(int warmup, int number, int repeat, float *results) {
+    if (number < 1 || repeat < 1 || warmup < 0) throw std::runtime_error("measure: warmup >= 0, number >= 1, repeat >= 1 required");
+    hipStream_t main = ctx_.stream(0);
+    for (int i = 0; i < warmup; i++) forward();
+    for (int i = 0; i < repeat; i++) {
+        IOS_HIP(hipDeviceSynchronize());
+        IOS_HIP(hipEventRecord(start_, main));
+        for (int t = 0; t < number; t++) forward();
+        IOS_HIP(hipEventRecord(stop_, main));
+        IOS_HIP(hipEventSynchronize(stop_));
+        float ms = 0.f;
+        IOS_HIP(hipEventElapsedTime(&ms, start_, stop_));
+        results[i] = ms / (float)number;
+    }
+    IOS_HIP(hipDeviceSynchronize());
+}
+
+void Session::profile_ops(int warmup, int repeat, float *ms_out) {
+    if (repeat < 1 || warmup < 0) throw std::runtime_error("profile_ops: warmup >= 0 and repeat >= 1 required");
+    hipStream_t main = ctx_.stream(0);
+    run();   // every operator sees the inputs it has in a real pass
+    for (size_t i = 0; i < plan_.ops.size(); i++) {
+        const PlanOp &op = plan_.ops[i];
+        for (int w = 0; w < warmup; w++) launch_op(op, main);
+        IOS_HIP(hipStreamSynchronize(main));
+        IOS_HIP(hipEventRecord(start_, main));
+        for (int r = 0; r < repeat; r++) launch_op(op, main);
+        IOS_HIP(hipEventRecord(stop_, main));
+        IOS_HIP(hipEventSynchronize(stop_));
+        float ms = 0.f;
+        IOS_HIP(hipEventElapsedTime(&ms, start_, stop_));
+        ms_out[i] = ms / (float)repeat;
+    }
+}
+
+}  // namespace ios

@@ -54,6 +54,8 @@ def _declare(handle):
     handle.ios_set_option.restype = i
     handle.ios_device_info.argtypes = [ctypes.c_char_p, i]
     handle.ios_device_info.restype = i
+    handle.ios_plan_describe.argtypes = [s, i, ctypes.c_char_p, i]
+    handle.ios_plan_describe.restype = i
     handle.ios_session_create.argtypes = [s, i]
     handle.ios_session_create.restype = vp
     handle.ios_session_destroy.argtypes = [vp]
@@ -108,6 +110,21 @@ def device_info() -> dict:
     buf = ctypes.create_string_buffer(4096)
     _check(get_lib().ios_device_info(buf, len(buf)), 'ios_device_info')
     return json.loads(buf.value.decode())
+
+
+def plan_describe(graph: Graph, batch_size=1) -> List[dict]:
+    """Device operations the library would launch for ``graph`` (host-only planning, needs no GPU)."""
+    handle = get_lib()
+    doc = c_string(json.dumps(graph.export_config()))
+    cap = 1 << 16
+    while True:
+        buf = ctypes.create_string_buffer(cap)
+        need = handle.ios_plan_describe(doc, c_int(batch_size), buf, c_int(cap))
+        if need < 0:
+            _check(1, 'ios_plan_describe')
+        if need < cap:
+            return json.loads(buf.value.decode())
+        cap = need + 1
 
 
 def _latency_call(fn_name, documents, batch_size, warmup, number, repeat, num_stages, profile_stage):

@@ -1,0 +1,289 @@
+"""
+GPU parity: the HIP runtime, called through its C ABI, against the CPU oracle on the same seeded inputs.
+Tolerance for fp32: |got - want| <= 1e-4 + 1e-3 * |want| (abs 1e-4, rel 1e-3).
+Schedule changes must not change results at all (bit-identical outputs).
+"""
+import numpy as np
+import pytest
+
+import ios
+from ios.contrib import ios_runtime as rt
+from ios.ir import Graph, Value
+from oracle import ios_oracle
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-3, 1e-4
+
+
+def assert_close(got, want, what=''):
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    bound = ATOL + RTOL * np.abs(want.astype(np.float64))
+    bad = err > bound
+    assert not bad.any(), (f'{what}: {bad.sum()} of {bad.size} elements out of tolerance, max abs err '
+                           f'{err.max():.3e} at {np.unravel_index(err.argmax(), err.shape)}, '
+                           f'want there {want.flat[err.argmax()]:.6f} got {got.flat[err.argmax()]:.6f}')
+
+
+@pytest.fixture(autouse=True)
+def default_options():
+    rt.set_option('conv_variant', -1)
+    rt.set_option('conv_split_k', 0)
+    rt.set_option('executor', 'streams')
+    yield
+    rt.set_option('conv_variant', -1)
+    rt.set_option('conv_split_k', 0)
+    rt.set_option('executor', 'streams')
+
+
+def single_op_graph(in_shape, build):
+    ios.reset_name()
+    v = ios.placeholder(in_shape)
+    block = ios.Block(v.node)
+    build(block, v)
+    graph = Graph('t', v.node, [block])
+    graph.init_weights(seed=7, scheme='he_normal')
+    for conv in graph.conv_nodes():   # non-zero bias so that a dropped bias fails
+        conv.bias = np.random.default_rng(int(conv.name) + 100).standard_normal(conv.bias.shape).astype(np.float32) * 0.5
+    graph.sequential_schedule()
+    return graph
+
+
+def run_both(graph, batch, seed=1):
+    x = np.random.default_rng(seed).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
+    got = rt.graph_inference(graph, batch, x)
+    want = ios_oracle.run(graph, x)
+    assert got.shape == want.shape
+    return got, want
+
+
+CONVS = [
+    # in_shape, out_channels, kernel, stride, padding, groups, act, batch
+    ((16, 9, 9), 24, (3, 3), (1, 1), (1, 1), 1, 'relu', 1),
+    ((3, 31, 31), 32, (3, 3), (2, 2), (0, 0), 1, 'relu', 2),
+    ((48, 17, 17), 64, (5, 5), (1, 1), (2, 2), 1, 'relu', 1),
+    ((40, 17, 17), 48, (1, 7), (1, 1), (0, 3), 1, 'relu', 1),
+    ((40, 17, 17), 48, (7, 1), (1, 1), (3, 0), 1, 'identity', 3),
+    ((192, 8, 8), 100, (1, 1), (1, 1), (0, 0), 1, 'tanh', 1),
+    ((70, 12, 12), 33, (1, 1), (2, 2), (0, 0), 1, 'sigmoid', 2),
+    ((375, 15, 15), 75, (3, 3), (1, 1), (1, 1), 1, 'relu', 1),       # odd channel counts (sample net)
+    ((32, 14, 14), 32, (3, 3), (1, 1), (1, 1), 32, 'identity', 2),   # depthwise 3x3
+    ((24, 15, 15), 24, (5, 5), (2, 2), (2, 2), 24, 'identity', 1),   # depthwise 5x5 strided
+    ((16, 13, 13), 16, (7, 7), (2, 2), (3, 3), 16, 'relu', 1),       # depthwise 7x7
+    ((32, 10, 10), 48, (3, 3), (1, 1), (1, 1), 4, 'relu', 2),        # grouped, matrix path per group
+    ((12, 10, 10), 12, (3, 3), (1, 1), (1, 1), 6, 'relu', 1),        # thin groups, direct path
+    ((8, 7, 7), 10, (3, 3), (1, 1), (2, 2), 1, 'identity', 1),       # padding larger than "same"
+]
+
+
+@pytest.mark.parametrize('case', CONVS)
+def test_conv_matches_oracle(case):
+    in_shape, oc, k, s, p, g, act, batch = case
+    graph = single_op_graph(in_shape, lambda b, v: ios.conv2d(b, [[v]], oc, k, s, p, g, act, is_exit=True))
+    got, want = run_both(graph, batch)
+    assert_close(got, want, f'conv {case}')
+
+
+@pytest.mark.parametrize('variant', range(8))
+@pytest.mark.parametrize('split_k', [1, 3])
+def test_every_conv_kernel_variant(variant, split_k):
+    rt.set_option('conv_variant', variant)
+    rt.set_option('conv_split_k', split_k)
+    for in_shape, oc, k, s, p, batch in [((72, 19, 19), 88, (3, 3), (1, 1), (1, 1), 2),
+                                          ((200, 8, 8), 136, (1, 1), (1, 1), (0, 0), 1),
+                                          ((20, 37, 37), 24, (5, 5), (2, 2), (2, 2), 1)]:
+        graph = single_op_graph(in_shape, lambda b, v: ios.conv2d(b, [[v]], oc, k, s, p, 1, 'relu', is_exit=True))
+        got, want = run_both(graph, batch)
+        assert_close(got, want, f'variant {variant} split {split_k} conv {in_shape}->{oc} {k}')
+        got2, _ = run_both(graph, batch)
+        np.testing.assert_array_equal(got, got2)      # split-K reduction order is fixed
+
+
+def test_split_k_counters_are_reusable_in_a_session():
+    rt.set_option('conv_split_k', 4)
+    graph = single_op_graph((64, 12, 12), lambda b, v: ios.conv2d(b, [[v]], 40, (3, 3), (1, 1), (1, 1), 1, 'relu', is_exit=True))
+    x = np.random.default_rng(3).standard_normal((2, 64, 12, 12)).astype(np.float32)
+    want = ios_oracle.run(graph, x)
+    with rt.Session(graph, 2) as session:
+        session.load_weights()
+        session.set_input(x)
+        for _ in range(3):
+            session.run()
+            assert_close(session.output(), want, 'repeated split-K run')
+
+
+POOLS = [
+    ((24, 35, 35), 'max', (3, 3), (2, 2), (0, 0), 1),
+    ((24, 17, 17), 'avg', (3, 3), (1, 1), (1, 1), 2),
+    ((10, 14, 14), 'max', (3, 3), (2, 2), (1, 1), 1),
+    ((10, 15, 15), 'avg', (3, 3), (2, 2), (1, 1), 1),
+    ((6, 8, 8), 'max', (2, 2), (2, 2), (0, 0), 3),
+    ((40, 8, 8), 'global_avg', (1, 1), (1, 1), (0, 0), 2),
+    ((9, 13, 13), 'global_max', (1, 1), (1, 1), (0, 0), 1),
+]
+
+
+@pytest.mark.parametrize('case', POOLS)
+def test_pool_matches_oracle(case):
+    in_shape, kind, k, s, p, batch = case
+    graph = single_op_graph(in_shape, lambda b, v: ios.pool2d(b, [[v]], kind, k, s, p, is_exit=True))
+    x = np.random.default_rng(2).standard_normal((batch, *in_shape)).astype(np.float32) - 2.0   # mostly negative
+    got = rt.graph_inference(graph, batch, x)
+    want = ios_oracle.run(graph, x)
+    assert_close(got, want, f'pool {case}')
+
+
+def test_input_algebra_sum_concat_slice_activation_element():
+    def build(b, v):
+        a = ios.conv2d(b, [[v]], 12, (1, 1), act='identity')
+        c = ios.conv2d(b, [[v]], 12, (3, 3), padding=(1, 1), act='identity')
+        s = ios.identity(b, [[a, c, a]])                                   # three-way sum
+        cat = ios.identity(b, [[a], [Value(c.node, 2, 8)], [a, c]])        # concat of value, slice, sum
+        r = ios.relu(b, [[cat]])
+        t = ios.activation(b, [[s], [Value(r.node, 0, 6)]], 'tanh', False)
+        m = ios.multiply(b, [[a, c]])
+        e = ios.addition(b, [[m, s]])
+        p = ios.pool2d(b, [[e, a]], 'avg', (3, 3), (1, 1), (1, 1))          # pool over a summed input
+        q = ios.conv2d(b, [[t], [p]], 10, (3, 3), padding=(1, 1))           # conv over a concatenated input
+        ios.identity(b, [[q], [Value(r.node, 3, 30)], [Value(t.node, 1, 18)]], is_exit=True)
+    graph = single_op_graph((5, 11, 11), build)
+    for batch in (1, 3):
+        x = np.random.default_rng(4).standard_normal((batch, 5, 11, 11)).astype(np.float32)
+        want = ios_oracle.run(graph, x, keep_all=True)
+        with rt.Session(graph, batch) as session:
+            session.load_weights()
+            session.set_input(x)
+            session.run()
+            for node in list(graph.nodes())[1:]:
+                assert_close(session.tensor(node), want[node.name], f'node {node.name} ({node.type}) batch {batch}')
+
+
+def test_wide_sum_uses_accumulation():
+    def build(b, v):
+        parts = [ios.conv2d(b, [[v]], 6, (1, 1), act='identity') for _ in range(11)]
+        ios.relu(b, [parts], is_exit=True)
+    graph = single_op_graph((4, 6, 6), build)
+    got, want = run_both(graph, 2)
+    assert_close(got, want, 'sum of 11 values')
+
+
+def test_sequential_units_and_folded_relu():
+    def build(b, v):
+        a = ios.relu_sep_conv(b, [[v]], 12, (3, 3), (2, 2), (1, 1))
+        c = ios.relu_conv(b, [[a]], 9, (1, 1))
+        d = ios.sep_conv(b, [[a]], 9, (5, 5), (1, 1), (2, 2))
+        ios.relu_sep_conv(b, [[c, d]], 7, (3, 3), (1, 1), (1, 1), is_exit=True)
+    graph = single_op_graph((8, 12, 12), build)
+    for batch in (1, 2):
+        got, want = run_both(graph, batch)
+        assert_close(got, want, 'sequential units')
+
+
+def model_cases():
+    return [
+        ('sample', lambda: ios.models.sample_network(init_seed=0, init_scheme='he_normal'), 1),
+        ('squeezenet_1_1', lambda: ios.models.squeezenet_1_1(init_seed=0, init_scheme='he_normal'), 1),
+        ('inception_v3', lambda: ios.models.inception_v3(init_seed=0, init_scheme='he_normal'), 1),
+        ('randwire_small', lambda: ios.models.randwire_small(init_seed=0, init_scheme='he_normal'), 1),
+        ('nasnet_mobile', lambda: ios.models.nasnet_mobile(init_seed=0, init_scheme='he_normal'), 1),
+        ('inception_v3_b4', lambda: ios.models.inception_v3(init_seed=0, init_scheme='he_normal'), 4),
+    ]
+
+
+@pytest.mark.parametrize('name,make,batch', model_cases(), ids=[c[0] for c in model_cases()])
+def test_network_matches_oracle_and_schedules_agree_bitwise(name, make, batch):
+    graph = make()
+    graph.sequential_schedule()
+    x = np.random.default_rng(1).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
+    want_all = ios_oracle.run(graph, x, keep_all=True)
+    want = want_all[graph.exit_node.name]
+    with rt.Session(graph, batch) as session:
+        session.load_weights()
+        session.set_input(x)
+        session.run()
+        got = session.output()
+        if not np.allclose(got, want, rtol=RTOL, atol=ATOL):
+            # name the first operator that went wrong
+            for node in list(graph.nodes())[1:]:
+                assert_close(session.tensor(node), want_all[node.name], f'{name}: node {node.name} ({node.type})')
+    assert_close(got, want, name)
+    assert np.isfinite(got).all() and np.abs(got).max() > 0
+
+    graph.greedy_schedule(4)
+    greedy = rt.graph_inference(graph, batch, x)
+    np.testing.assert_array_equal(greedy, got)
+
+    optimized = ios.optimize(graph, batch, ios.AnalyticCostModel(), 'dp_parallel', max_group_size=2,
+                             max_num_groups=4 if name.startswith(('randwire', 'nasnet')) else 8,
+                             max_part_size=12 if name.startswith('randwire') else 100, compute_weight=True)
+    assert any(len(stage) > 1 for block in optimized.blocks for stage in block.stages)
+    parallel = rt.graph_inference(optimized, batch, x)
+    np.testing.assert_array_equal(parallel, got)
+
+    rt.set_option('executor', 'graph')
+    with rt.Session(optimized, batch) as session:
+        session.load_weights()
+        session.set_input(x)
+        for _ in range(3):      # replays of the captured graph with host work in between
+            session.run()
+            np.testing.assert_array_equal(session.output(), got)
+
+
+def test_merged_convolutions_match_unmerged():
+    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    merged = ios.optimize(graph, 1, ios.AnalyticCostModel(launch=1.0, rate=2e7, sync=1.5), 'dp_parallel_merge',
+                          compute_weight=True)
+    assert any(' ' in node.hint_name for node in merged.nodes())
+    x = np.random.default_rng(1).standard_normal((2, 3, 299, 299)).astype(np.float32)
+    graph.sequential_schedule()
+    want = ios_oracle.run(graph, x)
+    for batch in (1, 2):    # channel slices of merged convolutions are read in place at any batch size
+        got = rt.graph_inference(merged, batch, x[:batch])
+        assert_close(got, want[:batch], f'merged graph batch {batch}')
+
+
+def test_latency_entry_points():
+    graph = ios.models.sample_network()
+    graph.sequential_schedule()
+    lat = rt.graph_latency(graph, batch_size=1, warmup=1, number=2, repeat=3)
+    assert len(lat) == 3 and all(0 < v < 1000 for v in lat)
+    lat, stages = rt.graph_latency(graph, batch_size=1, warmup=1, number=2, repeat=3, profile_stage=True)
+    table = np.array(stages).reshape(3, -1)
+    assert table.shape == (3, 5) and (table >= 0).all()
+    assert table.sum(axis=1) == pytest.approx(np.array(lat), rel=0.05, abs=0.02)
+    blk = rt.block_latency(graph.blocks[0], 1, 1, 2, 3)
+    assert len(blk) == 3 and all(v > 0 for v in blk)
+    nodes = graph.blocks[0].inner_nodes
+    one = rt.stage_latency([[nodes[0]]], 1, 1, 2, 3)
+    two = rt.stage_latency([[nodes[0], nodes[3]], [nodes[1]], [nodes[2]]], 1, 1, 2, 3)
+    assert len(one) == 3 and len(two) == 3 and all(v > 0 for v in one + two)
+    with pytest.raises(RuntimeError):
+        rt.stage_latency([[nodes[0]]], 1, 1, 2, 3, profile_stage=True)
+
+
+def test_optimize_with_measured_cost_model_on_sample_net():
+    graph = ios.models.sample_network(init_seed=0, init_scheme='he_normal')
+    optimized = ios.optimize(graph, batch_size=1, opt_type='dp_parallel', compute_weight=True, warmup=1, number=2, repeat=2)
+    names = sorted(n for stage in optimized.blocks[0].stages for group in stage for n in group)
+    assert names == ['1', '2', '3', '4', '5']
+    x = np.random.default_rng(0).standard_normal((1, 375, 15, 15))      # float64 on purpose: the glue converts
+    got = rt.graph_inference(optimized, 1, x)
+    graph.sequential_schedule()
+    assert_close(got, ios_oracle.run(graph, x.astype(np.float32)), 'optimized sample net')
+
+
+def test_errors_are_reported_not_fatal():
+    graph = ios.models.sample_network(init_seed=0)
+    with pytest.raises(RuntimeError, match='no schedule'):
+        rt._latency_call('graph_latency', [__import__('json').dumps(graph.export_config())], 1, 1, 1, 1, 1, False)
+    graph.blocks[0].stages = [[['1'], ['4']], [['2'], ['3']], [['5']]]
+    with pytest.raises(RuntimeError, match='not topological'):
+        rt.graph_latency(graph, 1, 1, 1, 1)
+    graph.blocks[0].stages = [[[str(i)] for i in range(1, 5)] * 5, [['5']]]
+    with pytest.raises(RuntimeError):
+        rt.graph_latency(graph, 1, 1, 1, 1)
+    graph.sequential_schedule()
+    x = np.zeros((1, 375, 15, 15), np.float32)
+    with pytest.raises(ValueError):
+        rt.graph_inference(graph, 2, x)
+    assert rt.graph_inference(graph, 1, x).shape == (1, 1875, 15, 15)     # still alive after the failures

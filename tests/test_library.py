@@ -1,0 +1,79 @@
+"""The shared library loads without a GPU, exports every declared symbol and plans graphs on the host."""
+import collections
+import ctypes
+import os
+import re
+
+import pytest
+
+import ios
+from ios.contrib import ios_runtime as rt
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    with open(os.path.join(ROOT, 'include', 'ios_runtime.h')) as f:
+        text = re.sub(r'/\*.*?\*/', '', f.read(), flags=re.S)
+    return sorted(set(re.findall(r'\b(\w+)\s*\(', ' '.join(line for line in text.splitlines() if not line.startswith('#')))))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = rt.get_lib()
+    names = declared_symbols()
+    assert {'graph_latency', 'block_latency', 'stage_latency', 'graph_inference', 'ios_last_error',
+            'ios_session_create'} <= set(names)
+    for name in names:
+        assert getattr(lib, name) is not None, name
+
+
+def test_missing_library_raises_file_not_found(monkeypatch):
+    monkeypatch.setattr(rt, 'libname_list', ['nowhere/libios_runtime.so'])
+    monkeypatch.delenv('IOS_RUNTIME_LIB', raising=False)
+    with pytest.raises(FileNotFoundError, match='IOS Backend library not found'):
+        rt.load_ios_library()
+
+
+def test_host_planner_fuses_concats_and_folds_relus():
+    graph = ios.models.inception_v3()
+    graph.sequential_schedule()
+    ops = rt.plan_describe(graph, 1)
+    kinds = collections.Counter(op['kind'] for op in ops)
+    # 94 convolutions, 13 window pools, 1 global pool and not a single copy: every concat is written in place
+    assert kinds == {'conv_mfma': 94, 'pool': 13, 'global_pool': 1}
+    by_node = {op['node']: op for op in ops}
+    # conv '8' writes 64 channels into the 256-channel concat buffer of block 2: at batch 1 the stride is moot,
+    # at batch 2 the batch stride must be that of the concat buffer
+    ops2 = {op['node']: op for op in rt.plan_describe(graph, 2)}
+    assert ops2['8']['out'] == [64, 35, 35] and ops2['8']['out_bstride'] == 256 * 35 * 35
+    assert by_node['1']['conv']['sh'] == 2 and by_node['1']['out'] == [32, 149, 149]
+
+    rw = ios.models.randwire_small()
+    rw.sequential_schedule()
+    kinds = collections.Counter(op['kind'] for op in rt.plan_describe(rw, 1))
+    assert kinds['conv_depthwise'] == 96 and kinds['conv_mfma'] == 99
+    folded = [op for op in rt.plan_describe(rw, 1) if op['kind'] == 'conv_depthwise' and op['conv']['pre_relu']]
+    assert len(folded) > 0      # single-input nodes fold their ReLU into the depth-wise convolution
+    nm = ios.models.nasnet_mobile()
+    nm.sequential_schedule()
+    assert len(rt.plan_describe(nm, 1)) > 400
+
+
+def test_host_planner_rejects_bad_documents():
+    graph = ios.models.sample_network()
+    with pytest.raises(RuntimeError, match='no schedule'):
+        rt.plan_describe(graph, 1)
+    graph.blocks[0].stages = [[['1'], ['4']], [['2'], ['3']], [['5']]]
+    with pytest.raises(RuntimeError, match='not topological'):
+        rt.plan_describe(graph, 1)
+    graph.blocks[0].stages = [[['1']], [['2']], [['3']], [['5']]]
+    with pytest.raises(RuntimeError, match="'5' runs before|missing"):
+        rt.plan_describe(graph, 1)
+    graph.sequential_schedule()
+    config = graph.export_config()
+    config['blocks'][0]['inner_nodes'][0]['type'] = 'softmax'
+    doc = rt.c_string(__import__('json').dumps(config))
+    assert rt.get_lib().ios_plan_describe(doc, 1, None, 0) == -1
+    assert b'unsupported type softmax' in rt.get_lib().ios_last_error()
+    with pytest.raises(RuntimeError):
+        rt.plan_describe(graph, 0)
