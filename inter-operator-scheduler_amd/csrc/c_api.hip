@@ -16,14 +16,7 @@ std::string g_last_error;
 
 ios::LaunchChooser device_chooser() {
     ios::DeviceContext &ctx = ios::DeviceContext::get();
-    const int cus = ctx.num_cus();
-    const int variant = ctx.forced_variant(), split = ctx.forced_split_k();
-    return [cus, variant, split](const ios::ConvProblem &p) {
-        ios::ConvLaunch launch = ios::conv_pick_launch(p, cus);
-        if (variant >= 0) launch.variant = variant;
-        if (split > 0) launch.split_k = split;
-        return launch;
-    };
+    return [&ctx](const ios::ConvProblem &p) { return ctx.choose_launch(p); };
 }
 
 template <typename F>

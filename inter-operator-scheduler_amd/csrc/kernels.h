@@ -49,27 +49,25 @@ const ConvVariant &conv_variant(int index);
 
 struct ConvLaunch {
     int variant = 0;
-    int split_k = 1;  // number of grid slices along K; > 1 needs workspace and counters
+    int split_k = 1;  // number of grid slices along K; > 1 needs workspace
 };
 
-// Bytes of workspace / number of tile counters a launch configuration needs.
+// Floats of workspace a launch configuration needs (split_k partial outputs).
 size_t conv_workspace_floats(const ConvProblem &p, const ConvLaunch &l);
-size_t conv_num_counters(const ConvProblem &p, const ConvLaunch &l);
+// The matrix path indexes k with 16 bits and pixels / input offsets with 31 bits.
+bool conv_matrix_path_supported(const ConvProblem &p);
 
 // Default configuration from a closed-form occupancy model (num_cus = compute units of the device).
 ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus);
 
-// Filter packing: w[OC][ICg][KH][KW] -> packed[g][K][OCgP] (K = ICg*KH*KW, zero padded rows), and the
-// per-k gather table {c*H*W + kh*W + kw, kh << 16 | kw} used by the implicit-GEMM input loader.
+// Filter packing: w[OC][ICg][KH][KW] -> packed[g][K][OCgP] (K = ICg*KH*KW, rows zero padded to OCgP).
 size_t conv_packed_floats(const ConvProblem &p);
 void launch_pack_filters(const ConvProblem &p, const float *w, float *packed, hipStream_t stream);
-void launch_build_ktab(const ConvProblem &p, int2 *ktab, hipStream_t stream);
 
-// y = act(conv(x, w) + bias).  `packed` and `ktab` come from the two functions above.  `workspace` holds
-// split_k partial tiles, `counters` must be zero before the first launch and is left zero afterwards.
+// y = act(conv(x, w) + bias).  `packed` comes from launch_pack_filters.  `workspace` holds the split_k
+// partial outputs (conv_workspace_floats); with split_k > 1 a second kernel reduces them on the same stream.
 void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
-                      const int2 *ktab, const float *bias, const TensorView &y, float *workspace,
-                      unsigned *counters, hipStream_t stream);
+                      const float *bias, const TensorView &y, float *workspace, hipStream_t stream);
 
 // Depth-wise convolution (groups == IC == OC), filters in their original [C][1][KH][KW] layout.
 void launch_dwconv(const ConvProblem &p, const TensorView &x, const float *w, const float *bias,

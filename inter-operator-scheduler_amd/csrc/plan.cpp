@@ -479,13 +479,12 @@ private:
         OpKind kind;
         if (p.is_depthwise()) {
             kind = OpKind::ConvDepthwise;
-        } else if (p.groups > 1 && (p.ICg() < 4 || p.OCg() < 8)) {
+        } else if ((p.groups > 1 && (p.ICg() < 4 || p.OCg() < 8)) || !conv_matrix_path_supported(p)) {
             kind = OpKind::ConvDirect;
         } else {
             kind = OpKind::ConvMfma;
             conv.matrix_path = true;
             conv.packed_off = reserve(conv_packed_floats(p));
-            conv.ktab_off = reserve((size_t)p.K() * 2);
             conv.launch = chooser_(p);
         }
         if (plan_.conv_index.count(n.name)) throw std::runtime_error("duplicate convolution name '" + n.name + "'");
@@ -592,11 +591,7 @@ private:
         for (PlanConv &conv : plan_.convs) {
             if (!conv.matrix_path) continue;
             conv.ws_floats = conv_workspace_floats(conv.problem, conv.launch);
-            conv.num_counters = conv_num_counters(conv.problem, conv.launch);
-            if (conv.ws_floats > 0) {
-                conv.ws_off = reserve(conv.ws_floats);
-                conv.counter_off = reserve(conv.num_counters);
-            }
+            if (conv.ws_floats > 0) conv.ws_off = reserve(conv.ws_floats);
         }
     }
 

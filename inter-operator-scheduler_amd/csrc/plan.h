@@ -1,8 +1,8 @@
 // Execution plan: the flat list of device operations, tensor views and the memory layout that a graph,
 // block or stage document compiles to.  Planning is pure host code; nothing here touches the device.
 //
-// Memory model: one arena of 4-byte words.  Every operator output, temporary, filter, bias, gather table,
-// split-K workspace and tile counter is a region of it at a 256-byte aligned offset.  Tensor views are
+// Memory model: one arena of 4-byte words.  Every operator output, temporary, filter, bias and split-K
+// workspace is a region of it at a 256-byte aligned offset.  Tensor views are
 // (offset, C, H, W, batch stride); a channel slice or a window of a concat buffer is again a view, so
 //   * an identity with one input value is an alias (no memory, no work),
 //   * a producer whose whole output is one term of a concat writes directly into the concat buffer,
@@ -43,9 +43,8 @@ struct PlanConv {
     std::string name;
     ConvProblem problem;
     size_t weight_off = 0, bias_off = 0;       // original layouts
-    size_t packed_off = 0, ktab_off = 0;       // matrix path only
-    size_t ws_off = 0, counter_off = 0;        // split-K only
-    size_t ws_floats = 0, num_counters = 0;
+    size_t packed_off = 0;                     // matrix path only
+    size_t ws_off = 0, ws_floats = 0;          // split-K only
     ConvLaunch launch;
     bool matrix_path = false;
 };

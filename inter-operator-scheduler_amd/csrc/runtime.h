@@ -39,11 +39,20 @@ public:
     int forced_split_k() const { return forced_split_k_; }
     std::string info_json() const;
 
-    // measured kernel configurations, keyed by problem signature
+    // Kernel configuration for a matrix-path convolution: the measured best when autotuning is on (cached
+    // per problem signature for the life of the process, and in the file named by IOS_TUNE_CACHE when set),
+    // else the closed-form model; the testing overrides win over both.
+    ConvLaunch choose_launch(const ConvProblem &p);
     std::map<std::string, ConvLaunch> tuned;
 
 private:
     DeviceContext();
+    ConvLaunch tune_conv(const ConvProblem &p);
+    float *tuning_buffer(int which, size_t floats);
+    void load_tune_cache();
+    float *tune_buf_[4] = {nullptr, nullptr, nullptr, nullptr};
+    size_t tune_floats_[4] = {0, 0, 0, 0};
+    std::string tune_cache_path_;
     int num_cus_ = 0;
     std::string name_, arch_;
     hipStream_t streams_[kMaxGroups];

@@ -46,6 +46,132 @@ DeviceContext::DeviceContext() {
     if (mode != nullptr) set_option("executor", mode);
     const char *tune = getenv("IOS_AUTOTUNE");
     if (tune != nullptr) set_option("autotune", tune);
+    const char *cache = getenv("IOS_TUNE_CACHE");
+    if (cache != nullptr && cache[0] != '\0') {
+        tune_cache_path_ = cache;
+        load_tune_cache();
+    }
+}
+
+// ---- kernel configuration choice ----------------------------------------------------------------------------------
+static std::string conv_signature(const ConvProblem &p) {
+    std::ostringstream os;
+    os << p.B << ' ' << p.IC << ' ' << p.H << ' ' << p.W << ' ' << p.OC << ' ' << p.KH << ' ' << p.KW << ' ' << p.sh << ' ' << p.sw
+       << ' ' << p.ph << ' ' << p.pw << ' ' << p.groups;
+    return os.str();
+}
+
+void DeviceContext::load_tune_cache() {
+    FILE *f = fopen(tune_cache_path_.c_str(), "r");
+    if (f == nullptr) return;
+    int v[12], variant, split;
+    char name[128];
+    // line: 12 problem integers, variant name, split_k
+    while (fscanf(f, "%d %d %d %d %d %d %d %d %d %d %d %d %127s %d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5], &v[6], &v[7], &v[8],
+                  &v[9], &v[10], &v[11], name, &split) == 14) {
+        variant = -1;
+        for (int i = 0; i < conv_num_variants(); i++)
+            if (strcmp(conv_variant(i).name, name) == 0) variant = i;
+        if (variant < 0 || split < 1) continue;
+        std::ostringstream os;
+        for (int i = 0; i < 12; i++) os << (i ? " " : "") << v[i];
+        ConvLaunch l;
+        l.variant = variant;
+        l.split_k = split;
+        tuned[os.str()] = l;
+    }
+    fclose(f);
+}
+
+float *DeviceContext::tuning_buffer(int which, size_t floats) {
+    if (floats > tune_floats_[which]) {
+        IOS_HIP(hipDeviceSynchronize());
+        if (tune_buf_[which] != nullptr) IOS_HIP(hipFree(tune_buf_[which]));
+        tune_buf_[which] = nullptr;
+        tune_floats_[which] = 0;
+        const size_t want = floats + floats / 2 + 1024;
+        IOS_HIP(hipMalloc(reinterpret_cast<void **>(&tune_buf_[which]), want * sizeof(float)));
+        tune_floats_[which] = want;
+        launch_fill_pattern(tune_buf_[which], want, 0x51f15e + which, streams_[0]);
+        IOS_HIP(hipStreamSynchronize(streams_[0]));
+    }
+    return tune_buf_[which];
+}
+
+ConvLaunch DeviceContext::tune_conv(const ConvProblem &p) {
+    // Like the reference's exhaustive algorithm search on first sight of a shape: run every kernel
+    // configuration on scratch tensors of the real shape and keep the fastest.
+    static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
+    const size_t kMaxWorkspace = size_t(96) << 20;   // floats
+    TensorView x, y;
+    x.C = p.IC; x.H = p.H; x.W = p.W; x.bstride = (long long)p.IC * p.H * p.W;
+    y.C = p.OC; y.H = p.OH; y.W = p.OW; y.bstride = (long long)p.OC * p.OH * p.OW;
+    x.ptr = tuning_buffer(0, (size_t)p.B * x.bstride);
+    y.ptr = tuning_buffer(1, (size_t)p.B * y.bstride);
+    float *packed = tuning_buffer(2, conv_packed_floats(p) + p.OC);
+    float *bias = packed + conv_packed_floats(p);
+    hipStream_t stream = streams_[0];
+    hipEvent_t start, stop;
+    IOS_HIP(hipEventCreate(&start));
+    IOS_HIP(hipEventCreate(&stop));
+    ConvLaunch best = conv_pick_launch(p, num_cus_);
+    float best_ms = 1e30f;
+    for (int v = 0; v < conv_num_variants(); v++) {
+        const ConvVariant &cv = conv_variant(v);
+        // tiles more than twice as tall / wide as the problem only waste lanes
+        if (cv.BM >= 2 * p.OCg() + 32 || cv.BN >= 2 * p.Npix() + 32) continue;
+        int last_effective = -1;
+        for (int split : kSplits) {
+            ConvLaunch l;
+            l.variant = v;
+            l.split_k = split;
+            const size_t ws = conv_workspace_floats(p, l);
+            const int effective = ws == 0 ? 1 : (int)(ws / ((size_t)p.OC * p.Npix()));
+            if (effective == last_effective) continue;   // asks for more slices than there are K tiles
+            last_effective = effective;
+            if (ws > kMaxWorkspace) break;
+            float *workspace = ws ? tuning_buffer(3, ws) : nullptr;
+            launch_conv_mfma(p, l, x, packed, bias, y, workspace, stream);   // warm-up
+            IOS_HIP(hipEventRecord(start, stream));
+            const int reps = 4;
+            for (int r = 0; r < reps; r++) launch_conv_mfma(p, l, x, packed, bias, y, workspace, stream);
+            IOS_HIP(hipEventRecord(stop, stream));
+            IOS_HIP(hipEventSynchronize(stop));
+            float ms = 0.f;
+            IOS_HIP(hipEventElapsedTime(&ms, start, stop));
+            ms /= reps;
+            if (ms < best_ms) {
+                best_ms = ms;
+                best = l;
+            }
+            if (ms > 3.f * best_ms) break;   // more slices only add reduction work from here on
+        }
+    }
+    IOS_HIP(hipEventDestroy(start));
+    IOS_HIP(hipEventDestroy(stop));
+    if (!tune_cache_path_.empty()) {
+        FILE *f = fopen(tune_cache_path_.c_str(), "a");
+        if (f != nullptr) {
+            fprintf(f, "%s %s %d\n", conv_signature(p).c_str(), conv_variant(best.variant).name, best.split_k);
+            fclose(f);
+        }
+    }
+    return best;
+}
+
+ConvLaunch DeviceContext::choose_launch(const ConvProblem &p) {
+    ConvLaunch launch;
+    if (autotune_) {
+        const std::string key = conv_signature(p);
+        auto it = tuned.find(key);
+        if (it == tuned.end()) it = tuned.emplace(key, tune_conv(p)).first;
+        launch = it->second;
+    } else {
+        launch = conv_pick_launch(p, num_cus_);
+    }
+    if (forced_variant_ >= 0) launch.variant = forced_variant_;
+    if (forced_split_k_ > 0) launch.split_k = forced_split_k_;
+    return launch;
 }
 
 float *DeviceContext::shared_arena(size_t floats) {
@@ -140,8 +266,6 @@ void Session::setup() {
     if (owns_memory_) launch_fill_pattern(base_, plan_.arena_floats, 0x2468aceu, main);
     for (const PlanConv &conv : plan_.convs) {
         if (!conv.matrix_path) continue;
-        launch_build_ktab(conv.problem, reinterpret_cast<int2 *>(base_ + conv.ktab_off), main);
-        if (conv.ws_floats > 0) launch_fill_u32(reinterpret_cast<unsigned *>(base_ + conv.counter_off), conv.num_counters, 0u, main);
         // the probes never upload filters: pack whatever the filter region holds so that the matrix
         // path reads initialised memory
         launch_pack_filters(conv.problem, base_ + conv.weight_off, base_ + conv.packed_off, main);
@@ -215,9 +339,8 @@ void Session::launch_op(const PlanOp &op, hipStream_t stream) {
     switch (op.kind) {
         case OpKind::ConvMfma: {
             const PlanConv &c = plan_.convs[op.conv];
-            launch_conv_mfma(c.problem, c.launch, tv(op.in), base_ + c.packed_off, reinterpret_cast<const int2 *>(base_ + c.ktab_off),
-                             base_ + c.bias_off, tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr,
-                             c.ws_floats ? reinterpret_cast<unsigned *>(base_ + c.counter_off) : nullptr, stream);
+            launch_conv_mfma(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off, tv(op.out),
+                             c.ws_floats ? base_ + c.ws_off : nullptr, stream);
             break;
         }
         case OpKind::ConvDepthwise: {

@@ -210,23 +210,29 @@ class _PartSearch:
                 if count_bits(group) <= self.max_group_size:
                     window.append((u, group))
             windows.append(window)
-        # mixed-radix enumeration, chain 0 is the fastest digit, the last digit value means "unused"
-        digit_ranges = [range(len(w) + 1) for w in reversed(windows)]
-        for digits in itertools.product(*digit_ranges):
-            used = 0
-            groups = []
-            for window, digit in zip(windows, reversed(digits)):
-                if digit == len(window):
-                    continue
-                group = window[digit][1]
-                if used & group:
-                    groups = None
-                    break
-                used |= group
-                groups.append(group)
-            if not groups or len(groups) > self.max_num_groups:
-                continue
-            yield [bits_of(group) for group in groups]
+        # Enumeration order: mixed radix over the chains with chain 0 as the fastest digit and "unused" as
+        # the last value of every digit.  The recursion fixes the slowest digit first and abandons a prefix
+        # as soon as it has too many or overlapping groups, which skips whole sub-ranges without changing
+        # the order of the survivors.
+        limit = self.max_num_groups
+        chosen: List[int] = []
+
+        def walk(chain_index: int, used: int):
+            if chain_index < 0:
+                if chosen:
+                    # groups are reported in chain order
+                    yield [bits_of(group) for group in reversed(chosen)]
+                return
+            if len(chosen) < limit:
+                for _, group in windows[chain_index]:
+                    if used & group:
+                        continue
+                    chosen.append(group)
+                    yield from walk(chain_index - 1, used | group)
+                    chosen.pop()
+            yield from walk(chain_index - 1, used)
+
+        yield from walk(len(windows) - 1, 0)
 
     # -- stage cost -------------------------------------------------------------------------------
     def _measure(self, stage_nodes: List[List[Node]]) -> float:

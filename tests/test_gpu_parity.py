@@ -84,7 +84,7 @@ def test_conv_matches_oracle(case):
     assert_close(got, want, f'conv {case}')
 
 
-@pytest.mark.parametrize('variant', range(8))
+@pytest.mark.parametrize('variant', range(10))
 @pytest.mark.parametrize('split_k', [1, 3])
 def test_every_conv_kernel_variant(variant, split_k):
     rt.set_option('conv_variant', variant)
@@ -99,7 +99,7 @@ def test_every_conv_kernel_variant(variant, split_k):
         np.testing.assert_array_equal(got, got2)      # split-K reduction order is fixed
 
 
-def test_split_k_counters_are_reusable_in_a_session():
+def test_split_k_is_repeatable_in_a_session():
     rt.set_option('conv_split_k', 4)
     graph = single_op_graph((64, 12, 12), lambda b, v: ios.conv2d(b, [[v]], 40, (3, 3), (1, 1), (1, 1), 1, 'relu', is_exit=True))
     x = np.random.default_rng(3).standard_normal((2, 64, 12, 12)).astype(np.float32)
@@ -213,9 +213,12 @@ def test_network_matches_oracle_and_schedules_agree_bitwise(name, make, batch):
     greedy = rt.graph_inference(graph, batch, x)
     np.testing.assert_array_equal(greedy, got)
 
+    big = name.startswith(('randwire', 'nasnet'))
+    if big:     # keep the pure-Python search short: small consecutive parts instead of whole cells
+        for block in graph.blocks:
+            block.parts = None
     optimized = ios.optimize(graph, batch, ios.AnalyticCostModel(), 'dp_parallel', max_group_size=2,
-                             max_num_groups=4 if name.startswith(('randwire', 'nasnet')) else 8,
-                             max_part_size=12 if name.startswith('randwire') else 100, compute_weight=True)
+                             max_num_groups=4 if big else 8, max_part_size=10 if big else 100, compute_weight=True)
     assert any(len(stage) > 1 for block in optimized.blocks for stage in block.stages)
     parallel = rt.graph_inference(optimized, batch, x)
     np.testing.assert_array_equal(parallel, got)
