@@ -39,7 +39,10 @@ def main():
     parser.add_argument('--steps', type=int, default=300)
     parser.add_argument('--warmup', type=int, default=30)
     parser.add_argument('--batch', type=int, default=1)
-    parser.add_argument('--executor', default=os.environ.get('IOS_BENCH_EXECUTOR', 'graph'), choices=['streams', 'graph'])
+    parser.add_argument('--executor', default=os.environ.get('IOS_BENCH_EXECUTOR', 'fused_graph'),
+                        choices=['streams', 'graph', 'fused', 'fused_graph'])
+    parser.add_argument('--search-executor', default='fused', choices=['streams', 'fused'],
+                        help='executor under which the schedule search measures candidate stages')
     parser.add_argument('--sweep', action='store_true', help='also time batch 16 and 64 with the same schedule')
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     args = parser.parse_args()
@@ -57,7 +60,8 @@ def main():
     x = np.random.default_rng(1).standard_normal((batch, 3, 299, 299)).astype(np.float32)
 
     # schedule search with measured stage latencies (not part of the timed steps)
-    rt.set_option('executor', 'streams')
+    rt.set_option('autotune', 1)        # measure kernel configurations on first sight of a shape
+    rt.set_option('executor', args.search_executor)
     t0 = time.time()
     optimized = ios.optimize(graph, batch_size=batch, opt_type='dp_parallel', compute_weight=True,
                              warmup=2, number=6, repeat=3)

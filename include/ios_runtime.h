@@ -57,7 +57,8 @@ int graph_inference(const char *graph_json, int batch_size, float *input, int nu
 /* Message of the most recent failure (valid until the next failing call). */
 const char *ios_last_error(void);
 
-/* Options: "executor" = "streams" | "graph" (hipGraph replay); "autotune" = "0" | "1" (measure convolution
+/* Options: "executor" = "streams" (one HIP stream per group, event fork/join) | "graph" (the same, captured into a
+ * hipGraph and replayed) | "fused" (the groups of a stage share one kernel launch per level) | "fused_graph"; "autotune" = "0" | "1" (measure convolution
  * kernel configurations on first use, like the reference's cudnnFind-based selection,
  * src/ios/ios_runtime.cu:150-205); "clear_tuning" = anything;
  * "conv_variant" = index or -1 and "conv_split_k" = count or 0 force one convolution kernel configuration (testing). */

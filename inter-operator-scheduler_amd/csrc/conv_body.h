@@ -1,0 +1,502 @@
+// Implicit-GEMM convolution on the CDNA4 fp32 matrix cores.
+//
+// GEMM view per group:  Y[m][n] = sum_k Wp[k][m] * X_im2col[k][n]
+//   m = output channel inside the group (OCg), n = flattened (image, oh, ow) pixel, k = (c, kh, kw).
+// The filter matrix is pre-packed k-major (launch_pack_filters) so that a block's BK x BM slice is read
+// with 16-byte loads along m.  The BK x BN input slice is gathered straight from the NCHW input view:
+// consecutive lanes take consecutive pixels, k is decomposed into (c, kh, kw) with multiply-high
+// divisions by launch constants, and padding is resolved by predication.  Global loads run PD tiles
+// ahead of the math in registers (the loop is latency bound at batch 1, where a block sees only a few
+// K tiles), tiles are staged in LDS (double buffered, one barrier per K tile) and consumed by
+// v_mfma_f32_32x32x2_f32 / v_mfma_f32_16x16x4_f32: lane l supplies A[k = l / MT][m = l % MT] and
+// B[k = l / MT][n = l % MT].
+//
+// Parallelism for small problems comes from three places: WK wavefronts of a block split each K tile
+// and add their accumulators through LDS at the end; split_k grid slices along K write partial tiles
+// to a workspace that a second small kernel sums in slice order (fixed order, so results do not depend
+// on scheduling; no device-scope fences inside the main kernel); everything else is M x N tiling.
+// The epilogue adds the bias, applies the activation and stores through the output view, i.e. directly
+// into the consumer's channel window when the output lives inside a concat buffer.
+// Device-side bodies of the convolution kernels; included by the translation units that instantiate them
+// (the stand-alone kernels and the fused stage kernel).
+#pragma once
+
+#include "kernels.h"
+
+namespace ios {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+struct ConvKernelArgs {
+    const float *x;
+    const float *wp;
+    const float *bias;
+    float *y;
+    float *ws;
+    int H, W, OH, OW, sh, sw, ph, pw;
+    int KW, KHKW;
+    unsigned magic_khkw, magic_kw;   // floor(2^32 / d) + 1; exact quotients for k < 2^16
+    int ICg, OCg, OCgP, K, HW, OHW, groups;
+    long long x_bs, y_bs;
+    int Npix;
+    int act, pre_relu;
+    int split_k, k_chunk;
+    int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ float apply_act(float v, int act) {
+    switch (act) {
+        case ACT_RELU: return fmaxf(v, 0.0f);
+        case ACT_TANH: return tanhf(v);
+        case ACT_SIGMOID: return 1.0f / (1.0f + __expf(-v));
+        default: return v;
+    }
+}
+
+template <int MT>
+struct Mfma;
+
+template <>
+struct Mfma<32> {
+    static constexpr int KSTEP = 2;
+    static constexpr int ACC = 16;
+    typedef floatx16 acc_t;
+    __device__ static __forceinline__ acc_t run(float a, float b, acc_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+    }
+    // row of accumulator element v held by `lane` inside the 32 x 32 tile; the column is lane % 32
+    __device__ static __forceinline__ int row(int v, int lane) { return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3); }
+};
+
+template <>
+struct Mfma<16> {
+    static constexpr int KSTEP = 4;
+    static constexpr int ACC = 4;
+    typedef floatx4 acc_t;
+    __device__ static __forceinline__ acc_t run(float a, float b, acc_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ int row(int v, int lane) { return 4 * (lane >> 4) + v; }
+};
+
+template <int BM, int BN, int BK, int WM, int WN, int WK, int MT, int PD, bool POINTWISE>
+struct ConvTiled {
+    using M = Mfma<MT>;
+    static constexpr int T = 64 * WM * WN * WK;
+    static constexpr int THREADS = T;
+    static constexpr int PAD = MT == 16 ? 16 : 4;   // MT 16 reads four rows per instruction: rows must not share banks
+    static constexpr int LDA = BM + PAD, LDB = BN + PAD;
+    static constexpr int TILE_FLOATS = 2 * BK * (LDA + LDB);
+    static constexpr int RED_FLOATS = (WK - 1) * BM * BN;
+    static constexpr int SMEM_FLOATS = TILE_FLOATS > RED_FLOATS ? TILE_FLOATS : RED_FLOATS;
+
+    // one block: output tile `tile` of group `g`, K slice `z`; smem holds SMEM_FLOATS floats, 16-byte aligned
+    __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *smem, int tile, int g, int z) {
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TM = WTM / MT, TN = WTN / MT;
+    constexpr int KSLICE = BK / WK;
+    constexpr int A_VEC_PER_ROW = BM / 4;
+    constexpr int A_SLOTS = BK * A_VEC_PER_ROW;
+    constexpr int A_ITERS = (A_SLOTS + T - 1) / T;
+    constexpr int B_ROWS_PER_PASS = T / BN;
+    constexpr int B_ITERS = BK / B_ROWS_PER_PASS;
+    static_assert(WTM % MT == 0 && WTN % MT == 0, "wave tile must be a multiple of the MFMA tile");
+    static_assert(KSLICE % M::KSTEP == 0, "K slice per wavefront must be a multiple of the MFMA depth");
+    static_assert(T % BN == 0 && BK % B_ROWS_PER_PASS == 0, "input loader shape");
+    float *As = smem;                  // [2][BK][LDA]
+    float *Bs = smem + 2 * BK * LDA;   // [2][BK][LDB]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wn = wave % WN;
+    const int wm = (wave / WN) % WM;
+    const int wk = wave / (WN * WM);
+
+    const int tm = tile % a.tiles_m;
+    const int tn = tile / a.tiles_m;
+    const int m0 = tm * BM;
+    const int n0 = tn * BN;
+    const int k_begin = z * a.k_chunk;
+    const int k_end = min(a.K, k_begin + a.k_chunk);
+    const int nkt = (k_end - k_begin + BK - 1) / BK;
+
+    // ---- per-thread loader state ---------------------------------------------------------------------
+    const int bn_l = tid % BN;
+    const int bk_l = tid / BN;
+    const int n = n0 + bn_l;
+    const bool n_ok = n < a.Npix;
+    int ih0 = 0, iw0 = 0;
+    long long x_off = 0;
+    {
+        const int nn = n_ok ? n : 0;
+        const int b = nn / a.OHW;
+        const int r = nn - b * a.OHW;
+        const int oh = r / a.OW;
+        const int ow = r - oh * a.OW;
+        ih0 = oh * a.sh - a.ph;
+        iw0 = ow * a.sw - a.pw;
+        x_off = (long long)b * a.x_bs + (long long)g * a.ICg * a.HW + (long long)ih0 * a.W + iw0;
+    }
+    const float *xg = a.x + x_off;
+    const float *wg = a.wp + (size_t)g * a.K * a.OCgP;
+
+    floatx4 a_reg[PD][A_ITERS];
+    float b_reg[PD][B_ITERS];
+
+    auto load_tile = [&](int kt, floatx4(&ar)[A_ITERS], float(&br)[B_ITERS]) {
+        const int k0 = k_begin + kt * BK;
+#pragma unroll
+        for (int i = 0; i < A_ITERS; i++) {
+            const int slot = tid + i * T;
+            const int row = slot / A_VEC_PER_ROW;
+            const int c4 = slot % A_VEC_PER_ROW;
+            const int k = k0 + row;
+            const int m = m0 + c4 * 4;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if ((A_SLOTS % T == 0 || slot < A_SLOTS) && k < k_end && m < a.OCgP)
+                v = *reinterpret_cast<const floatx4 *>(wg + (size_t)k * a.OCgP + m);
+            ar[i] = v;
+        }
+#pragma unroll
+        for (int i = 0; i < B_ITERS; i++) {
+            const int k = k0 + bk_l + i * B_ROWS_PER_PASS;
+            float v = 0.f;
+            if (k < k_end && n_ok) {
+                if (POINTWISE) {
+                    v = xg[(long long)k * a.HW];
+                } else {
+                    const int c = a.KHKW == 1 ? k : (int)__umulhi((unsigned)k, a.magic_khkw);
+                    const int rem = k - c * a.KHKW;
+                    const int kh = a.KW == 1 ? rem : (int)__umulhi((unsigned)rem, a.magic_kw);
+                    const int kw = rem - kh * a.KW;
+                    if ((unsigned)(ih0 + kh) < (unsigned)a.H && (unsigned)(iw0 + kw) < (unsigned)a.W)
+                        v = xg[(long long)c * a.HW + kh * a.W + kw];
+                }
+            }
+            br[i] = v;
+        }
+    };
+
+    auto store_tile = [&](int buf, const floatx4(&ar)[A_ITERS], const float(&br)[B_ITERS]) {
+        float *Ab = As + buf * BK * LDA;
+        float *Bb = Bs + buf * BK * LDB;
+#pragma unroll
+        for (int i = 0; i < A_ITERS; i++) {
+            const int slot = tid + i * T;
+            if (A_SLOTS % T == 0 || slot < A_SLOTS) {
+                const int row = slot / A_VEC_PER_ROW;
+                const int c4 = slot % A_VEC_PER_ROW;
+                *reinterpret_cast<floatx4 *>(Ab + row * LDA + c4 * 4) = ar[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < B_ITERS; i++) {
+            float v = br[i];
+            if (a.pre_relu) v = fmaxf(v, 0.f);
+            Bb[(bk_l + i * B_ROWS_PER_PASS) * LDB + bn_l] = v;
+        }
+    };
+
+    typename M::acc_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < M::ACC; v++) acc[i][j][v] = 0.f;
+
+    // ---- main loop: global -> registers (PD tiles ahead) -> LDS (double buffered) -> MFMA -----------------
+    // Register stage s holds tile kt with kt % PD == s.  In iteration kt the stage of tile kt is free (the
+    // tile already sits in LDS buffer kt & 1), so it is refilled with tile kt + PD; the stage of tile kt + 1,
+    // requested PD - 1 iterations ago, is written to the other LDS buffer after the math.
+#pragma unroll
+    for (int s = 0; s < PD; s++)
+        if (s < nkt) load_tile(s, a_reg[s], b_reg[s]);
+    if (nkt > 0) store_tile(0, a_reg[0], b_reg[0]);
+    __syncthreads();
+    const int lk = lane / MT;   // k offset of this lane inside an MFMA step
+    const int lc = lane % MT;   // row (A) / column (B) of this lane inside an MFMA tile
+    for (int kt0 = 0; kt0 < nkt; kt0 += PD) {
+#pragma unroll
+        for (int s = 0; s < PD; s++) {
+            const int kt = kt0 + s;
+            if (kt >= nkt) break;
+            const int buf = kt & 1;
+            if (kt + PD < nkt) load_tile(kt + PD, a_reg[s], b_reg[s]);
+            const float *Ab = As + buf * BK * LDA + (wk * KSLICE + lk) * LDA + wm * WTM + lc;
+            const float *Bb = Bs + buf * BK * LDB + (wk * KSLICE + lk) * LDB + wn * WTN + lc;
+#pragma unroll
+            for (int kk = 0; kk < KSLICE; kk += M::KSTEP) {
+                float av[TM], bv[TN];
+#pragma unroll
+                for (int i = 0; i < TM; i++) av[i] = Ab[kk * LDA + i * MT];
+#pragma unroll
+                for (int j = 0; j < TN; j++) bv[j] = Bb[kk * LDB + j * MT];
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) acc[i][j] = M::run(av[i], bv[j], acc[i][j]);
+            }
+            if (kt + 1 < nkt) store_tile(buf ^ 1, a_reg[(s + 1) % PD], b_reg[(s + 1) % PD]);
+            __syncthreads();
+        }
+    }
+
+    // ---- fold the WK wavefronts that worked on the same output tile -------------------------------------------
+    if (WK > 1) {
+        constexpr int PER_WAVE = TM * TN * M::ACC;        // accumulator floats per lane
+        constexpr int MN_WAVES = WM * WN;
+        float *red = smem;                                // [(WK-1)][PER_WAVE][MN_WAVES * 64]
+        const int slot = (wm * WN + wn) * 64 + lane;
+        if (wk > 0) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int v = 0; v < M::ACC; v++)
+                        red[((size_t)(wk - 1) * PER_WAVE + (i * TN + j) * M::ACC + v) * (MN_WAVES * 64) + slot] =
+                            acc[i][j][v];
+        }
+        __syncthreads();
+        if (wk == 0) {
+            for (int s = 0; s < WK - 1; s++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+#pragma unroll
+                        for (int v = 0; v < M::ACC; v++)
+                            acc[i][j][v] += red[((size_t)s * PER_WAVE + (i * TN + j) * M::ACC + v) * (MN_WAVES * 64) + slot];
+        }
+    }
+
+    // ---- epilogue -------------------------------------------------------------------------------------------
+    if (a.split_k == 1) {
+        if (wk == 0) {
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const int nn = n0 + wn * WTN + j * MT + lc;
+                if (nn >= a.Npix) continue;
+                const int b = nn / a.OHW;
+                const int r = nn - b * a.OHW;
+                float *yb = a.y + (long long)b * a.y_bs + (long long)g * a.OCg * a.OHW + r;
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int v = 0; v < M::ACC; v++) {
+                        const int m = m0 + wm * WTM + i * MT + M::row(v, lane);
+                        if (m < a.OCg) yb[(long long)m * a.OHW] = apply_act(acc[i][j][v] + a.bias[g * a.OCg + m], a.act);
+                    }
+            }
+        }
+        return;
+    }
+
+    // split-K: store this slice's partial tile; splitk_reduce_kernel adds the slices, bias and activation
+    float *wsz = a.ws + ((size_t)z * a.groups + g) * a.OCg * (size_t)a.Npix;
+    if (wk == 0) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int nn = n0 + wn * WTN + j * MT + lc;
+            if (nn >= a.Npix) continue;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int v = 0; v < M::ACC; v++) {
+                    const int m = m0 + wm * WTM + i * MT + M::row(v, lane);
+                    if (m < a.OCg) wsz[(size_t)m * a.Npix + nn] = acc[i][j][v];
+                }
+        }
+    }
+    }   // run
+};
+
+// y[b][oc][r] = act(bias[oc] + sum_s ws[s][oc][n]),  n = b * OHW + r; slices are added in index order
+struct ReduceArgs {
+    const float *ws;
+    const float *bias;
+    float *y;
+    int slices, OC, Npix, OHW, act;
+    long long slice_floats, y_bs;
+};
+
+__device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int block, int num_blocks) {
+    const long long total = (long long)a.OC * a.Npix;
+    for (long long i = block * (long long)blockDim.x + threadIdx.x; i < total; i += (long long)num_blocks * blockDim.x) {
+        const int oc = (int)(i / a.Npix);
+        const int n = (int)(i - (long long)oc * a.Npix);
+        float sum = 0.f;
+        for (int s = 0; s < a.slices; s++) sum += a.ws[s * a.slice_floats + i];
+        const int b = n / a.OHW;
+        const int r = n - b * a.OHW;
+        a.y[b * a.y_bs + (long long)oc * a.OHW + r] = apply_act(sum + a.bias[oc], a.act);
+    }
+}
+
+
+// ---- wave-split variant: no LDS staging, K divided among the wavefronts of a block ---------------------------------------
+// For batch-1 layers (tens to hundreds of pixels, K in the thousands) the LDS-tiled kernel is bound by the chain
+// load -> LDS -> barrier per K tile, and slicing K over blocks costs a second kernel.  Here every wavefront of a
+// block owns a contiguous K range of the same BM x BN output tile and feeds the MFMA straight from global memory in
+// the instruction's operand layout (lane l: A[k = l / MT][m = l % MT], B[k = l / MT][n = l % MT]); there is no barrier
+// inside the K loop, two register batches of U k-steps keep dozens of loads in flight per lane, and the NW partial
+// tiles meet once in LDS, where the wavefronts share the bias + activation + store work.  The sum order is fixed
+// (k ascending inside a wavefront, wavefronts ascending), so results are reproducible.
+template <int MT, int TM, int TN, int NW, int U, bool POINTWISE>
+struct ConvWsplit {
+    using M = Mfma<MT>;
+    static constexpr int BM = TM * MT, BN = TN * MT;
+    static constexpr int E = TM * TN * M::ACC;
+    static constexpr int THREADS = 64 * NW;
+    static constexpr int SMEM_FLOATS = NW * E * 64;
+
+    __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *red, int tile, int g, int /*z*/) {
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int lk = lane / MT;
+    const int lc = lane % MT;
+    const int tm = tile % a.tiles_m;
+    const int tn = tile / a.tiles_m;
+    const int m0 = tm * BM;
+    const int n0 = tn * BN;
+
+    const int steps_total = (a.K + M::KSTEP - 1) / M::KSTEP;
+    const int steps_per_wave = (steps_total + NW - 1) / NW;
+    const int s_begin = wave * steps_per_wave;
+    const int s_end = min(steps_total, s_begin + steps_per_wave);
+
+    int ih0[TN], iw0[TN];
+    const float *xg[TN];
+    bool n_ok[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int n = n0 + j * MT + lc;
+        n_ok[j] = n < a.Npix;
+        const int nn = n_ok[j] ? n : 0;
+        const int b = nn / a.OHW;
+        const int r = nn - b * a.OHW;
+        const int oh = r / a.OW;
+        const int ow = r - oh * a.OW;
+        ih0[j] = oh * a.sh - a.ph;
+        iw0[j] = ow * a.sw - a.pw;
+        xg[j] = a.x + (long long)b * a.x_bs + (long long)g * a.ICg * a.HW + (long long)ih0[j] * a.W + iw0[j];
+    }
+    const float *wg = a.wp + (size_t)g * a.K * a.OCgP + m0 + lc;
+    bool m_ok[TM];
+#pragma unroll
+    for (int i = 0; i < TM; i++) m_ok[i] = m0 + i * MT + lc < a.OCgP;
+
+    typename M::acc_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < M::ACC; v++) acc[i][j][v] = 0.f;
+
+    float av[2][U][TM], bv[2][U][TN];
+
+    auto load_batch = [&](int s0, float(&A)[U][TM], float(&B)[U][TN]) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int k = (s0 + u) * M::KSTEP + lk;
+            const bool k_ok = (s0 + u) < s_end && k < a.K;
+#pragma unroll
+            for (int i = 0; i < TM; i++) A[u][i] = (k_ok && m_ok[i]) ? wg[(size_t)k * a.OCgP + i * MT] : 0.f;
+            if (POINTWISE) {
+#pragma unroll
+                for (int j = 0; j < TN; j++) B[u][j] = (k_ok && n_ok[j]) ? xg[j][(long long)k * a.HW] : 0.f;
+            } else {
+                const int c = a.KHKW == 1 ? k : (int)__umulhi((unsigned)k, a.magic_khkw);
+                const int rem = k - c * a.KHKW;
+                const int kh = a.KW == 1 ? rem : (int)__umulhi((unsigned)rem, a.magic_kw);
+                const int kw = rem - kh * a.KW;
+                const long long off = (long long)c * a.HW + kh * a.W + kw;
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const bool ok = k_ok && n_ok[j] && (unsigned)(ih0[j] + kh) < (unsigned)a.H &&
+                                    (unsigned)(iw0[j] + kw) < (unsigned)a.W;
+                    B[u][j] = ok ? xg[j][off] : 0.f;
+                }
+            }
+        }
+    };
+    auto compute = [&](const float(&A)[U][TM], const float(&B)[U][TN]) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const float bval = a.pre_relu ? fmaxf(B[u][j], 0.f) : B[u][j];
+                    acc[i][j] = M::run(A[u][i], bval, acc[i][j]);
+                }
+    };
+
+    const int batches = (s_end - s_begin + U - 1) / U;   // <= 0 for wavefronts beyond the end of K
+    if (batches > 0) load_batch(s_begin, av[0], bv[0]);
+    for (int b = 0; b < batches; b += 2) {
+        if (b + 1 < batches) load_batch(s_begin + (b + 1) * U, av[1], bv[1]);
+        compute(av[0], bv[0]);
+        if (b + 1 < batches) {
+            if (b + 2 < batches) load_batch(s_begin + (b + 2) * U, av[0], bv[0]);
+            compute(av[1], bv[1]);
+        }
+    }
+
+    // partial tiles meet in LDS: element e of lane l of wavefront w lives at red[(w * E + e) * 64 + l]
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < M::ACC; v++) red[(wave * E + (i * TN + j) * M::ACC + v) * 64 + lane] = acc[i][j][v];
+    __syncthreads();
+    for (int e = wave; e < E; e += NW) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; w++) sum += red[(w * E + e) * 64 + lane];
+        const int v = e % M::ACC;
+        const int j = (e / M::ACC) % TN;
+        const int i = e / (M::ACC * TN);
+        const int m = m0 + i * MT + M::row(v, lane);
+        const int nn = n0 + j * MT + lc;
+        if (m < a.OCg && nn < a.Npix) {
+            const int b = nn / a.OHW;
+            const int r = nn - b * a.OHW;
+            a.y[(long long)b * a.y_bs + ((long long)g * a.OCg + m) * a.OHW + r] = apply_act(sum + a.bias[g * a.OCg + m], a.act);
+        }
+    }
+}   // run
+};
+
+// ---- kernel configurations ------------------------------------------------------------------------------------------
+// X(index, name, BM, BN, BK, WM, WN, WK, MT, PD) for the LDS-tiled kernel
+#define IOS_TILED_VARIANTS(X)                                  \
+    X(0, "m64n64k32_w2x2x1_t32", 64, 64, 32, 2, 2, 1, 32, 3)   \
+    X(1, "m128n128k16_w2x2x1_t32", 128, 128, 16, 2, 2, 1, 32, 3) \
+    X(2, "m32n32k64_w1x1x4_t32", 32, 32, 64, 1, 1, 4, 32, 4)   \
+    X(3, "m64n32k32_w2x1x2_t32", 64, 32, 32, 2, 1, 2, 32, 4)   \
+    X(4, "m32n64k32_w1x2x2_t32", 32, 64, 32, 1, 2, 2, 32, 4)   \
+    X(5, "m128n64k16_w2x2x1_t32", 128, 64, 16, 2, 2, 1, 32, 3) \
+    X(6, "m64n16k64_w4x1x1_t16", 64, 16, 64, 4, 1, 1, 16, 3)   \
+    X(7, "m32n16k64_w2x1x2_t16", 32, 16, 64, 2, 1, 2, 16, 4)   \
+    X(8, "m16n16k128_w1x1x4_t16", 16, 16, 128, 1, 1, 4, 16, 3)
+// X(index, name, MT, TM, TN, NW, U) for the wave-split kernel
+#define IOS_WSPLIT_VARIANTS(X)                     \
+    X(9, "ws_m32n16_w16_t16", 16, 2, 1, 16, 4)     \
+    X(10, "ws_m16n16_w16_t16", 16, 1, 1, 16, 8)    \
+    X(11, "ws_m32n32_w16_t16", 16, 2, 2, 16, 4)    \
+    X(12, "ws_m64n16_w16_t16", 16, 4, 1, 16, 4)    \
+    X(13, "ws_m32n16_w8_t16", 16, 2, 1, 8, 4)      \
+    X(14, "ws_m32n16_w4_t16", 16, 2, 1, 4, 8)      \
+    X(15, "ws_m32n32_w16_t32", 32, 1, 1, 16, 8)    \
+    X(16, "ws_m16n32_w16_t16", 16, 1, 2, 16, 4)
+constexpr int kNumConvVariants = 17;
+
+}  // namespace ios

@@ -1,0 +1,37 @@
+// Fused stage launch: several independent device operations in one kernel launch.
+//
+// On MI355X a fork + join across HIP streams costs tens of microseconds while the batch-1 operators it would
+// overlap run for 3-15 us each, so concurrent groups of a stage are expressed as *one* grid: a table of work
+// items, each owning a contiguous range of blocks; every block looks up its item and runs that operator's
+// device body.  Operators of one group that depend on each other go to consecutive launches ("levels") on
+// the same stream, which orders them without any cross-queue synchronisation.
+#pragma once
+
+#include "launch_internal.h"
+
+namespace ios {
+
+enum WorkKind : int { WORK_CONV = 0, WORK_REDUCE, WORK_POOL, WORK_GLOBAL_POOL, WORK_DWCONV, WORK_CONV_DIRECT, WORK_NARY };
+
+struct WorkItem {
+    int kind;
+    int variant, pointwise;        // convolution kernel configuration
+    int tiles, groups;             // convolution grid decomposition: block = (tile, group, K slice)
+    int first_block, num_blocks;   // range of this item inside the fused grid
+    int reserved;
+    union {
+        ConvKernelArgs conv;
+        ReduceArgs reduce;
+        PoolArgs pool;
+        DirectConvArgs direct;
+        NaryKernelArgs nary;
+    };
+};
+
+// thread-block sizes the fused kernel is instantiated for
+constexpr int kFusedThreadClasses[] = {256, 512, 1024};
+
+// Launch `num_items` items (device pointer) as one grid of `total_blocks` blocks of `threads` threads.
+void launch_fused(int threads, const WorkItem *device_items, int num_items, int total_blocks, int smem_bytes, hipStream_t stream);
+
+}  // namespace ios

@@ -1,0 +1,93 @@
+// The fused stage kernel: see fused.h.
+#include "fused.h"
+
+#include <stdexcept>
+
+namespace ios {
+
+template <int T>
+__global__ __launch_bounds__(T) void fused_kernel(const WorkItem *__restrict__ items, int num_items) {
+    extern __shared__ floatx4 fused_smem[];
+    float *smem = reinterpret_cast<float *>(fused_smem);
+    const int bid = blockIdx.x;
+    int index = 0;
+    while (index + 1 < num_items && bid >= items[index + 1].first_block) index++;
+    const WorkItem &item = items[index];
+    const int local = bid - item.first_block;
+    const int num_blocks = item.num_blocks;
+    switch (item.kind) {
+        case WORK_CONV: {
+            const ConvKernelArgs a = item.conv;
+            const int tile = local % item.tiles;
+            const int rest = local / item.tiles;
+            const int g = rest % item.groups;
+            const int z = rest / item.groups;
+            const bool pointwise = item.pointwise != 0;
+            switch (item.variant) {
+#define IOS_CASE_TILED(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                          \
+    case IDX:                                                                                              \
+        if constexpr (64 * WM * WN * WK == T) {                                                            \
+            if (pointwise) ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD, true>::run(a, smem, tile, g, z);      \
+            else ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD, false>::run(a, smem, tile, g, z);               \
+        }                                                                                                  \
+        break;
+#define IOS_CASE_WSPLIT(IDX, NAME, MT, TM, TN, NW, U)                                        \
+    case IDX:                                                                                \
+        if constexpr (64 * NW == T) {                                                        \
+            if (pointwise) ConvWsplit<MT, TM, TN, NW, U, true>::run(a, smem, tile, g, z);    \
+            else ConvWsplit<MT, TM, TN, NW, U, false>::run(a, smem, tile, g, z);             \
+        }                                                                                    \
+        break;
+                IOS_TILED_VARIANTS(IOS_CASE_TILED)
+                IOS_WSPLIT_VARIANTS(IOS_CASE_WSPLIT)
+#undef IOS_CASE_TILED
+#undef IOS_CASE_WSPLIT
+                default: break;
+            }
+            break;
+        }
+        case WORK_REDUCE: {
+            const ReduceArgs a = item.reduce;
+            splitk_reduce_body(a, local, num_blocks);
+            break;
+        }
+        case WORK_POOL: {
+            const PoolArgs a = item.pool;
+            pool_body(a, local, num_blocks);
+            break;
+        }
+        case WORK_GLOBAL_POOL: {
+            const PoolArgs a = item.pool;
+            global_pool_body(a, local, num_blocks);
+            break;
+        }
+        case WORK_DWCONV: {
+            const DirectConvArgs a = item.direct;
+            dwconv_dispatch(a, local, num_blocks);
+            break;
+        }
+        case WORK_CONV_DIRECT: {
+            const DirectConvArgs a = item.direct;
+            conv_direct_body(a, local, num_blocks);
+            break;
+        }
+        case WORK_NARY: {
+            nary_dispatch(item.nary, local, num_blocks);   // read in place: the source table is indexed dynamically
+            break;
+        }
+        default: break;
+    }
+}
+
+void launch_fused(int threads, const WorkItem *device_items, int num_items, int total_blocks, int smem_bytes, hipStream_t stream) {
+    if (num_items < 1 || total_blocks < 1) throw std::runtime_error("fused launch: nothing to do");
+    const dim3 grid((unsigned)total_blocks);
+    switch (threads) {
+        case 256: hipLaunchKernelGGL(fused_kernel<256>, grid, dim3(256), smem_bytes, stream, device_items, num_items); break;
+        case 512: hipLaunchKernelGGL(fused_kernel<512>, grid, dim3(512), smem_bytes, stream, device_items, num_items); break;
+        case 1024: hipLaunchKernelGGL(fused_kernel<1024>, grid, dim3(1024), smem_bytes, stream, device_items, num_items); break;
+        default: throw std::runtime_error("fused launch: unsupported block size");
+    }
+}
+
+}  // namespace ios

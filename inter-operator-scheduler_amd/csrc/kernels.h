@@ -37,10 +37,12 @@ struct ConvProblem {
 };
 
 // One implicit-GEMM kernel configuration: block tile BM (output channels) x BN (pixels) x BK, a grid of
-// WM x WN x WK wavefronts (WK wavefronts split the block's K tile) built from MT x MT fp32 MFMA tiles.
+// WM x WN x WK wavefronts (WK wavefronts split K) built from MT x MT fp32 MFMA tiles.  `wave_split` selects
+// the kernel without LDS staging whose WK wavefronts each own a contiguous range of K (split_k is ignored).
 struct ConvVariant {
     const char *name;
     int BM, BN, BK, WM, WN, WK, MT;
+    bool wave_split;
     int threads() const { return 64 * WM * WN * WK; }
 };
 

@@ -1,0 +1,28 @@
+// Host-side builders of kernel argument blocks, shared by the stand-alone launchers and the fused stage kernel.
+#pragma once
+
+#include "conv_body.h"
+#include "pointwise_body.h"
+
+namespace ios {
+
+struct ConvDispatch {
+    ConvKernelArgs args;
+    int variant;
+    bool pointwise;
+    int threads, smem_bytes;
+    int tiles, groups, slices;       // grid of the main kernel
+    bool has_reduce;                 // split-K: a reduce pass must follow the main kernel
+    ReduceArgs reduce;
+    int reduce_blocks;
+};
+
+ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
+                                const float *bias, const TensorView &y, float *workspace);
+PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorView &y, bool global, int *blocks);
+DirectConvArgs make_direct_conv_args(const ConvProblem &p, const TensorView &x, const float *w, const float *bias,
+                                     const TensorView &y, int *blocks);
+NaryKernelArgs make_nary_args(const NaryArgs &in, int multiply, int accumulate, int act, int B, long long chw,
+                              const TensorView &y, int *blocks);
+
+}  // namespace ios

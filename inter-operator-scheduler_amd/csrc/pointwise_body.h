@@ -1,0 +1,225 @@
+// Device-side bodies of the memory-bound kernels (pooling, depth-wise and direct convolution, n-ary add /
+// multiply / activation / strided copy).  Every body processes the elements of logical block `block` out of
+// `num_blocks` with a block-stride loop, so the same code serves a stand-alone launch and a slice of the
+// fused stage kernel.  Tensors are NCHW views; consecutive lanes cover consecutive output columns.
+#pragma once
+
+#include "kernels.h"
+
+namespace ios {
+
+typedef float pw_floatx4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float act_apply(float v, int act) {
+    switch (act) {
+        case ACT_RELU: return fmaxf(v, 0.0f);
+        case ACT_TANH: return tanhf(v);
+        case ACT_SIGMOID: return 1.0f / (1.0f + __expf(-v));
+        default: return v;
+    }
+}
+
+struct PoolArgs {
+    const float *x;
+    float *y;
+    long long x_bs, y_bs;
+    PoolProblem p;
+};
+
+__device__ __forceinline__ void pool_body(const PoolArgs &a, int block, int num_blocks) {
+    const PoolProblem &p = a.p;
+    const long long per_image = (long long)p.C * p.OH * p.OW;
+    const long long total = per_image * p.B;
+    const float inv = 1.0f / (float)(p.KH * p.KW);
+    for (long long i = block * (long long)blockDim.x + threadIdx.x; i < total; i += (long long)num_blocks * blockDim.x) {
+        const int b = (int)(i / per_image);
+        const int o = (int)(i - b * per_image);
+        const int c = o / (p.OH * p.OW);
+        const int r = o - c * p.OH * p.OW;
+        const int oh = r / p.OW;
+        const int ow = r - oh * p.OW;
+        const float *xc = a.x + b * a.x_bs + (long long)c * p.H * p.W;
+        const int h0 = oh * p.sh - p.ph, w0 = ow * p.sw - p.pw;
+        const int hb = max(h0, 0), he = min(h0 + p.KH, p.H);
+        const int wb = max(w0, 0), we = min(w0 + p.KW, p.W);
+        float best = -INFINITY, sum = 0.f;
+        for (int h = hb; h < he; h++)
+            for (int w = wb; w < we; w++) {
+                const float v = xc[h * p.W + w];
+                best = fmaxf(best, v);
+                sum += v;
+            }
+        a.y[b * a.y_bs + o] = p.is_max ? best : sum * inv;
+    }
+}
+
+// window == whole map: one wavefront reduces one (image, channel) plane
+__device__ __forceinline__ void global_pool_body(const PoolArgs &a, int block, int num_blocks) {
+    const PoolProblem &p = a.p;
+    const int planes = p.B * p.C;
+    const int HW = p.H * p.W;
+    const int waves_per_block = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63;
+    for (int plane = block * waves_per_block + (threadIdx.x >> 6); plane < planes; plane += num_blocks * waves_per_block) {
+        const int b = plane / p.C, c = plane - b * p.C;
+        const float *xc = a.x + b * a.x_bs + (long long)c * HW;
+        float best = -INFINITY, sum = 0.f;
+        for (int i = lane; i < HW; i += 64) {
+            const float v = xc[i];
+            best = fmaxf(best, v);
+            sum += v;
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            best = fmaxf(best, __shfl_xor(best, off, 64));
+            sum += __shfl_xor(sum, off, 64);
+        }
+        if (lane == 0) a.y[b * a.y_bs + c] = p.is_max ? best : sum / (float)HW;
+    }
+}
+
+struct DirectConvArgs {
+    const float *x;
+    const float *w;
+    const float *bias;
+    float *y;
+    long long x_bs, y_bs;
+    ConvProblem p;
+};
+
+template <int KH, int KW>
+__device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, int num_blocks) {
+    const ConvProblem &p = a.p;
+    const int kh_n = KH > 0 ? KH : p.KH, kw_n = KW > 0 ? KW : p.KW;
+    const long long per_image = (long long)p.OC * p.OH * p.OW;
+    const long long total = per_image * p.B;
+    for (long long i = block * (long long)blockDim.x + threadIdx.x; i < total; i += (long long)num_blocks * blockDim.x) {
+        const int b = (int)(i / per_image);
+        const int o = (int)(i - b * per_image);
+        const int c = o / (p.OH * p.OW);
+        const int r = o - c * p.OH * p.OW;
+        const int oh = r / p.OW;
+        const int ow = r - oh * p.OW;
+        const float *xc = a.x + b * a.x_bs + (long long)c * p.H * p.W;
+        const float *wc = a.w + (size_t)c * kh_n * kw_n;
+        const int h0 = oh * p.sh - p.ph, w0 = ow * p.sw - p.pw;
+        float acc = a.bias[c];
+#pragma unroll
+        for (int i2 = 0; i2 < kh_n; i2++) {
+            const int h = h0 + i2;
+            if ((unsigned)h >= (unsigned)p.H) continue;
+#pragma unroll
+            for (int j = 0; j < kw_n; j++) {
+                const int ww = w0 + j;
+                if ((unsigned)ww >= (unsigned)p.W) continue;
+                float v = xc[h * p.W + ww];
+                if (p.pre_relu) v = fmaxf(v, 0.f);
+                acc = fmaf(v, wc[i2 * kw_n + j], acc);
+            }
+        }
+        a.y[b * a.y_bs + o] = act_apply(acc, p.act);
+    }
+}
+
+__device__ __forceinline__ void dwconv_dispatch(const DirectConvArgs &a, int block, int num_blocks) {
+    const ConvProblem &p = a.p;
+    if (p.KH == 3 && p.KW == 3) dwconv_body<3, 3>(a, block, num_blocks);
+    else if (p.KH == 5 && p.KW == 5) dwconv_body<5, 5>(a, block, num_blocks);
+    else if (p.KH == 7 && p.KW == 7) dwconv_body<7, 7>(a, block, num_blocks);
+    else dwconv_body<0, 0>(a, block, num_blocks);
+}
+
+__device__ __forceinline__ void conv_direct_body(const DirectConvArgs &a, int block, int num_blocks) {
+    const ConvProblem &p = a.p;
+    const int icg = p.IC / p.groups, ocg = p.OC / p.groups;
+    const long long per_image = (long long)p.OC * p.OH * p.OW;
+    const long long total = per_image * p.B;
+    for (long long i = block * (long long)blockDim.x + threadIdx.x; i < total; i += (long long)num_blocks * blockDim.x) {
+        const int b = (int)(i / per_image);
+        const int o = (int)(i - b * per_image);
+        const int oc = o / (p.OH * p.OW);
+        const int r = o - oc * p.OH * p.OW;
+        const int oh = r / p.OW;
+        const int ow = r - oh * p.OW;
+        const int g = oc / ocg;
+        const float *xg = a.x + b * a.x_bs + (long long)g * icg * p.H * p.W;
+        const float *wo = a.w + (size_t)oc * icg * p.KH * p.KW;
+        const int h0 = oh * p.sh - p.ph, w0 = ow * p.sw - p.pw;
+        float acc = a.bias[oc];
+        for (int c = 0; c < icg; c++)
+            for (int i2 = 0; i2 < p.KH; i2++) {
+                const int h = h0 + i2;
+                if ((unsigned)h >= (unsigned)p.H) continue;
+                for (int j = 0; j < p.KW; j++) {
+                    const int ww = w0 + j;
+                    if ((unsigned)ww >= (unsigned)p.W) continue;
+                    float v = xg[(long long)c * p.H * p.W + h * p.W + ww];
+                    if (p.pre_relu) v = fmaxf(v, 0.f);
+                    acc = fmaf(v, wo[(c * p.KH + i2) * p.KW + j], acc);
+                }
+            }
+        a.y[b * a.y_bs + o] = act_apply(acc, p.act);
+    }
+}
+
+struct NaryKernelArgs {
+    NaryArgs in;
+    float *y;
+    long long y_bs, chw, total;   // total counts VEC-wide packets
+    int multiply, accumulate, act, vec;
+};
+
+template <int VEC>
+__device__ __forceinline__ void nary_body(const NaryKernelArgs &k, int block, int num_blocks) {
+    // indices count VEC-wide packets; chw and every batch stride are multiples of VEC on this path
+    const NaryArgs &a = k.in;
+    const long long chw_v = k.chw / VEC;
+    for (long long i = block * (long long)blockDim.x + threadIdx.x; i < k.total; i += (long long)num_blocks * blockDim.x) {
+        const long long b = i / chw_v;
+        const long long o = (i - b * chw_v) * VEC;
+        float r[VEC];
+        float *dst = k.y + b * k.y_bs + o;
+        int first = 0;
+        if (k.accumulate) {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) r[e] = dst[e];
+        } else {
+            const float *s0 = a.src[0] + b * a.src_bstride[0] + o;
+            if (VEC == 4) {
+                const pw_floatx4 v = *reinterpret_cast<const pw_floatx4 *>(s0);
+#pragma unroll
+                for (int e = 0; e < VEC; e++) r[e] = v[e];
+            } else {
+                r[0] = s0[0];
+            }
+            first = 1;
+        }
+        for (int j = first; j < a.count; j++) {
+            const float *s = a.src[j] + b * a.src_bstride[j] + o;
+            float t[VEC];
+            if (VEC == 4) {
+                const pw_floatx4 v = *reinterpret_cast<const pw_floatx4 *>(s);
+#pragma unroll
+                for (int e = 0; e < VEC; e++) t[e] = v[e];
+            } else {
+                t[0] = s[0];
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; e++) r[e] = k.multiply ? r[e] * t[e] : r[e] + t[e];
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; e++) r[e] = act_apply(r[e], k.act);
+        if (VEC == 4) {
+            pw_floatx4 v = {r[0], r[1], r[2], r[3]};
+            *reinterpret_cast<pw_floatx4 *>(dst) = v;
+        } else {
+            dst[0] = r[0];
+        }
+    }
+}
+
+__device__ __forceinline__ void nary_dispatch(const NaryKernelArgs &k, int block, int num_blocks) {
+    if (k.vec == 4) nary_body<4>(k, block, num_blocks);
+    else nary_body<1>(k, block, num_blocks);
+}
+
+}  // namespace ios

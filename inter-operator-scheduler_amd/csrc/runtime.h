@@ -17,7 +17,9 @@ namespace ios {
 void hip_check(hipError_t status, const char *what, const char *file, int line);
 #define IOS_HIP(call) ::ios::hip_check((call), #call, __FILE__, __LINE__)
 
-enum class ExecMode { Streams, Graph };
+// Streams: one HIP stream per group, event fork/join.  Fused: one launch per level of a multi-group stage
+// (see fused.h).  The *Graph modes capture the same issue sequence into a hipGraph and replay it.
+enum class ExecMode { Streams, Graph, Fused, FusedGraph };
 
 class DeviceContext {
 public:
@@ -30,6 +32,7 @@ public:
 
     // a process-wide arena reused by the stateless latency / inference entry points
     float *shared_arena(size_t floats);
+    void *shared_table(size_t bytes);   // companion buffer for the launch tables of such sessions
 
     void set_option(const std::string &key, const std::string &value);
     ExecMode exec_mode() const { return exec_mode_; }
@@ -58,6 +61,8 @@ private:
     hipStream_t streams_[kMaxGroups];
     float *arena_ = nullptr;
     size_t arena_floats_ = 0;
+    void *table_ = nullptr;
+    size_t table_bytes_ = 0;
     ExecMode exec_mode_ = ExecMode::Streams;
     bool autotune_ = false;
     int forced_variant_ = -1;
@@ -92,7 +97,10 @@ private:
     void setup();
     void tune_convs();
     void launch_op(const PlanOp &op, hipStream_t stream);
-    void enqueue(bool stage_events);   // issue one forward pass on the stream pool
+    void enqueue(bool stage_events);   // issue one forward pass according to the execution mode
+    void enqueue_streams(bool stage_events);
+    void enqueue_fused(bool stage_events);
+    void build_fused();
     void forward();                    // enqueue or graph launch according to the execution mode
     void build_graph();
     void copy_out(const ViewRef &view, float *host);
@@ -106,7 +114,14 @@ private:
     std::vector<std::vector<hipEvent_t>> join_events_;    // per stage, per extra group
     std::vector<hipEvent_t> stage_events_;                // per stage, profile mode
     hipEvent_t start_ = nullptr, stop_ = nullptr;
+    struct FusedLaunch {
+        int threads, first_item, num_items, total_blocks, smem_bytes;
+    };
+    std::vector<std::vector<FusedLaunch>> fused_stages_;   // per stage; empty for single-group stages
+    void *fused_items_ = nullptr;                          // device copy of all work items
+    bool fused_built_ = false;
     hipGraph_t graph_ = nullptr;
+    ExecMode graph_mode_ = ExecMode::Graph;                // mode the captured graph was built for
     hipGraphExec_t graph_exec_ = nullptr;
 };
 

@@ -12,6 +12,8 @@
 // one event pair.
 #include "runtime.h"
 
+#include "fused.h"
+
 #include <cstdio>
 #include <cstring>
 #include <sstream>
@@ -190,11 +192,26 @@ float *DeviceContext::shared_arena(size_t floats) {
     return arena_;
 }
 
+void *DeviceContext::shared_table(size_t bytes) {
+    if (bytes > table_bytes_) {
+        IOS_HIP(hipDeviceSynchronize());
+        if (table_ != nullptr) IOS_HIP(hipFree(table_));
+        table_ = nullptr;
+        table_bytes_ = 0;
+        const size_t want = bytes * 2 + 4096;
+        IOS_HIP(hipMalloc(&table_, want));
+        table_bytes_ = want;
+    }
+    return table_;
+}
+
 void DeviceContext::set_option(const std::string &key, const std::string &value) {
     if (key == "executor") {
         if (value == "streams") exec_mode_ = ExecMode::Streams;
         else if (value == "graph") exec_mode_ = ExecMode::Graph;
-        else throw std::runtime_error("option executor: expected 'streams' or 'graph', got '" + value + "'");
+        else if (value == "fused") exec_mode_ = ExecMode::Fused;
+        else if (value == "fused_graph") exec_mode_ = ExecMode::FusedGraph;
+        else throw std::runtime_error("option executor: expected streams, graph, fused or fused_graph, got '" + value + "'");
     } else if (key == "autotune") {
         autotune_ = !(value == "0" || value == "false" || value == "off" || value.empty());
     } else if (key == "conv_variant") {
@@ -215,8 +232,10 @@ void DeviceContext::set_option(const std::string &key, const std::string &value)
 std::string DeviceContext::info_json() const {
     std::ostringstream os;
     os << "{\"name\":\"" << name_ << "\",\"arch\":\"" << arch_ << "\",\"compute_units\":" << num_cus_
-       << ",\"executor\":\"" << (exec_mode_ == ExecMode::Graph ? "graph" : "streams") << "\",\"autotune\":" << (autotune_ ? "true" : "false")
-       << ",\"max_groups\":" << kMaxGroups << "}";
+       << ",\"executor\":\"" << (exec_mode_ == ExecMode::Graph ? "graph" : exec_mode_ == ExecMode::Fused ? "fused" : exec_mode_ == ExecMode::FusedGraph ? "fused_graph" : "streams") << "\",\"autotune\":" << (autotune_ ? "true" : "false")
+       << ",\"max_groups\":" << kMaxGroups << ",\"conv_variants\":[";
+    for (int i = 0; i < conv_num_variants(); i++) os << (i ? "," : "") << '"' << conv_variant(i).name << '"';
+    os << "]}";
     return os.str();
 }
 
@@ -248,6 +267,7 @@ Session::~Session() {
     for (hipEvent_t e : stage_events_) (void)hipEventDestroy(e);
     if (start_ != nullptr) (void)hipEventDestroy(start_);
     if (stop_ != nullptr) (void)hipEventDestroy(stop_);
+    if (owns_memory_ && fused_items_ != nullptr) (void)hipFree(fused_items_);
     if (owns_memory_ && base_ != nullptr) (void)hipFree(base_);
 }
 
@@ -369,7 +389,7 @@ void Session::launch_op(const PlanOp &op, hipStream_t stream) {
     }
 }
 
-void Session::enqueue(bool stage_events) {
+void Session::enqueue_streams(bool stage_events) {
     hipStream_t main = ctx_.stream(0);
     for (size_t s = 0; s < plan_.stages.size(); s++) {
         const auto &groups = plan_.stages[s];
@@ -385,6 +405,154 @@ void Session::enqueue(bool stage_events) {
                 IOS_HIP(hipEventRecord(join_events_[s][g - 1], ctx_.stream((int)g)));
                 IOS_HIP(hipStreamWaitEvent(main, join_events_[s][g - 1], 0));
             }
+        }
+        if (stage_events) IOS_HIP(hipEventRecord(stage_events_[s], main));
+    }
+}
+
+void Session::enqueue(bool stage_events) {
+    const ExecMode mode = ctx_.exec_mode();
+    if (mode == ExecMode::Fused || mode == ExecMode::FusedGraph) enqueue_fused(stage_events);
+    else enqueue_streams(stage_events);
+}
+
+// ---- fused stage launches -----------------------------------------------------------------------------------------
+// A multi-group stage is cut into levels: level l holds the l-th kernel of every group (a split-K convolution
+// contributes its main kernel and, one level later, its reduction).  The kernels of one level are independent
+// and become work items of one fused launch per thread-block size; levels follow each other on the main stream.
+void Session::build_fused() {
+    if (fused_built_) return;
+    std::vector<WorkItem> items;
+    fused_stages_.assign(plan_.stages.size(), {});
+    struct Pending {
+        WorkItem item;
+        int threads;     // 0: any block size
+        int smem_bytes;
+    };
+    for (size_t s = 0; s < plan_.stages.size(); s++) {
+        const auto &groups = plan_.stages[s];
+        if (groups.size() <= 1) continue;
+        std::vector<std::vector<Pending>> chains(groups.size());
+        for (size_t g = 0; g < groups.size(); g++) {
+            for (int index : groups[g]) {
+                const PlanOp &op = plan_.ops[index];
+                Pending pend;
+                memset(&pend.item, 0, sizeof(WorkItem));
+                pend.threads = 0;
+                pend.smem_bytes = 0;
+                int blocks = 0;
+                switch (op.kind) {
+                    case OpKind::ConvMfma: {
+                        const PlanConv &c = plan_.convs[op.conv];
+                        const ConvDispatch d = make_conv_dispatch(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off,
+                                                                  tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr);
+                        pend.item.kind = WORK_CONV;
+                        pend.item.variant = d.variant;
+                        pend.item.pointwise = d.pointwise ? 1 : 0;
+                        pend.item.tiles = d.tiles;
+                        pend.item.groups = d.groups;
+                        pend.item.num_blocks = d.tiles * d.groups * d.slices;
+                        pend.item.conv = d.args;
+                        pend.threads = d.threads;
+                        pend.smem_bytes = d.smem_bytes;
+                        chains[g].push_back(pend);
+                        if (d.has_reduce) {
+                            Pending red;
+                            memset(&red.item, 0, sizeof(WorkItem));
+                            red.item.kind = WORK_REDUCE;
+                            red.item.num_blocks = d.reduce_blocks;
+                            red.item.reduce = d.reduce;
+                            red.threads = 0;
+                            red.smem_bytes = 0;
+                            chains[g].push_back(red);
+                        }
+                        continue;
+                    }
+                    case OpKind::ConvDepthwise:
+                    case OpKind::ConvDirect: {
+                        const PlanConv &c = plan_.convs[op.conv];
+                        pend.item.kind = op.kind == OpKind::ConvDepthwise ? WORK_DWCONV : WORK_CONV_DIRECT;
+                        pend.item.direct = make_direct_conv_args(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), &blocks);
+                        break;
+                    }
+                    case OpKind::Pool:
+                    case OpKind::GlobalPool:
+                        pend.item.kind = op.kind == OpKind::Pool ? WORK_POOL : WORK_GLOBAL_POOL;
+                        pend.item.pool = make_pool_args(op.pool, tv(op.in), tv(op.out), op.kind == OpKind::GlobalPool, &blocks);
+                        break;
+                    case OpKind::Nary:
+                    case OpKind::Unary: {
+                        NaryArgs in;
+                        if (op.kind == OpKind::Unary) {
+                            in.count = 1;
+                            in.src[0] = base_ + op.in.offset;
+                            in.src_bstride[0] = op.in.bstride;
+                        } else {
+                            in.count = (int)op.srcs.size();
+                            for (int i = 0; i < in.count; i++) {
+                                in.src[i] = base_ + op.srcs[i].offset;
+                                in.src_bstride[i] = op.srcs[i].bstride;
+                            }
+                        }
+                        pend.item.kind = WORK_NARY;
+                        pend.item.nary = make_nary_args(in, op.multiply, op.accumulate, op.act, plan_.batch,
+                                                        (long long)op.out.image_floats(), tv(op.out), &blocks);
+                        break;
+                    }
+                }
+                pend.item.num_blocks = blocks;   // sized for 256-thread blocks, rescaled below
+                chains[g].push_back(pend);
+            }
+        }
+        size_t depth = 0;
+        for (const auto &chain : chains) depth = std::max(depth, chain.size());
+        for (size_t level = 0; level < depth; level++) {
+            std::vector<Pending *> here;
+            int widest = 0;
+            for (auto &chain : chains)
+                if (level < chain.size()) {
+                    here.push_back(&chain[level]);
+                    widest = std::max(widest, chain[level].threads);
+                }
+            if (widest == 0) widest = 256;
+            for (int threads : kFusedThreadClasses) {
+                FusedLaunch launch{threads, (int)items.size(), 0, 0, 0};
+                for (Pending *pend : here) {
+                    const int wants = pend->threads == 0 ? widest : pend->threads;
+                    if (wants != threads) continue;
+                    WorkItem item = pend->item;
+                    if (pend->threads == 0) item.num_blocks = std::max(1, (item.num_blocks * 256 + threads - 1) / threads);
+                    item.first_block = launch.total_blocks;
+                    launch.total_blocks += item.num_blocks;
+                    launch.smem_bytes = std::max(launch.smem_bytes, pend->smem_bytes);
+                    launch.num_items++;
+                    items.push_back(item);
+                }
+                if (launch.num_items > 0) fused_stages_[s].push_back(launch);
+            }
+        }
+    }
+    if (!items.empty()) {
+        if (owns_memory_) IOS_HIP(hipMalloc(&fused_items_, items.size() * sizeof(WorkItem)));
+        else fused_items_ = ctx_.shared_table(items.size() * sizeof(WorkItem));
+        IOS_HIP(hipMemcpyAsync(fused_items_, items.data(), items.size() * sizeof(WorkItem), hipMemcpyHostToDevice, ctx_.stream(0)));
+        IOS_HIP(hipStreamSynchronize(ctx_.stream(0)));
+    }
+    fused_built_ = true;
+}
+
+void Session::enqueue_fused(bool stage_events) {
+    build_fused();
+    hipStream_t main = ctx_.stream(0);
+    const WorkItem *items = static_cast<const WorkItem *>(fused_items_);
+    for (size_t s = 0; s < plan_.stages.size(); s++) {
+        const auto &groups = plan_.stages[s];
+        if (groups.size() <= 1) {
+            for (const auto &group : groups)
+                for (int op : group) launch_op(plan_.ops[op], main);
+        } else {
+            for (const FusedLaunch &l : fused_stages_[s])
+                launch_fused(l.threads, items + l.first_item, l.num_items, l.total_blocks, l.smem_bytes, main);
         }
         if (stage_events) IOS_HIP(hipEventRecord(stage_events_[s], main));
     }
@@ -406,8 +574,19 @@ void Session::build_graph() {
 }
 
 void Session::forward() {
-    if (ctx_.exec_mode() == ExecMode::Graph) {
-        if (graph_exec_ == nullptr) build_graph();
+    const ExecMode mode = ctx_.exec_mode();
+    if (mode == ExecMode::Graph || mode == ExecMode::FusedGraph) {
+        if (graph_exec_ != nullptr && graph_mode_ != mode) {   // the option changed since the capture
+            IOS_HIP(hipGraphExecDestroy(graph_exec_));
+            IOS_HIP(hipGraphDestroy(graph_));
+            graph_exec_ = nullptr;
+            graph_ = nullptr;
+        }
+        if (graph_exec_ == nullptr) {
+            if (mode == ExecMode::FusedGraph) build_fused();   // allocations and copies stay outside the capture
+            build_graph();
+            graph_mode_ = mode;
+        }
         IOS_HIP(hipGraphLaunch(graph_exec_, ctx_.stream(0)));
     } else {
         enqueue(false);

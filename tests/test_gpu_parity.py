@@ -84,9 +84,14 @@ def test_conv_matches_oracle(case):
     assert_close(got, want, f'conv {case}')
 
 
-@pytest.mark.parametrize('variant', range(10))
+@pytest.mark.parametrize('variant', range(32))
 @pytest.mark.parametrize('split_k', [1, 3])
 def test_every_conv_kernel_variant(variant, split_k):
+    names = rt.device_info()['conv_variants']
+    if variant >= len(names):
+        pytest.skip('no such kernel variant')
+    if names[variant].startswith('ws_') and split_k > 1:
+        pytest.skip('wave-split kernels divide K inside the block')
     rt.set_option('conv_variant', variant)
     rt.set_option('conv_split_k', split_k)
     for in_shape, oc, k, s, p, batch in [((72, 19, 19), 88, (3, 3), (1, 1), (1, 1), 2),
@@ -158,6 +163,41 @@ def test_input_algebra_sum_concat_slice_activation_element():
                 assert_close(session.tensor(node), want[node.name], f'node {node.name} ({node.type}) batch {batch}')
 
 
+def test_fused_stage_launch_covers_every_operator_kind():
+    # one stage whose groups hold every kind of device operation, run as fused launches and on streams
+    def build(b, v):
+        a = ios.conv2d(b, [[v]], 40, (3, 3), padding=(1, 1))                       # matrix path
+        c = ios.conv2d(b, [[v]], 16, (3, 3), padding=(1, 1), groups=16)            # depth-wise
+        d = ios.conv2d(b, [[v]], 16, (3, 3), padding=(1, 1), groups=8)             # thin groups: direct path
+        e = ios.pool2d(b, [[v]], 'avg', (3, 3), (1, 1), (1, 1))
+        f = ios.pool2d(b, [[v]], 'global_avg')
+        s = ios.relu(b, [[v, v]])
+        u = ios.activation(b, [[Value(v.node, 2, 9)]], 'tanh', False)
+        a2 = ios.conv2d(b, [[a]], 24, (1, 1))
+        s2 = ios.relu_sep_conv(b, [[s]], 12, (3, 3), (1, 1), (1, 1))
+        ios.identity(b, [[a2], [c], [d], [e], [s2], [u]], is_exit=True)
+        return f
+    graph = single_op_graph((16, 14, 14), build)
+    names = [n.name for n in graph.blocks[0].inner_nodes]
+    # groups: conv chain, the others one per group
+    graph.blocks[0].stages = [[[names[0], names[7]], [names[1]], [names[2]], [names[3]], [names[4]], [names[5], names[8]], [names[6]]],
+                              [[graph.blocks[0].exit_node.name]]]
+    for split in (0, 3):
+        rt.set_option('conv_split_k', split)
+        for variant in (-1, 0, 9):
+            rt.set_option('conv_variant', variant)
+            for batch in (1, 2):
+                x = np.random.default_rng(5).standard_normal((batch, 16, 14, 14)).astype(np.float32)
+                want = ios_oracle.run(graph, x)
+                outs = {}
+                for executor in ('streams', 'fused', 'fused_graph'):
+                    rt.set_option('executor', executor)
+                    outs[executor] = rt.graph_inference(graph, batch, x)
+                    assert_close(outs[executor], want, f'{executor} split {split} variant {variant} batch {batch}')
+                np.testing.assert_array_equal(outs['fused'], outs['streams'])
+                np.testing.assert_array_equal(outs['fused_graph'], outs['streams'])
+
+
 def test_wide_sum_uses_accumulation():
     def build(b, v):
         parts = [ios.conv2d(b, [[v]], 6, (1, 1), act='identity') for _ in range(11)]
@@ -223,13 +263,17 @@ def test_network_matches_oracle_and_schedules_agree_bitwise(name, make, batch):
     parallel = rt.graph_inference(optimized, batch, x)
     np.testing.assert_array_equal(parallel, got)
 
-    rt.set_option('executor', 'graph')
-    with rt.Session(optimized, batch) as session:
-        session.load_weights()
-        session.set_input(x)
-        for _ in range(3):      # replays of the captured graph with host work in between
-            session.run()
-            np.testing.assert_array_equal(session.output(), got)
+    for executor in ('graph', 'fused', 'fused_graph'):
+        rt.set_option('executor', executor)
+        with rt.Session(optimized, batch) as session:
+            session.load_weights()
+            session.set_input(x)
+            for _ in range(3):      # replays (of the captured graph) with host work in between
+                session.run()
+                np.testing.assert_array_equal(session.output(), got, err_msg=executor)
+        if not big:
+            graph.greedy_schedule(8)
+            np.testing.assert_array_equal(rt.graph_inference(graph, batch, x), got, err_msg=executor + ' greedy')
 
 
 def test_merged_convolutions_match_unmerged():
