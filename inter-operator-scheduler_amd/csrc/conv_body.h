@@ -1,11 +1,13 @@
 // Implicit-GEMM convolution on the CDNA4 fp32 matrix cores.
 //
 // GEMM view per group:  Y[m][n] = sum_k Wp[k][m] * X_im2col[k][n]
-//   m = output channel inside the group (OCg), n = flattened (image, oh, ow) pixel, k = (c, kh, kw).
+//   m = output channel inside the group (OCg), n = flattened (image, oh, ow) pixel,
+//   k = (kh, kw, c) tap-major with the channels of every tap zero-padded to a multiple of the K tile.
 // The filter matrix is pre-packed k-major (launch_pack_filters) so that a block's BK x BM slice is read
 // with 16-byte loads along m.  The BK x BN input slice is gathered straight from the NCHW input view:
-// consecutive lanes take consecutive pixels, k is decomposed into (c, kh, kw) with multiply-high
-// divisions by launch constants, and padding is resolved by predication.  Global loads run PD tiles
+// consecutive lanes take consecutive pixels; because a K tile lies inside one filter tap, the tap's
+// (kh, kw), its padding test and its base offset are computed once per tile and an element costs one
+// address add (with k = (c, kh, kw) the gather spent ~17 VALU instructions per MFMA).  Global loads run PD tiles
 // ahead of the math in registers (the loop is latency bound at batch 1, where a block sees only a few
 // K tiles), tiles are staged in LDS (double buffered, one barrier per K tile) and consumed by
 // v_mfma_f32_32x32x2_f32 / v_mfma_f32_16x16x4_f32: lane l supplies A[k = l / MT][m = l % MT] and
@@ -35,10 +37,11 @@ struct ConvKernelArgs {
     float *y;
     float *ws;
     int H, W, OH, OW, sh, sw, ph, pw;
-    int KW, KHKW;
-    unsigned magic_khkw, magic_kw;   // floor(2^32 / d) + 1; exact quotients for k < 2^16
-    int ICg, OCg, OCgP, K, HW, OHW, groups;
+    int KW, taps;                     // taps = KH * KW
+    unsigned magic_icgp, magic_kw;    // floor(2^32 / d) + 1: exact quotients for dividends < 2^16
+    int ICg, ICgP, OCg, OCgP, Kq, HW, OHW, groups;   // Kq = taps * ICgP rows of the packed filter matrix
     long long x_bs, y_bs;
+    unsigned x_bytes, w_bytes;        // extents of the input view and of the packed filters, both < 2^31
     int Npix;
     int act, pre_relu;
     int split_k, k_chunk;
@@ -52,6 +55,25 @@ __device__ __forceinline__ float apply_act(float v, int act) {
         case ACT_SIGMOID: return 1.0f / (1.0f + __expf(-v));
         default: return v;
     }
+}
+
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+
+// Raw buffer loads: a 32-bit byte offset against a base + extent descriptor; offsets at or beyond the extent
+// read as zero, so an invalid element (padding, channel padding, tile overhang) is a load from kOutOfRange
+// and no branch or select on the loaded value is needed.
+constexpr unsigned kOutOfRange = 0x80000000u;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const float *base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ float buffer_load_f32(__amdgpu_buffer_rsrc_t r, unsigned byte_offset) {
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_offset, 0, 0));
+}
+__device__ __forceinline__ floatx4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, unsigned byte_offset) {
+    const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, 0, 0);
+    floatx4 f = {__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
+    return f;
 }
 
 template <int MT>
@@ -80,11 +102,12 @@ struct Mfma<16> {
     __device__ static __forceinline__ int row(int v, int lane) { return 4 * (lane >> 4) + v; }
 };
 
-template <int BM, int BN, int BK, int WM, int WN, int WK, int MT, int PD, bool POINTWISE>
+template <int BM, int BN, int BK, int WM, int WN, int WK, int MT, int PD>
 struct ConvTiled {
     using M = Mfma<MT>;
     static constexpr int T = 64 * WM * WN * WK;
     static constexpr int THREADS = T;
+    static constexpr int CPAD = BK;   // channel padding of the packed filters: a K tile never straddles two taps
     static constexpr int PAD = MT == 16 ? 16 : 4;   // MT 16 reads four rows per instruction: rows must not share banks
     static constexpr int LDA = BM + PAD, LDB = BN + PAD;
     static constexpr int TILE_FLOATS = 2 * BK * (LDA + LDB);
@@ -119,8 +142,8 @@ struct ConvTiled {
     const int m0 = tm * BM;
     const int n0 = tn * BN;
     const int k_begin = z * a.k_chunk;
-    const int k_end = min(a.K, k_begin + a.k_chunk);
-    const int nkt = (k_end - k_begin + BK - 1) / BK;
+    const int k_end = min(a.Kq, k_begin + a.k_chunk);
+    const int nkt = (k_end - k_begin) / BK;   // Kq and k_chunk are multiples of BK
 
     // ---- per-thread loader state ---------------------------------------------------------------------
     const int bn_l = tid % BN;
@@ -128,7 +151,7 @@ struct ConvTiled {
     const int n = n0 + bn_l;
     const bool n_ok = n < a.Npix;
     int ih0 = 0, iw0 = 0;
-    long long x_off = 0;
+    unsigned x_thread = 0;   // byte offset of (image, group, ih0, iw0); may wrap below zero, the tap offset brings it back
     {
         const int nn = n_ok ? n : 0;
         const int b = nn / a.OHW;
@@ -137,45 +160,51 @@ struct ConvTiled {
         const int ow = r - oh * a.OW;
         ih0 = oh * a.sh - a.ph;
         iw0 = ow * a.sw - a.pw;
-        x_off = (long long)b * a.x_bs + (long long)g * a.ICg * a.HW + (long long)ih0 * a.W + iw0;
+        x_thread = (unsigned)(((long long)b * a.x_bs + (long long)g * a.ICg * a.HW + (long long)ih0 * a.W + iw0) * 4);
     }
-    const float *xg = a.x + x_off;
-    const float *wg = a.wp + (size_t)g * a.K * a.OCgP;
+    const __amdgpu_buffer_rsrc_t xr = buffer_of(a.x, a.x_bytes);
+    const __amdgpu_buffer_rsrc_t wr = buffer_of(a.wp, a.w_bytes);
+    // constant per-thread byte offsets inside a tile: filter element (row, 4 columns) and input row (channel)
+    unsigned a_off[A_ITERS];
+#pragma unroll
+    for (int i = 0; i < A_ITERS; i++) {
+        const int slot = tid + i * T;
+        const int row = slot / A_VEC_PER_ROW;
+        const int c4 = slot % A_VEC_PER_ROW;
+        const bool ok = (A_SLOTS % T == 0 || slot < A_SLOTS) && m0 + c4 * 4 < a.OCgP;
+        a_off[i] = ok ? (unsigned)(((size_t)g * a.Kq * a.OCgP + (size_t)row * a.OCgP + m0 + c4 * 4) * 4) : kOutOfRange;
+    }
+    unsigned b_off[B_ITERS];
+#pragma unroll
+    for (int i = 0; i < B_ITERS; i++) b_off[i] = x_thread + (unsigned)((bk_l + i * B_ROWS_PER_PASS) * a.HW) * 4u;
 
     floatx4 a_reg[PD][A_ITERS];
     float b_reg[PD][B_ITERS];
 
+    // K is ordered tap-major: row k of the packed filters is (tap = k / ICgP, c = k % ICgP) with ICgP a
+    // multiple of BK, so a K tile lies inside one filter tap: (kh, kw) and the tile's base offsets are scalar,
+    // the padding test is one compare pair per thread, and an element costs an add and a select of its offset.
     auto load_tile = [&](int kt, floatx4(&ar)[A_ITERS], float(&br)[B_ITERS]) {
         const int k0 = k_begin + kt * BK;
+        const int tap = (int)__umulhi((unsigned)k0, a.magic_icgp);
+        const int c0 = k0 - tap * a.ICgP;
+        const int kh = a.KW == 1 ? tap : (int)__umulhi((unsigned)tap, a.magic_kw);
+        const int kw = tap - kh * a.KW;
+        const unsigned w_tile = (unsigned)(k0 * a.OCgP) * 4u;
+        const unsigned tile_kill = kt < nkt ? 0u : kOutOfRange;   // tiles past the end of the K range load zeros
 #pragma unroll
-        for (int i = 0; i < A_ITERS; i++) {
-            const int slot = tid + i * T;
-            const int row = slot / A_VEC_PER_ROW;
-            const int c4 = slot % A_VEC_PER_ROW;
-            const int k = k0 + row;
-            const int m = m0 + c4 * 4;
-            floatx4 v = {0.f, 0.f, 0.f, 0.f};
-            if ((A_SLOTS % T == 0 || slot < A_SLOTS) && k < k_end && m < a.OCgP)
-                v = *reinterpret_cast<const floatx4 *>(wg + (size_t)k * a.OCgP + m);
-            ar[i] = v;
-        }
+        for (int i = 0; i < A_ITERS; i++) ar[i] = buffer_load_f32x4(wr, (a_off[i] + w_tile) | tile_kill);
+        // invalid elements get the top offset bit set, which is beyond every extent; plain bit arithmetic keeps
+        // the loads of a tile in one basic block so that they are issued back to back
+        const unsigned in_h = (unsigned)(ih0 + kh) < (unsigned)a.H ? 1u : 0u;
+        const unsigned in_w = (unsigned)(iw0 + kw) < (unsigned)a.W ? 1u : 0u;
+        const unsigned kill = (((in_h & in_w & (n_ok ? 1u : 0u)) ^ 1u) << 31) | tile_kill;
+        const unsigned x_tile = (unsigned)(c0 * a.HW + kh * a.W + kw) * 4u;
+        const int c_last = a.ICg - c0 - 1 - bk_l;   // this thread's rows beyond c_last are channel padding
 #pragma unroll
         for (int i = 0; i < B_ITERS; i++) {
-            const int k = k0 + bk_l + i * B_ROWS_PER_PASS;
-            float v = 0.f;
-            if (k < k_end && n_ok) {
-                if (POINTWISE) {
-                    v = xg[(long long)k * a.HW];
-                } else {
-                    const int c = a.KHKW == 1 ? k : (int)__umulhi((unsigned)k, a.magic_khkw);
-                    const int rem = k - c * a.KHKW;
-                    const int kh = a.KW == 1 ? rem : (int)__umulhi((unsigned)rem, a.magic_kw);
-                    const int kw = rem - kh * a.KW;
-                    if ((unsigned)(ih0 + kh) < (unsigned)a.H && (unsigned)(iw0 + kw) < (unsigned)a.W)
-                        v = xg[(long long)c * a.HW + kh * a.W + kw];
-                }
-            }
-            br[i] = v;
+            const unsigned pad = (unsigned)(c_last - i * B_ROWS_PER_PASS) & kOutOfRange;   // sign bit
+            br[i] = buffer_load_f32(xr, (b_off[i] + x_tile) | kill | pad);
         }
     };
 
@@ -211,10 +240,11 @@ struct ConvTiled {
     // Register stage s holds tile kt with kt % PD == s.  In iteration kt the stage of tile kt is free (the
     // tile already sits in LDS buffer kt & 1), so it is refilled with tile kt + PD; the stage of tile kt + 1,
     // requested PD - 1 iterations ago, is written to the other LDS buffer after the math.
+    // The loop runs in rounds of PD tiles with a straight-line body; tiles past the end of the K range are
+    // loaded as zeros (see tile_kill) and cost at most PD - 1 idle MFMA tiles per block.
 #pragma unroll
-    for (int s = 0; s < PD; s++)
-        if (s < nkt) load_tile(s, a_reg[s], b_reg[s]);
-    if (nkt > 0) store_tile(0, a_reg[0], b_reg[0]);
+    for (int s = 0; s < PD; s++) load_tile(s, a_reg[s], b_reg[s]);
+    store_tile(0, a_reg[0], b_reg[0]);
     __syncthreads();
     const int lk = lane / MT;   // k offset of this lane inside an MFMA step
     const int lc = lane % MT;   // row (A) / column (B) of this lane inside an MFMA tile
@@ -222,9 +252,8 @@ struct ConvTiled {
 #pragma unroll
         for (int s = 0; s < PD; s++) {
             const int kt = kt0 + s;
-            if (kt >= nkt) break;
             const int buf = kt & 1;
-            if (kt + PD < nkt) load_tile(kt + PD, a_reg[s], b_reg[s]);
+            load_tile(kt + PD, a_reg[s], b_reg[s]);
             const float *Ab = As + buf * BK * LDA + (wk * KSLICE + lk) * LDA + wm * WTM + lc;
             const float *Bb = Bs + buf * BK * LDB + (wk * KSLICE + lk) * LDB + wn * WTN + lc;
 #pragma unroll
@@ -239,7 +268,7 @@ struct ConvTiled {
 #pragma unroll
                     for (int j = 0; j < TN; j++) acc[i][j] = M::run(av[i], bv[j], acc[i][j]);
             }
-            if (kt + 1 < nkt) store_tile(buf ^ 1, a_reg[(s + 1) % PD], b_reg[(s + 1) % PD]);
+            store_tile(buf ^ 1, a_reg[(s + 1) % PD], b_reg[(s + 1) % PD]);
             __syncthreads();
         }
     }
@@ -345,13 +374,14 @@ __device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int bloc
 // inside the K loop, two register batches of U k-steps keep dozens of loads in flight per lane, and the NW partial
 // tiles meet once in LDS, where the wavefronts share the bias + activation + store work.  The sum order is fixed
 // (k ascending inside a wavefront, wavefronts ascending), so results are reproducible.
-template <int MT, int TM, int TN, int NW, int U, bool POINTWISE>
+template <int MT, int TM, int TN, int NW, int U>
 struct ConvWsplit {
     using M = Mfma<MT>;
     static constexpr int BM = TM * MT, BN = TN * MT;
     static constexpr int E = TM * TN * M::ACC;
     static constexpr int THREADS = 64 * NW;
     static constexpr int SMEM_FLOATS = NW * E * 64;
+    static constexpr int CPAD = 8;   // channel padding of the packed filters this kernel expects
 
     __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *red, int tile, int g, int /*z*/) {
 
@@ -365,13 +395,13 @@ struct ConvWsplit {
     const int m0 = tm * BM;
     const int n0 = tn * BN;
 
-    const int steps_total = (a.K + M::KSTEP - 1) / M::KSTEP;
+    const int steps_total = a.Kq / M::KSTEP;   // Kq is a multiple of 8
     const int steps_per_wave = (steps_total + NW - 1) / NW;
     const int s_begin = wave * steps_per_wave;
     const int s_end = min(steps_total, s_begin + steps_per_wave);
 
     int ih0[TN], iw0[TN];
-    const float *xg[TN];
+    unsigned x_lane[TN];   // byte offset of (image, group channel lk, ih0, iw0); wraps like x_thread above
     bool n_ok[TN];
 #pragma unroll
     for (int j = 0; j < TN; j++) {
@@ -384,12 +414,18 @@ struct ConvWsplit {
         const int ow = r - oh * a.OW;
         ih0[j] = oh * a.sh - a.ph;
         iw0[j] = ow * a.sw - a.pw;
-        xg[j] = a.x + (long long)b * a.x_bs + (long long)g * a.ICg * a.HW + (long long)ih0[j] * a.W + iw0[j];
+        x_lane[j] = (unsigned)(((long long)b * a.x_bs + ((long long)g * a.ICg + lk) * a.HW + (long long)ih0[j] * a.W + iw0[j]) * 4);
     }
-    const float *wg = a.wp + (size_t)g * a.K * a.OCgP + m0 + lc;
-    bool m_ok[TM];
+    const __amdgpu_buffer_rsrc_t xr = buffer_of(a.x, a.x_bytes);
+    const __amdgpu_buffer_rsrc_t wr = buffer_of(a.wp, a.w_bytes);
+    unsigned w_lane[TM], w_kill[TM], n_kill[TN];
 #pragma unroll
-    for (int i = 0; i < TM; i++) m_ok[i] = m0 + i * MT + lc < a.OCgP;
+    for (int i = 0; i < TM; i++) {
+        w_kill[i] = m0 + i * MT + lc < a.OCgP ? 0u : kOutOfRange;
+        w_lane[i] = (unsigned)(((size_t)g * a.Kq * a.OCgP + (size_t)lk * a.OCgP + m0 + i * MT + lc) * 4);
+    }
+#pragma unroll
+    for (int j = 0; j < TN; j++) n_kill[j] = n_ok[j] ? 0u : kOutOfRange;
 
     typename M::acc_t acc[TM][TN];
 #pragma unroll
@@ -401,28 +437,29 @@ struct ConvWsplit {
 
     float av[2][U][TM], bv[2][U][TN];
 
+    // k-step s covers rows k = s * KSTEP + lk of the tap-major packed filters; ICgP is a multiple of KSTEP, so a
+    // step lies inside one filter tap and (tap, kh, kw, first channel) are wavefront-uniform
     auto load_batch = [&](int s0, float(&A)[U][TM], float(&B)[U][TN]) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int k = (s0 + u) * M::KSTEP + lk;
-            const bool k_ok = (s0 + u) < s_end && k < a.K;
+            const bool s_ok = (s0 + u) < s_end;
+            const int kb = (s0 + u) * M::KSTEP;
+            const int tap = (int)__umulhi((unsigned)kb, a.magic_icgp);
+            const int cb = kb - tap * a.ICgP;
+            const int kh = a.KW == 1 ? tap : (int)__umulhi((unsigned)tap, a.magic_kw);
+            const int kw = tap - kh * a.KW;
+            const unsigned w_step = (unsigned)(kb * a.OCgP) * 4u;
+            const unsigned step_kill = s_ok ? 0u : kOutOfRange;   // wavefront-uniform
 #pragma unroll
-            for (int i = 0; i < TM; i++) A[u][i] = (k_ok && m_ok[i]) ? wg[(size_t)k * a.OCgP + i * MT] : 0.f;
-            if (POINTWISE) {
+            for (int i = 0; i < TM; i++) A[u][i] = buffer_load_f32(wr, (w_lane[i] + w_step) | w_kill[i] | step_kill);
+            const unsigned x_step = (unsigned)(cb * a.HW + kh * a.W + kw) * 4u;
+            const unsigned c_kill = (unsigned)(a.ICg - 1 - cb - lk) & kOutOfRange;   // sign bit: channel padding
 #pragma unroll
-                for (int j = 0; j < TN; j++) B[u][j] = (k_ok && n_ok[j]) ? xg[j][(long long)k * a.HW] : 0.f;
-            } else {
-                const int c = a.KHKW == 1 ? k : (int)__umulhi((unsigned)k, a.magic_khkw);
-                const int rem = k - c * a.KHKW;
-                const int kh = a.KW == 1 ? rem : (int)__umulhi((unsigned)rem, a.magic_kw);
-                const int kw = rem - kh * a.KW;
-                const long long off = (long long)c * a.HW + kh * a.W + kw;
-#pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const bool ok = k_ok && n_ok[j] && (unsigned)(ih0[j] + kh) < (unsigned)a.H &&
-                                    (unsigned)(iw0[j] + kw) < (unsigned)a.W;
-                    B[u][j] = ok ? xg[j][off] : 0.f;
-                }
+            for (int j = 0; j < TN; j++) {
+                const unsigned in_h = (unsigned)(ih0[j] + kh) < (unsigned)a.H ? 1u : 0u;
+                const unsigned in_w = (unsigned)(iw0[j] + kw) < (unsigned)a.W ? 1u : 0u;
+                const unsigned kill = ((in_h & in_w) ^ 1u) << 31;
+                B[u][j] = buffer_load_f32(xr, (x_lane[j] + x_step) | kill | c_kill | n_kill[j] | step_kill);
             }
         }
     };

@@ -22,17 +22,16 @@ typedef void (*ConvKernelFn)(ConvKernelArgs);
 
 struct VariantEntry {
     ConvVariant v;
-    ConvKernelFn general;
-    ConvKernelFn pointwise;
+    ConvKernelFn kernel;
     int smem_floats;
 };
 
-#define IOS_TILED_ENTRY(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                                    \
-    {{NAME, BM, BN, BK, WM, WN, WK, MT, false}, conv_kernel<ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD, false>>,         \
-     conv_kernel<ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD, true>>, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD, false>::SMEM_FLOATS},
-#define IOS_WSPLIT_ENTRY(IDX, NAME, MT, TM, TN, NW, U)                                                                 \
-    {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true}, conv_kernel<ConvWsplit<MT, TM, TN, NW, U, false>>, \
-     conv_kernel<ConvWsplit<MT, TM, TN, NW, U, true>>, ConvWsplit<MT, TM, TN, NW, U, false>::SMEM_FLOATS},
+#define IOS_TILED_ENTRY(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                        \
+    {{NAME, BM, BN, BK, WM, WN, WK, MT, false, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::CPAD},           \
+     conv_kernel<ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>>, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::SMEM_FLOATS},
+#define IOS_WSPLIT_ENTRY(IDX, NAME, MT, TM, TN, NW, U)                                                                \
+    {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U>::CPAD},         \
+     conv_kernel<ConvWsplit<MT, TM, TN, NW, U>>, ConvWsplit<MT, TM, TN, NW, U>::SMEM_FLOATS},
 
 static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)};
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -48,15 +47,16 @@ const ConvVariant &conv_variant(int index) {
 static int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
 static int k_chunk_of(const ConvProblem &p, const ConvLaunch &l) {
-    if (kVariants[l.variant].v.wave_split) return p.K();   // one slice: K is divided inside the block
-    const int BK = kVariants[l.variant].v.BK;
-    const int tiles_k = ceil_div(p.K(), BK);
-    return ceil_div(tiles_k, l.split_k) * BK;
+    const ConvVariant &v = kVariants[l.variant].v;
+    const int kq = p.Kq(v.cpad);
+    if (v.wave_split) return kq;   // one slice: K is divided inside the block
+    const int tiles_k = kq / v.BK;
+    return ceil_div(tiles_k, l.split_k) * v.BK;
 }
 
 // split_k may ask for more slices than there are K tiles; the effective count leaves no slice empty
 static int effective_split(const ConvProblem &p, const ConvLaunch &l) {
-    return std::max(1, ceil_div(p.K(), k_chunk_of(p, l)));
+    return std::max(1, ceil_div(p.Kq(kVariants[l.variant].v.cpad), k_chunk_of(p, l)));
 }
 
 size_t conv_workspace_floats(const ConvProblem &p, const ConvLaunch &l) {
@@ -84,7 +84,7 @@ ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus) {
     const int pick = 7;   // 32 x 16 tile, four wavefronts
     const ConvVariant &v = kVariants[pick].v;
     const long long blocks = (long long)ceil_div(M, v.BM) * ceil_div(N, v.BN) * p.groups;
-    const int tiles_k = ceil_div(p.K(), v.BK);
+    const int tiles_k = p.Kq(v.cpad) / v.BK;
     int split = (int)std::min<long long>((want + blocks - 1) / blocks, std::max(1, tiles_k / 2));
     best.variant = pick;
     best.split_k = std::max(1, std::min(split, 32));
@@ -92,7 +92,10 @@ ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus) {
 }
 
 bool conv_matrix_path_supported(const ConvProblem &p) {
-    return p.K() < 65536 && p.Npix() < (1LL << 31) && (long long)p.IC * p.H * p.W < (1LL << 31);
+    // packed filter rows are indexed with 16 bits, input and filter byte offsets with 31 bits
+    const unsigned long long x_bytes = (unsigned long long)p.B * p.IC * p.H * p.W * 4ull;
+    const unsigned long long w_bytes = (unsigned long long)p.groups * p.Kq(128) * p.OCgP() * 4ull;
+    return p.Kq(128) < 65536 && p.Npix() < (1LL << 31) && x_bytes < (1ull << 30) && w_bytes < (1ull << 31);
 }
 
 ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
@@ -112,12 +115,17 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     a.ws = workspace;
     a.H = p.H; a.W = p.W; a.OH = p.OH; a.OW = p.OW;
     a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw;
-    a.KW = p.KW; a.KHKW = p.KH * p.KW;
-    a.magic_khkw = (unsigned)((1ULL << 32) / (unsigned)a.KHKW + 1);   // unused when the divisor is 1
-    a.magic_kw = (unsigned)((1ULL << 32) / (unsigned)a.KW + 1);
-    a.ICg = p.ICg(); a.OCg = p.OCg(); a.OCgP = p.OCgP(); a.K = p.K();
+    a.KW = p.KW; a.taps = p.KH * p.KW;
+    a.ICg = p.ICg(); a.ICgP = p.ICgP(e.v.cpad); a.OCg = p.OCg(); a.OCgP = p.OCgP(); a.Kq = p.Kq(e.v.cpad);
+    a.magic_icgp = (unsigned)((1ULL << 32) / (unsigned)a.ICgP + 1);   // ICgP >= 8
+    a.magic_kw = (unsigned)((1ULL << 32) / (unsigned)a.KW + 1);       // unused when KW == 1
     a.HW = p.H * p.W; a.OHW = p.OH * p.OW; a.groups = p.groups;
     a.x_bs = x.bstride; a.y_bs = y.bstride;
+    const unsigned long long x_bytes = ((unsigned long long)(p.B - 1) * x.bstride + (unsigned long long)p.IC * p.H * p.W) * 4ull;
+    const unsigned long long w_bytes = (unsigned long long)p.groups * p.Kq(e.v.cpad) * p.OCgP() * 4ull;
+    if (x_bytes >= (1ull << 31) || w_bytes >= (1ull << 31)) throw std::runtime_error("conv: tensor too large for 31-bit buffer offsets");
+    a.x_bytes = (unsigned)x_bytes;
+    a.w_bytes = (unsigned)w_bytes;
     a.Npix = (int)p.Npix();
     a.act = p.act; a.pre_relu = p.pre_relu;
     a.k_chunk = k_chunk_of(p, l);
@@ -127,7 +135,6 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     if (a.split_k > 1 && workspace == nullptr) throw std::runtime_error("conv: split-K launch without workspace");
     if (p.groups > 65535 || a.split_k > 65535) throw std::runtime_error("conv: grid too large");
     d.variant = l.variant;
-    d.pointwise = p.is_pointwise();
     d.threads = e.v.threads();
     d.smem_bytes = e.smem_floats * (int)sizeof(float);
     d.tiles = a.tiles_m * a.tiles_n;
@@ -157,30 +164,42 @@ void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorVie
     const ConvDispatch d = make_conv_dispatch(p, l, x, packed, bias, y, workspace);
     const VariantEntry &e = kVariants[d.variant];
     const dim3 grid((unsigned)d.tiles, (unsigned)d.groups, (unsigned)d.slices);
-    hipLaunchKernelGGL(d.pointwise ? e.pointwise : e.general, grid, dim3(d.threads), d.smem_bytes, stream, d.args);
+    hipLaunchKernelGGL(e.kernel, grid, dim3(d.threads), d.smem_bytes, stream, d.args);
     if (d.has_reduce) hipLaunchKernelGGL(splitk_reduce_kernel, dim3(d.reduce_blocks), dim3(256), 0, stream, d.reduce);
 }
 
 // ---- filter packing ------------------------------------------------------------------------
-__global__ void pack_filters_kernel(const float *w, float *packed, int OCg, int OCgP, int K, int groups) {
-    // packed[g][k][m] = w[g*OCg + m][k]   (k runs over (c, kh, kw) exactly as in the original layout)
-    const size_t total = (size_t)groups * K * OCgP;
+__global__ void pack_filters_kernel(const float *w, float *packed, int OCg, int OCgP, int ICg, int ICgP, int taps, int groups) {
+    // packed[g][tap * ICgP + c][m] = w[g * OCg + m][c][tap];  rows with c >= ICg and columns with m >= OCg are zero
+    const size_t total = (size_t)groups * taps * ICgP * OCgP;
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const int m = (int)(i % OCgP);
         const size_t gk = i / OCgP;
-        const int k = (int)(gk % K);
-        const int g = (int)(gk / K);
-        packed[i] = m < OCg ? w[((size_t)g * OCg + m) * K + k] : 0.f;
+        const int c = (int)(gk % ICgP);
+        const size_t gt = gk / ICgP;
+        const int tap = (int)(gt % taps);
+        const int g = (int)(gt / taps);
+        packed[i] = (m < OCg && c < ICg) ? w[(((size_t)g * OCg + m) * ICg + c) * taps + tap] : 0.f;
     }
 }
 
-size_t conv_packed_floats(const ConvProblem &p) { return (size_t)p.groups * p.K() * p.OCgP(); }
+size_t conv_packed_floats(const ConvProblem &p, const ConvLaunch &l) {
+    if (l.variant < 0 || l.variant >= kNumVariants) throw std::runtime_error("conv: bad variant");
+    return (size_t)p.groups * p.Kq(kVariants[l.variant].v.cpad) * p.OCgP();
+}
 
-void launch_pack_filters(const ConvProblem &p, const float *w, float *packed, hipStream_t stream) {
-    const size_t total = conv_packed_floats(p);
+size_t conv_packed_floats_max(const ConvProblem &p) {
+    size_t most = 0;
+    for (const VariantEntry &e : kVariants) most = std::max(most, (size_t)p.groups * p.Kq(e.v.cpad) * p.OCgP());
+    return most;
+}
+
+void launch_pack_filters(const ConvProblem &p, const ConvLaunch &l, const float *w, float *packed, hipStream_t stream) {
+    const size_t total = conv_packed_floats(p, l);
+    const int cpad = kVariants[l.variant].v.cpad;
     const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 65535);
-    hipLaunchKernelGGL(pack_filters_kernel, dim3(blocks), dim3(256), 0, stream, w, packed, p.OCg(), p.OCgP(), p.K(),
-                       p.groups);
+    hipLaunchKernelGGL(pack_filters_kernel, dim3(blocks), dim3(256), 0, stream, w, packed, p.OCg(), p.OCgP(), p.ICg(), p.ICgP(cpad),
+                       p.KH * p.KW, p.groups);
 }
 
 }  // namespace ios

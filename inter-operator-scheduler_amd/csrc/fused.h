@@ -15,7 +15,7 @@ enum WorkKind : int { WORK_CONV = 0, WORK_REDUCE, WORK_POOL, WORK_GLOBAL_POOL, W
 
 struct WorkItem {
     int kind;
-    int variant, pointwise;        // convolution kernel configuration
+    int variant, reserved0;        // convolution kernel configuration
     int tiles, groups;             // convolution grid decomposition: block = (tile, group, K slice)
     int first_block, num_blocks;   // range of this item inside the fused grid
     int reserved;

@@ -22,21 +22,14 @@ __global__ __launch_bounds__(T) void fused_kernel(const WorkItem *__restrict__ i
             const int rest = local / item.tiles;
             const int g = rest % item.groups;
             const int z = rest / item.groups;
-            const bool pointwise = item.pointwise != 0;
             switch (item.variant) {
 #define IOS_CASE_TILED(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                          \
     case IDX:                                                                                              \
-        if constexpr (64 * WM * WN * WK == T) {                                                            \
-            if (pointwise) ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD, true>::run(a, smem, tile, g, z);      \
-            else ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD, false>::run(a, smem, tile, g, z);               \
-        }                                                                                                  \
+        if constexpr (64 * WM * WN * WK == T) ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::run(a, smem, tile, g, z); \
         break;
 #define IOS_CASE_WSPLIT(IDX, NAME, MT, TM, TN, NW, U)                                        \
     case IDX:                                                                                \
-        if constexpr (64 * NW == T) {                                                        \
-            if (pointwise) ConvWsplit<MT, TM, TN, NW, U, true>::run(a, smem, tile, g, z);    \
-            else ConvWsplit<MT, TM, TN, NW, U, false>::run(a, smem, tile, g, z);             \
-        }                                                                                    \
+        if constexpr (64 * NW == T) ConvWsplit<MT, TM, TN, NW, U>::run(a, smem, tile, g, z); \
         break;
                 IOS_TILED_VARIANTS(IOS_CASE_TILED)
                 IOS_WSPLIT_VARIANTS(IOS_CASE_WSPLIT)

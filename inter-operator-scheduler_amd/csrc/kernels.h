@@ -29,10 +29,12 @@ struct ConvProblem {
     int ICg() const { return IC / groups; }
     int OCg() const { return OC / groups; }
     int K() const { return ICg() * KH * KW; }
+    // rows of the packed filter matrix when the channels of every tap are padded to a multiple of cpad
+    int ICgP(int cpad) const { return (ICg() + cpad - 1) / cpad * cpad; }
+    int Kq(int cpad) const { return KH * KW * ICgP(cpad); }
     long long Npix() const { return (long long)B * OH * OW; }
     int OCgP() const { return (OCg() + 3) & ~3; }  // row length of the packed filter matrix
     bool is_depthwise() const { return groups > 1 && IC == groups && OC == groups; }
-    bool is_pointwise() const { return KH == 1 && KW == 1 && ph == 0 && pw == 0; }
     double flops() const { return 2.0 * (double)Npix() * OC * K(); }
 };
 
@@ -43,6 +45,7 @@ struct ConvVariant {
     const char *name;
     int BM, BN, BK, WM, WN, WK, MT;
     bool wave_split;
+    int cpad;   // channel padding of the packed filters this configuration reads
     int threads() const { return 64 * WM * WN * WK; }
 };
 
@@ -56,15 +59,17 @@ struct ConvLaunch {
 
 // Floats of workspace a launch configuration needs (split_k partial outputs).
 size_t conv_workspace_floats(const ConvProblem &p, const ConvLaunch &l);
-// The matrix path indexes k with 16 bits and pixels / input offsets with 31 bits.
+// The matrix path indexes packed filter rows with 16 bits and pixels / input offsets with 31 bits.
 bool conv_matrix_path_supported(const ConvProblem &p);
 
 // Default configuration from a closed-form occupancy model (num_cus = compute units of the device).
 ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus);
 
-// Filter packing: w[OC][ICg][KH][KW] -> packed[g][K][OCgP] (K = ICg*KH*KW, rows zero padded to OCgP).
-size_t conv_packed_floats(const ConvProblem &p);
-void launch_pack_filters(const ConvProblem &p, const float *w, float *packed, hipStream_t stream);
+// Filter packing for a kernel configuration: w[OC][ICg][KH][KW] -> packed[g][(kh*KW + kw)*ICgP + c][OCgP],
+// ICgP = ICg rounded up to the configuration's channel padding (zero rows), OCgP = OCg rounded up to 4.
+size_t conv_packed_floats(const ConvProblem &p, const ConvLaunch &l);
+size_t conv_packed_floats_max(const ConvProblem &p);   // over all configurations
+void launch_pack_filters(const ConvProblem &p, const ConvLaunch &l, const float *w, float *packed, hipStream_t stream);
 
 // y = act(conv(x, w) + bias).  `packed` comes from launch_pack_filters.  `workspace` holds the split_k
 // partial outputs (conv_workspace_floats); with split_k > 1 a second kernel reduces them on the same stream.

@@ -9,7 +9,6 @@ namespace ios {
 struct ConvDispatch {
     ConvKernelArgs args;
     int variant;
-    bool pointwise;
     int threads, smem_bytes;
     int tiles, groups, slices;       // grid of the main kernel
     bool has_reduce;                 // split-K: a reduce pass must follow the main kernel

@@ -479,13 +479,15 @@ private:
         OpKind kind;
         if (p.is_depthwise()) {
             kind = OpKind::ConvDepthwise;
-        } else if ((p.groups > 1 && (p.ICg() < 4 || p.OCg() < 8)) || !conv_matrix_path_supported(p)) {
+        } else if ((p.groups > 1 && (p.ICg() < 4 || p.OCg() < 8)) || !conv_matrix_path_supported(p) ||
+                   ((unsigned long long)(batch_ - 1) * in.bstride + in.image_floats()) * 4ull >= (1ull << 31)) {
+            // thin groups, or an input view whose extent does not fit the matrix path's 31-bit byte offsets
             kind = OpKind::ConvDirect;
         } else {
             kind = OpKind::ConvMfma;
             conv.matrix_path = true;
-            conv.packed_off = reserve(conv_packed_floats(p));
             conv.launch = chooser_(p);
+            conv.packed_off = reserve(conv_packed_floats(p, conv.launch));
         }
         if (plan_.conv_index.count(n.name)) throw std::runtime_error("duplicate convolution name '" + n.name + "'");
         plan_.conv_index[n.name] = static_cast<int>(plan_.convs.size());

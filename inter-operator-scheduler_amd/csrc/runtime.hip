@@ -110,8 +110,8 @@ ConvLaunch DeviceContext::tune_conv(const ConvProblem &p) {
     y.C = p.OC; y.H = p.OH; y.W = p.OW; y.bstride = (long long)p.OC * p.OH * p.OW;
     x.ptr = tuning_buffer(0, (size_t)p.B * x.bstride);
     y.ptr = tuning_buffer(1, (size_t)p.B * y.bstride);
-    float *packed = tuning_buffer(2, conv_packed_floats(p) + p.OC);
-    float *bias = packed + conv_packed_floats(p);
+    float *packed = tuning_buffer(2, conv_packed_floats_max(p) + p.OC);
+    float *bias = packed + conv_packed_floats_max(p);
     hipStream_t stream = streams_[0];
     hipEvent_t start, stop;
     IOS_HIP(hipEventCreate(&start));
@@ -288,7 +288,7 @@ void Session::setup() {
         if (!conv.matrix_path) continue;
         // the probes never upload filters: pack whatever the filter region holds so that the matrix
         // path reads initialised memory
-        launch_pack_filters(conv.problem, base_ + conv.weight_off, base_ + conv.packed_off, main);
+        launch_pack_filters(conv.problem, conv.launch, base_ + conv.weight_off, base_ + conv.packed_off, main);
     }
     const size_t num_stages = plan_.stages.size();
     fork_events_.assign(num_stages, nullptr);
@@ -325,7 +325,7 @@ bool Session::set_conv_weights(const char *name, const float *weight, const floa
     hipStream_t main = ctx_.stream(0);
     IOS_HIP(hipMemcpyAsync(base_ + conv.weight_off, weight, (size_t)p.OC * p.K() * sizeof(float), hipMemcpyHostToDevice, main));
     IOS_HIP(hipMemcpyAsync(base_ + conv.bias_off, bias, (size_t)p.OC * sizeof(float), hipMemcpyHostToDevice, main));
-    if (conv.matrix_path) launch_pack_filters(p, base_ + conv.weight_off, base_ + conv.packed_off, main);
+    if (conv.matrix_path) launch_pack_filters(p, conv.launch, base_ + conv.weight_off, base_ + conv.packed_off, main);
     IOS_HIP(hipStreamSynchronize(main));
     return true;
 }
@@ -448,7 +448,6 @@ void Session::build_fused() {
                                                                   tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr);
                         pend.item.kind = WORK_CONV;
                         pend.item.variant = d.variant;
-                        pend.item.pointwise = d.pointwise ? 1 : 0;
                         pend.item.tiles = d.tiles;
                         pend.item.groups = d.groups;
                         pend.item.num_blocks = d.tiles * d.groups * d.slices;
