@@ -486,8 +486,7 @@ private:
         } else {
             kind = OpKind::ConvMfma;
             conv.matrix_path = true;
-            conv.launch = chooser_(p);
-            conv.packed_off = reserve(conv_packed_floats(p, conv.launch));
+            // the kernel configuration depends on how many groups share the stage: chosen in finish()
         }
         if (plan_.conv_index.count(n.name)) throw std::runtime_error("duplicate convolution name '" + n.name + "'");
         plan_.conv_index[n.name] = static_cast<int>(plan_.convs.size());
@@ -590,8 +589,18 @@ private:
         int out_node = last_stage_units.back();
         plan_.output = view_of(out_node);
         plan_.output_name = nodes_[out_node].name;
-        for (PlanConv &conv : plan_.convs) {
+        std::vector<int> share(plan_.convs.size(), 1);
+        for (const PlanOp &op : plan_.ops)
+            if (op.conv >= 0 && op.stage >= 0) {
+                int busy = 0;
+                for (const auto &group : plan_.stages[op.stage]) busy += group.empty() ? 0 : 1;
+                share[op.conv] = std::max(1, busy);
+            }
+        for (size_t i = 0; i < plan_.convs.size(); i++) {
+            PlanConv &conv = plan_.convs[i];
             if (!conv.matrix_path) continue;
+            conv.launch = chooser_(conv.problem, share[i]);
+            conv.packed_off = reserve(conv_packed_floats(conv.problem, conv.launch));
             conv.ws_floats = conv_workspace_floats(conv.problem, conv.launch);
             if (conv.ws_floats > 0) conv.ws_off = reserve(conv.ws_floats);
         }

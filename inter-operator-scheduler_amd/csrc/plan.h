@@ -78,8 +78,10 @@ struct Plan {
 
 enum class PlanMode { Graph, Block, Stage };
 
-// Picks the kernel configuration of a matrix-path convolution (closed-form model or measured).
-typedef std::function<ConvLaunch(const ConvProblem &)> LaunchChooser;
+// Picks the kernel configuration of a matrix-path convolution (closed-form model or measured).  `share` is the
+// number of groups that run concurrently in the convolution's stage: a kernel that shares the device with
+// share - 1 others should occupy about 1 / share of it rather than all of it.
+typedef std::function<ConvLaunch(const ConvProblem &, int share)> LaunchChooser;
 
 // Compile a document.  `extra` is the input-shape document of stage mode ({name: [C, H, W]}).
 // Throws std::runtime_error on malformed documents, unknown operator types, non-topological schedules

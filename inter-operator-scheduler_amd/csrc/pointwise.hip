@@ -24,6 +24,7 @@ PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorV
         throw std::runtime_error("pool: tensor views do not match the problem");
     if (global && (p.KH != p.H || p.KW != p.W || p.OH != 1 || p.OW != 1))
         throw std::runtime_error("global pool: window must be the whole map");
+    if ((long long)p.B * p.C * p.OH * p.OW >= (1LL << 31)) throw std::runtime_error("pool: tensor too large for 32-bit indexing");
     PoolArgs a;
     a.x = x.ptr;
     a.y = y.ptr;
@@ -39,6 +40,7 @@ DirectConvArgs make_direct_conv_args(const ConvProblem &p, const TensorView &x, 
                                      const TensorView &y, int *blocks) {
     if (x.C != p.IC || x.H != p.H || x.W != p.W || y.C != p.OC || y.H != p.OH || y.W != p.OW)
         throw std::runtime_error("conv: tensor views do not match the problem");
+    if ((long long)p.B * p.OC * p.OH * p.OW >= (1LL << 31)) throw std::runtime_error("conv: tensor too large for 32-bit indexing");
     DirectConvArgs a;
     a.x = x.ptr;
     a.w = w;
@@ -58,6 +60,7 @@ NaryKernelArgs make_nary_args(const NaryArgs &in, int multiply, int accumulate, 
     if (in.count < 1 || in.count > kMaxNaryInputs) throw std::runtime_error("nary: bad input count");
     bool vec = (chw % 4 == 0) && (y.bstride % 4 == 0) && aligned16(y.ptr);
     for (int j = 0; j < in.count; j++) vec = vec && (in.src_bstride[j] % 4 == 0) && aligned16(in.src[j]);
+    if ((long long)B * chw >= (1LL << 31)) throw std::runtime_error("nary: tensor too large for 32-bit indexing");
     NaryKernelArgs a;
     a.in = in;
     a.y = y.ptr;

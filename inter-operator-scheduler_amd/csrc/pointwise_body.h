@@ -28,17 +28,19 @@ struct PoolArgs {
 
 __device__ __forceinline__ void pool_body(const PoolArgs &a, int block, int num_blocks) {
     const PoolProblem &p = a.p;
-    const long long per_image = (long long)p.C * p.OH * p.OW;
-    const long long total = per_image * p.B;
+    // 32-bit index arithmetic: the host side rejects tensors with 2^31 or more elements
+    const unsigned plane = (unsigned)(p.OH * p.OW);
+    const unsigned per_image = (unsigned)p.C * plane;
+    const unsigned total = per_image * (unsigned)p.B;
     const float inv = 1.0f / (float)(p.KH * p.KW);
-    for (long long i = block * (long long)blockDim.x + threadIdx.x; i < total; i += (long long)num_blocks * blockDim.x) {
-        const int b = (int)(i / per_image);
-        const int o = (int)(i - b * per_image);
-        const int c = o / (p.OH * p.OW);
-        const int r = o - c * p.OH * p.OW;
-        const int oh = r / p.OW;
-        const int ow = r - oh * p.OW;
-        const float *xc = a.x + b * a.x_bs + (long long)c * p.H * p.W;
+    for (unsigned i = block * blockDim.x + threadIdx.x; i < total; i += num_blocks * blockDim.x) {
+        const unsigned b = i / per_image;
+        const unsigned o = i - b * per_image;
+        const unsigned c = o / plane;
+        const unsigned r = o - c * plane;
+        const int oh = (int)(r / (unsigned)p.OW);
+        const int ow = (int)r - oh * p.OW;
+        const float *xc = a.x + (long long)b * a.x_bs + (long long)c * p.H * p.W;
         const int h0 = oh * p.sh - p.ph, w0 = ow * p.sw - p.pw;
         const int hb = max(h0, 0), he = min(h0 + p.KH, p.H);
         const int wb = max(w0, 0), we = min(w0 + p.KW, p.W);
@@ -49,7 +51,7 @@ __device__ __forceinline__ void pool_body(const PoolArgs &a, int block, int num_
                 best = fmaxf(best, v);
                 sum += v;
             }
-        a.y[b * a.y_bs + o] = p.is_max ? best : sum * inv;
+        a.y[(long long)b * a.y_bs + o] = p.is_max ? best : sum * inv;
     }
 }
 
@@ -90,16 +92,17 @@ template <int KH, int KW>
 __device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, int num_blocks) {
     const ConvProblem &p = a.p;
     const int kh_n = KH > 0 ? KH : p.KH, kw_n = KW > 0 ? KW : p.KW;
-    const long long per_image = (long long)p.OC * p.OH * p.OW;
-    const long long total = per_image * p.B;
-    for (long long i = block * (long long)blockDim.x + threadIdx.x; i < total; i += (long long)num_blocks * blockDim.x) {
-        const int b = (int)(i / per_image);
-        const int o = (int)(i - b * per_image);
-        const int c = o / (p.OH * p.OW);
-        const int r = o - c * p.OH * p.OW;
-        const int oh = r / p.OW;
-        const int ow = r - oh * p.OW;
-        const float *xc = a.x + b * a.x_bs + (long long)c * p.H * p.W;
+    const unsigned plane = (unsigned)(p.OH * p.OW);
+    const unsigned per_image = (unsigned)p.OC * plane;
+    const unsigned total = per_image * (unsigned)p.B;
+    for (unsigned i = block * blockDim.x + threadIdx.x; i < total; i += num_blocks * blockDim.x) {
+        const unsigned b = i / per_image;
+        const unsigned o = i - b * per_image;
+        const unsigned c = o / plane;
+        const unsigned r = o - c * plane;
+        const int oh = (int)(r / (unsigned)p.OW);
+        const int ow = (int)r - oh * p.OW;
+        const float *xc = a.x + (long long)b * a.x_bs + (long long)c * p.H * p.W;
         const float *wc = a.w + (size_t)c * kh_n * kw_n;
         const int h0 = oh * p.sh - p.ph, w0 = ow * p.sw - p.pw;
         float acc = a.bias[c];
@@ -116,7 +119,7 @@ __device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, 
                 acc = fmaf(v, wc[i2 * kw_n + j], acc);
             }
         }
-        a.y[b * a.y_bs + o] = act_apply(acc, p.act);
+        a.y[(long long)b * a.y_bs + o] = act_apply(acc, p.act);
     }
 }
 
@@ -172,18 +175,19 @@ template <int VEC>
 __device__ __forceinline__ void nary_body(const NaryKernelArgs &k, int block, int num_blocks) {
     // indices count VEC-wide packets; chw and every batch stride are multiples of VEC on this path
     const NaryArgs &a = k.in;
-    const long long chw_v = k.chw / VEC;
-    for (long long i = block * (long long)blockDim.x + threadIdx.x; i < k.total; i += (long long)num_blocks * blockDim.x) {
-        const long long b = i / chw_v;
-        const long long o = (i - b * chw_v) * VEC;
+    const unsigned chw_v = (unsigned)(k.chw / VEC);
+    const unsigned total = (unsigned)k.total;
+    for (unsigned i = block * blockDim.x + threadIdx.x; i < total; i += num_blocks * blockDim.x) {
+        const unsigned b = i / chw_v;
+        const long long o = (long long)(i - b * chw_v) * VEC;
         float r[VEC];
-        float *dst = k.y + b * k.y_bs + o;
+        float *dst = k.y + (long long)b * k.y_bs + o;
         int first = 0;
         if (k.accumulate) {
 #pragma unroll
             for (int e = 0; e < VEC; e++) r[e] = dst[e];
         } else {
-            const float *s0 = a.src[0] + b * a.src_bstride[0] + o;
+            const float *s0 = a.src[0] + (long long)b * a.src_bstride[0] + o;
             if (VEC == 4) {
                 const pw_floatx4 v = *reinterpret_cast<const pw_floatx4 *>(s0);
 #pragma unroll
@@ -194,7 +198,7 @@ __device__ __forceinline__ void nary_body(const NaryKernelArgs &k, int block, in
             first = 1;
         }
         for (int j = first; j < a.count; j++) {
-            const float *s = a.src[j] + b * a.src_bstride[j] + o;
+            const float *s = a.src[j] + (long long)b * a.src_bstride[j] + o;
             float t[VEC];
             if (VEC == 4) {
                 const pw_floatx4 v = *reinterpret_cast<const pw_floatx4 *>(s);

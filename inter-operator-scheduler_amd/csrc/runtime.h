@@ -45,12 +45,17 @@ public:
     // Kernel configuration for a matrix-path convolution: the measured best when autotuning is on (cached
     // per problem signature for the life of the process, and in the file named by IOS_TUNE_CACHE when set),
     // else the closed-form model; the testing overrides win over both.
-    ConvLaunch choose_launch(const ConvProblem &p);
-    std::map<std::string, ConvLaunch> tuned;
+    // `share` = number of groups running concurrently with this convolution (1 = alone on the device).
+    ConvLaunch choose_launch(const ConvProblem &p, int share);
+    static constexpr int kShareClasses = 4;   // footprint budgets 1, 1/2, 1/4, 1/8 of the device
+    struct TunedConv {
+        ConvLaunch best[kShareClasses];
+    };
+    std::map<std::string, TunedConv> tuned;
 
 private:
     DeviceContext();
-    ConvLaunch tune_conv(const ConvProblem &p);
+    TunedConv tune_conv(const ConvProblem &p);
     float *tuning_buffer(int which, size_t floats);
     void load_tune_cache();
     float *tune_buf_[4] = {nullptr, nullptr, nullptr, nullptr};

@@ -66,21 +66,27 @@ static std::string conv_signature(const ConvProblem &p) {
 void DeviceContext::load_tune_cache() {
     FILE *f = fopen(tune_cache_path_.c_str(), "r");
     if (f == nullptr) return;
-    int v[12], variant, split;
-    char name[128];
-    // line: 12 problem integers, variant name, split_k
-    while (fscanf(f, "%d %d %d %d %d %d %d %d %d %d %d %d %127s %d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5], &v[6], &v[7], &v[8],
-                  &v[9], &v[10], &v[11], name, &split) == 14) {
-        variant = -1;
-        for (int i = 0; i < conv_num_variants(); i++)
-            if (strcmp(conv_variant(i).name, name) == 0) variant = i;
-        if (variant < 0 || split < 1) continue;
+    int v[12];
+    // line: 12 problem integers, then kShareClasses pairs (variant name, split_k)
+    while (true) {
+        bool ok = true;
+        for (int i = 0; i < 12 && ok; i++) ok = fscanf(f, "%d", &v[i]) == 1;
+        TunedConv entry;
+        for (int c = 0; c < kShareClasses && ok; c++) {
+            char name[128];
+            int split = 0;
+            ok = fscanf(f, "%127s %d", name, &split) == 2 && split >= 1;
+            int variant = -1;
+            for (int i = 0; ok && i < conv_num_variants(); i++)
+                if (strcmp(conv_variant(i).name, name) == 0) variant = i;
+            ok = ok && variant >= 0;
+            entry.best[c].variant = variant;
+            entry.best[c].split_k = split;
+        }
+        if (!ok) break;
         std::ostringstream os;
         for (int i = 0; i < 12; i++) os << (i ? " " : "") << v[i];
-        ConvLaunch l;
-        l.variant = variant;
-        l.split_k = split;
-        tuned[os.str()] = l;
+        tuned[os.str()] = entry;
     }
     fclose(f);
 }
@@ -100,7 +106,7 @@ float *DeviceContext::tuning_buffer(int which, size_t floats) {
     return tune_buf_[which];
 }
 
-ConvLaunch DeviceContext::tune_conv(const ConvProblem &p) {
+DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     // Like the reference's exhaustive algorithm search on first sight of a shape: run every kernel
     // configuration on scratch tensors of the real shape and keep the fastest.
     static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
@@ -116,8 +122,16 @@ ConvLaunch DeviceContext::tune_conv(const ConvProblem &p) {
     hipEvent_t start, stop;
     IOS_HIP(hipEventCreate(&start));
     IOS_HIP(hipEventCreate(&stop));
-    ConvLaunch best = conv_pick_launch(p, num_cus_);
-    float best_ms = 1e30f;
+    // one winner per footprint budget: the whole device, a half, a quarter, an eighth (threads in flight);
+    // a convolution that shares its stage with other groups uses the winner of the matching budget
+    const double capacity = (double)num_cus_ * 2048.0;
+    TunedConv result;
+    float best_ms[kShareClasses];
+    for (int c = 0; c < kShareClasses; c++) {
+        result.best[c] = conv_pick_launch(p, std::max(1, num_cus_ >> c));
+        best_ms[c] = 1e30f;
+    }
+    float fastest = 1e30f;
     for (int v = 0; v < conv_num_variants(); v++) {
         const ConvVariant &cv = conv_variant(v);
         // tiles more than twice as tall / wide as the problem only waste lanes
@@ -142,34 +156,48 @@ ConvLaunch DeviceContext::tune_conv(const ConvProblem &p) {
             float ms = 0.f;
             IOS_HIP(hipEventElapsedTime(&ms, start, stop));
             ms /= reps;
-            if (ms < best_ms) {
-                best_ms = ms;
-                best = l;
+            const double footprint = (double)cv.threads() * ((p.OCg() + cv.BM - 1) / cv.BM) * (double)((p.Npix() + cv.BN - 1) / cv.BN) *
+                                     p.groups * effective;
+            for (int c = 0; c < kShareClasses; c++) {
+                // class 0 is unconstrained; the others accept kernels that fit their share of the device
+                if (c > 0 && footprint > capacity / (1 << c)) continue;
+                if (ms < best_ms[c]) {
+                    best_ms[c] = ms;
+                    result.best[c] = l;
+                }
             }
-            if (ms > 3.f * best_ms) break;   // more slices only add reduction work from here on
+            fastest = std::min(fastest, ms);
+            if (ms > 3.f * fastest) break;   // more slices only add reduction work from here on
         }
     }
     IOS_HIP(hipEventDestroy(start));
     IOS_HIP(hipEventDestroy(stop));
+    // a budget nobody fits falls back to the next larger one
+    for (int c = 1; c < kShareClasses; c++)
+        if (best_ms[c] > 1e29f) result.best[c] = result.best[c - 1];
     if (!tune_cache_path_.empty()) {
         FILE *f = fopen(tune_cache_path_.c_str(), "a");
         if (f != nullptr) {
-            fprintf(f, "%s %s %d\n", conv_signature(p).c_str(), conv_variant(best.variant).name, best.split_k);
+            fprintf(f, "%s", conv_signature(p).c_str());
+            for (int c = 0; c < kShareClasses; c++) fprintf(f, " %s %d", conv_variant(result.best[c].variant).name, result.best[c].split_k);
+            fprintf(f, "\n");
             fclose(f);
         }
     }
-    return best;
+    return result;
 }
 
-ConvLaunch DeviceContext::choose_launch(const ConvProblem &p) {
+ConvLaunch DeviceContext::choose_launch(const ConvProblem &p, int share) {
+    int cls = 0;
+    while (cls + 1 < kShareClasses && (1 << (cls + 1)) <= share) cls++;   // floor(log2(share)), capped
     ConvLaunch launch;
     if (autotune_) {
         const std::string key = conv_signature(p);
         auto it = tuned.find(key);
         if (it == tuned.end()) it = tuned.emplace(key, tune_conv(p)).first;
-        launch = it->second;
+        launch = it->second.best[cls];
     } else {
-        launch = conv_pick_launch(p, num_cus_);
+        launch = conv_pick_launch(p, std::max(1, num_cus_ >> cls));
     }
     if (forced_variant_ >= 0) launch.variant = forced_variant_;
     if (forced_split_k_ > 0) launch.split_k = forced_split_k_;

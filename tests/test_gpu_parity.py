@@ -1,7 +1,9 @@
 """
 GPU parity: the HIP runtime, called through its C ABI, against the CPU oracle on the same seeded inputs.
-Tolerance for fp32: |got - want| <= 1e-4 + 1e-3 * |want| (abs 1e-4, rel 1e-3).
-Schedule changes must not change results at all (bit-identical outputs).
+Tolerance for fp32: |got - want| <= atol + 1e-3 * |want| with atol = 1e-4 * max(1, max|want|): rel 1e-3 / abs 1e-4,
+the absolute part taken relative to the tensor's scale because the seeded He-normal networks without batch norm
+(RandWire, NASNet) reach activations of 1e4 and more, where single fp32 roundings already exceed 1e-4.
+With the kernel configuration pinned, schedule and executor changes must not change results at all.
 """
 import numpy as np
 import pytest
@@ -18,7 +20,8 @@ RTOL, ATOL = 1e-3, 1e-4
 
 def assert_close(got, want, what=''):
     err = np.abs(got.astype(np.float64) - want.astype(np.float64))
-    bound = ATOL + RTOL * np.abs(want.astype(np.float64))
+    scale = max(1.0, float(np.abs(want).max())) if want.size else 1.0
+    bound = ATOL * scale + RTOL * np.abs(want.astype(np.float64))
     bad = err > bound
     assert not bad.any(), (f'{what}: {bad.sum()} of {bad.size} elements out of tolerance, max abs err '
                            f'{err.max():.3e} at {np.unravel_index(err.argmax(), err.shape)}, '
@@ -231,7 +234,12 @@ def model_cases():
 
 
 @pytest.mark.parametrize('name,make,batch', model_cases(), ids=[c[0] for c in model_cases()])
-def test_network_matches_oracle_and_schedules_agree_bitwise(name, make, batch):
+def test_network_matches_oracle_under_every_schedule_and_executor(name, make, batch):
+    """
+    Outputs match the CPU oracle within tolerance for the sequential, greedy and dp_parallel schedules under
+    every executor.  With the kernel configuration pinned (it otherwise depends on how many groups share a
+    stage, which changes the summation order) all schedules and executors agree bit for bit.
+    """
     graph = make()
     graph.sequential_schedule()
     x = np.random.default_rng(1).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
@@ -249,31 +257,39 @@ def test_network_matches_oracle_and_schedules_agree_bitwise(name, make, batch):
     assert_close(got, want, name)
     assert np.isfinite(got).all() and np.abs(got).max() > 0
 
-    graph.greedy_schedule(4)
-    greedy = rt.graph_inference(graph, batch, x)
-    np.testing.assert_array_equal(greedy, got)
-
     big = name.startswith(('randwire', 'nasnet'))
+    greedy = make()
+    greedy.greedy_schedule(4 if big else 8)
     if big:     # keep the pure-Python search short: small consecutive parts instead of whole cells
         for block in graph.blocks:
             block.parts = None
     optimized = ios.optimize(graph, batch, ios.AnalyticCostModel(), 'dp_parallel', max_group_size=2,
                              max_num_groups=4 if big else 8, max_part_size=10 if big else 100, compute_weight=True)
     assert any(len(stage) > 1 for block in optimized.blocks for stage in block.stages)
-    parallel = rt.graph_inference(optimized, batch, x)
-    np.testing.assert_array_equal(parallel, got)
 
-    for executor in ('graph', 'fused', 'fused_graph'):
-        rt.set_option('executor', executor)
-        with rt.Session(optimized, batch) as session:
-            session.load_weights()
-            session.set_input(x)
-            for _ in range(3):      # replays (of the captured graph) with host work in between
-                session.run()
-                np.testing.assert_array_equal(session.output(), got, err_msg=executor)
-        if not big:
-            graph.greedy_schedule(8)
-            np.testing.assert_array_equal(rt.graph_inference(graph, batch, x), got, err_msg=executor + ' greedy')
+    def run_all(pinned):
+        outs = {}
+        for executor in ('streams', 'graph', 'fused', 'fused_graph'):
+            rt.set_option('executor', executor)
+            for label, g in (('sequential', graph), ('greedy', greedy), ('dp_parallel', optimized)):
+                if label == 'sequential' and executor != 'streams':
+                    continue
+                with rt.Session(g, batch) as session:
+                    session.load_weights()
+                    session.set_input(x)
+                    for _ in range(2):      # the second pass replays the captured graph
+                        session.run()
+                    outs[(executor, label)] = session.output()
+                assert_close(outs[(executor, label)], want, f'{name} {executor} {label} pinned={pinned}')
+        return outs
+
+    run_all(pinned=False)
+    rt.set_option('conv_variant', 7)
+    rt.set_option('conv_split_k', 2)
+    outs = run_all(pinned=True)
+    first = outs[('streams', 'sequential')]
+    for key, value in outs.items():
+        np.testing.assert_array_equal(value, first, err_msg=str(key))
 
 
 def test_merged_convolutions_match_unmerged():
