@@ -3,7 +3,10 @@ Benchmark of the north-star path: Inception-v3 at batch 1 under the dp_parallel 
 dynamic-programming search with on-device stage measurements, on one MI355X.
 
 A step is one forward pass over one synthetic batch (weights and input already resident in HBM).  Prints one
-JSON line; see DESIGN.md for the definitions behind `roofline` and `cpu_baseline`.
+JSON line; DESIGN.md section 5 defines `roofline` and `cpu_baseline`.
+
+Probe modes for the profiler (`--probe copy`, `--probe pass`) run a fixed small workload and print what the
+counters should be compared with; they are used by the commands recorded under profiles/.
 """
 import argparse
 import json
@@ -20,17 +23,94 @@ PEAK_FP32_MATRIX_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
 
+def op_bound_ms(op):
+    return max(op['flops'] / (PEAK_FP32_MATRIX_TFLOPS * 1e12), op['bytes'] / (PEAK_HBM_GBS * 1e9)) * 1e3
+
+
 def network_roofline_ms(ops, parallel):
     """Sum over ops (or over stages of the slowest group) of max(flops / peak, bytes / bandwidth)."""
-    def bound(op):
-        return max(op['flops'] / (PEAK_FP32_MATRIX_TFLOPS * 1e12), op['bytes'] / (PEAK_HBM_GBS * 1e9)) * 1e3
     if not parallel:
-        return sum(bound(op) for op in ops)
+        return sum(op_bound_ms(op) for op in ops)
     stages = {}
     for op in ops:
         stages.setdefault(op['stage'], {}).setdefault(op['group'], 0.0)
-        stages[op['stage']][op['group']] += bound(op)
+        stages[op['stage']][op['group']] += op_bound_ms(op)
     return sum(max(groups.values()) for groups in stages.values())
+
+
+def timed_latency(rt, np, graph, batch, x, steps, warmup):
+    """Wall-clock ms per synchronised forward pass, event-timed latencies (reference protocol) and the output."""
+    with rt.Session(graph, batch) as session:
+        session.load_weights()
+        session.set_input(x)
+        for _ in range(warmup):
+            session.run()
+        t = time.perf_counter()
+        for _ in range(steps):
+            session.run()
+        wall = (time.perf_counter() - t) / steps * 1e3
+        events = session.measure(warmup=2, number=6, repeat=6)
+        return {'wall': wall, 'events_mean': float(np.mean(events)), 'events_min': float(np.min(events)),
+                'events_std': float(np.std(events))}, session.output()
+
+
+def conv_roofline(rt, graph, batch, x):
+    """Per-kernel HIP-event timing of one pass; returns (ops, ms per op, conv summary, memory-bound GB/s)."""
+    with rt.Session(graph, batch) as session:
+        session.load_weights()
+        session.set_input(x)
+        ops = session.describe()
+        op_ms = session.profile_ops(warmup=3, repeat=20)
+    conv = [(op, ms) for op, ms in zip(ops, op_ms) if op['kind'] == 'conv_mfma']
+    flops = sum(op['flops'] for op, _ in conv)
+    ms = sum(t for _, t in conv)
+    mem = [(op, t) for op, t in zip(ops, op_ms) if op['kind'] in ('pool', 'global_pool', 'nary', 'unary', 'conv_depthwise')]
+    mem_gbs = (sum(op['bytes'] for op, _ in mem) / (sum(t for _, t in mem) * 1e-3) / 1e9) if mem else None
+    achieved = flops / (ms * 1e-3) / 1e12
+    summary = {'bound': 'mfma', 'kernel': f'conv_kernel<...> ({len(conv)} convolution launches of one pass)',
+               'achieved': achieved, 'peak': PEAK_FP32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
+               'frac': achieved / PEAK_FP32_MATRIX_TFLOPS, 'traffic': None,
+               'flops_per_pass': flops, 'kernel_ms_per_pass': ms, 'launches': len(conv)}
+    return ops, op_ms, summary, mem_gbs
+
+
+def probe(args, np, ios, rt):
+    """Small fixed workloads for counter collection."""
+    rt.set_option('autotune', 1)
+    if args.probe == 'copy':
+        # y = relu(x) on 8 x 256 x 112 x 112: reads and writes 102,760,448 bytes per launch
+        ios.reset_name()
+        v = ios.placeholder((256, 112, 112))
+        block = ios.Block(v.node)
+        ios.relu(block, [[v]], is_exit=True)
+        graph = ios.Graph('copy', v.node, [block])
+        graph.sequential_schedule()
+        x = np.random.default_rng(0).standard_normal((8, 256, 112, 112)).astype(np.float32)
+        with rt.Session(graph, 8) as session:
+            session.set_input(x)
+            for _ in range(5):
+                session.run()
+            ms = session.profile_ops(1, 10)[0]
+        nbytes = x.nbytes
+        print(json.dumps({'probe': 'copy', 'kernel': 'nary_kernel', 'launches': 16, 'read_bytes_per_launch': nbytes,
+                          'write_bytes_per_launch': nbytes, 'ms_per_launch': ms,
+                          'gbs': 2 * nbytes / (ms * 1e-3) / 1e9}))
+        return
+    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    graph.sequential_schedule()
+    x = np.random.default_rng(1).standard_normal((args.batch, 3, 299, 299)).astype(np.float32)
+    rt.set_option('executor', 'streams')
+    with rt.Session(graph, args.batch) as session:
+        session.load_weights()
+        session.set_input(x)
+        for _ in range(3):
+            session.run()
+        ops = session.describe()
+    conv = [op for op in ops if op['kind'] == 'conv_mfma']
+    print(json.dumps({'probe': 'pass', 'batch': args.batch, 'passes': 3, 'schedule': 'sequential',
+                      'conv_launches_per_pass': len(conv),
+                      'conv_algorithmic_bytes_per_pass': sum(op['bytes'] for op in conv),
+                      'conv_flops_per_pass': sum(op['flops'] for op in conv)}))
 
 
 def main():
@@ -43,8 +123,13 @@ def main():
                         choices=['streams', 'graph', 'fused', 'fused_graph'])
     parser.add_argument('--search-executor', default='fused', choices=['streams', 'fused'],
                         help='executor under which the schedule search measures candidate stages')
-    parser.add_argument('--sweep', action='store_true', help='also time batch 16 and 64 with the same schedule')
+    parser.add_argument('--search', default='measured', choices=['measured', 'analytic'],
+                        help="cost model of the schedule search: on-device stage measurements (default) or the "
+                             "closed-form model (no device probes; keeps profiler traces small)")
+    parser.add_argument('--no-sweep', action='store_true', help='skip the batch 16 / 64 sweep')
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    parser.add_argument('--no-configs', action='store_true', help='skip the other four configuration networks')
+    parser.add_argument('--probe', choices=['copy', 'pass'], help='run a profiler probe instead of the benchmark')
     args = parser.parse_args()
     if args.gpus != 1:
         print('bench.py: this runtime is a single-GPU path; run with --gpus 1', file=sys.stderr)
@@ -53,6 +138,10 @@ def main():
     import numpy as np
     import ios
     from ios.contrib import ios_runtime as rt
+
+    if args.probe:
+        probe(args, np, ios, rt)
+        return
 
     device = rt.device_info()
     batch = args.batch
@@ -63,54 +152,28 @@ def main():
     rt.set_option('autotune', 1)        # measure kernel configurations on first sight of a shape
     rt.set_option('executor', args.search_executor)
     t0 = time.time()
-    optimized = ios.optimize(graph, batch_size=batch, opt_type='dp_parallel', compute_weight=True,
+    cost_model = ios.IOSCostModel() if args.search == 'measured' else ios.AnalyticCostModel()
+    optimized = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
                              warmup=2, number=6, repeat=3)
     search_s = time.time() - t0
     graph.sequential_schedule()
 
     rt.set_option('executor', args.executor)
+    seq, seq_out = timed_latency(rt, np, graph, batch, x, args.steps, args.warmup)
+    opt, opt_out = timed_latency(rt, np, optimized, batch, x, args.steps, args.warmup)
 
-    def timed_latency(g, b, xin, steps, warmup):
-        with rt.Session(g, b) as session:
-            session.load_weights()
-            session.set_input(xin)
-            for _ in range(warmup):
-                session.run()
-            t = time.perf_counter()
-            for _ in range(steps):
-                session.run()
-            wall = (time.perf_counter() - t) / steps * 1e3
-            events = session.measure(warmup=2, number=6, repeat=6)
-            out = session.output()
-            return wall, float(np.mean(events)), float(np.min(events)), float(np.std(events)), out
-
-    seq_wall, seq_ev, seq_min, seq_std, seq_out = timed_latency(graph, batch, x, args.steps, args.warmup)
-    opt_wall, opt_ev, opt_min, opt_std, opt_out = timed_latency(optimized, batch, x, args.steps, args.warmup)
-    schedule_diff = float(np.abs(seq_out - opt_out).max())
-
-    # per-kernel timing with HIP events on the launch stream, and the roofline of the dominant kernel
-    with rt.Session(optimized, batch) as session:
-        session.load_weights()
-        session.set_input(x)
-        ops = session.describe()
-        op_ms = session.profile_ops(warmup=3, repeat=20)
-    conv = [(op, ms) for op, ms in zip(ops, op_ms) if op['kind'] == 'conv_mfma']
-    conv_flops = sum(op['flops'] for op, _ in conv)
-    conv_ms = sum(ms for _, ms in conv)
-    achieved = conv_flops / (conv_ms * 1e-3) / 1e12
-    mem = [(op, ms) for op, ms in zip(ops, op_ms) if op['kind'] in ('pool', 'global_pool', 'nary', 'unary', 'conv_depthwise')]
-    mem_gbs = (sum(op['bytes'] for op, _ in mem) / (sum(ms for _, ms in mem) * 1e-3) / 1e9) if mem else None
+    ops, op_ms, roofline, mem_gbs = conv_roofline(rt, optimized, batch, x)
     roof_seq = network_roofline_ms(ops, parallel=False)
     roof_par = network_roofline_ms(ops, parallel=True)
 
     result = {
         'metric': 'batch-1 latency (ms) + images/s, Inception-v3 IOS dp_parallel schedule',
-        'value': batch / (opt_wall * 1e-3),
+        'value': batch / (opt['wall'] * 1e-3),
         'unit': 'images/s',
         'n_gpus': 1,
         'steps': args.steps,
         'warmup': args.warmup,
-        'ms_per_step': opt_wall,
+        'ms_per_step': opt['wall'],
         'higher_is_better': True,
         'scaling': 'weak',
         'vs_baseline': None,
@@ -118,32 +181,60 @@ def main():
         'data': 'synthetic (N(0,1) input, seeded He-normal weights, zero bias)',
         'config': {'workload': f'inception_v3 3x299x299 batch {batch}, dp_parallel schedule (r=3, s=8), {args.executor} executor',
                    'global_batch': batch},
-        'latency_ms': {'dp_parallel_wall': opt_wall, 'dp_parallel_events_mean': opt_ev, 'dp_parallel_events_min': opt_min,
-                       'dp_parallel_events_std': opt_std, 'sequential_wall': seq_wall, 'sequential_events_mean': seq_ev,
-                       'sequential_events_min': seq_min, 'sequential_events_std': seq_std},
-        'speedup_vs_own_sequential': seq_wall / opt_wall,
-        'max_abs_diff_between_schedules': schedule_diff,
+        'latency_ms': {'dp_parallel': opt, 'sequential': seq},
+        'speedup_vs_own_sequential': seq['wall'] / opt['wall'],
+        'max_abs_diff_between_schedules': float(np.abs(seq_out - opt_out).max()),
         'search_seconds': search_s,
         'num_stages': sum(len(b.stages) for b in optimized.blocks),
         'network_roofline_ms': {'sequential': roof_seq, 'critical_path': roof_par,
-                                'fraction_achieved': roof_par / opt_wall},
-        'roofline': {'bound': 'mfma', 'kernel': 'conv_mfma_kernel (all 94 convolution launches of one pass)',
-                     'achieved': achieved, 'peak': PEAK_FP32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': achieved / PEAK_FP32_MATRIX_TFLOPS, 'traffic': None,
-                     'flops_per_pass': conv_flops, 'kernel_ms_per_pass': conv_ms},
+                                'fraction_of_critical_path_roofline': roof_par / opt['wall'],
+                                'fraction_of_sequential_roofline': roof_seq / opt['wall']},
+        'roofline': roofline,
         'memory_bound_ops_gbs': mem_gbs,
-        'device': device,
+        'device': {k: device[k] for k in ('name', 'arch', 'compute_units')},
     }
 
-    if args.sweep:
+    if not args.no_sweep:
         sweep = {}
         for b in (16, 64):
             xb = np.random.default_rng(1).standard_normal((b, 3, 299, 299)).astype(np.float32)
             steps = max(10, args.steps // (b * 2))
-            w_seq = timed_latency(graph, b, xb, steps, 3)[0]
-            w_opt = timed_latency(optimized, b, xb, steps, 3)[0]
-            sweep[str(b)] = {'sequential_ms': w_seq, 'dp_parallel_ms': w_opt, 'images_per_s': b / (min(w_seq, w_opt) * 1e-3)}
+            s_seq, out_seq = timed_latency(rt, np, graph, b, xb, steps, 3)
+            s_opt, out_opt = timed_latency(rt, np, optimized, b, xb, steps, 3)
+            _, _, roof_b, _ = conv_roofline(rt, graph, b, xb)
+            ops_b = rt.plan_describe(graph, b)
+            best = min(s_seq['wall'], s_opt['wall'])
+            sweep[str(b)] = {'sequential_ms': s_seq['wall'], 'dp_parallel_batch1_schedule_ms': s_opt['wall'],
+                             'images_per_s': b / (best * 1e-3),
+                             'network_roofline_ms': network_roofline_ms(ops_b, parallel=False),
+                             'fraction_of_network_roofline': network_roofline_ms(ops_b, parallel=False) / best,
+                             'conv_tflops': roof_b['achieved'], 'conv_frac_of_fp32_matrix_peak': roof_b['frac']}
         result['batch_sweep'] = sweep
+
+    if not args.no_configs:
+        configs = {}
+        for name, make, search in (('sample_net', ios.models.sample_network, True),
+                                   ('squeezenet_1_1', ios.models.squeezenet_1_1, True),
+                                   ('randwire_small', ios.models.randwire_small, False),
+                                   ('nasnet_mobile', ios.models.nasnet_mobile, False)):
+            g = make(init_seed=0, init_scheme='he_normal')
+            xc = np.random.default_rng(1).standard_normal((1, *g.enter_node.output_shape)).astype(np.float32)
+            if search:
+                rt.set_option('executor', args.search_executor)
+                scheduled = ios.optimize(g, batch_size=1, opt_type='dp_parallel', compute_weight=True, warmup=2, number=6, repeat=3)
+                label = 'dp_parallel'
+                rt.set_option('executor', args.executor)
+            else:   # the pure-Python search takes tens of minutes on these graphs: use the greedy schedule
+                scheduled = make(init_seed=0, init_scheme='he_normal')
+                scheduled.greedy_schedule(4)
+                label = 'greedy'
+            g.sequential_schedule()
+            c_seq, _ = timed_latency(rt, np, g, 1, xc, 100, 10)
+            c_par, _ = timed_latency(rt, np, scheduled, 1, xc, 100, 10)
+            ops_c = rt.plan_describe(g, 1)
+            configs[name] = {'sequential_ms': c_seq['wall'], f'{label}_ms': c_par['wall'],
+                             'network_roofline_ms': network_roofline_ms(ops_c, parallel=False)}
+        result['other_configs_batch1'] = configs
 
     if not args.no_cpu:
         import torch

@@ -3,7 +3,7 @@
 set -euo pipefail
 cd "$(dirname "$0")"
 mkdir -p build
-FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclang -packed-fp32-ops -Wno-unused-result"
+FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclang -packed-fp32-ops -mllvm -amdgpu-mfma-vgpr-form=1 -Wno-unused-result"
 pids=()
 for src in conv_mfma.hip pointwise.hip fused.hip runtime.hip c_api.hip; do
     hipcc $FLAGS -c "$src" -o "build/${src%.hip}.o" &

@@ -46,7 +46,25 @@ struct ConvKernelArgs {
     int act, pre_relu;
     int split_k, k_chunk;
     int tiles_m, tiles_n;
+    int weights_major;   // 1: consecutive tiles share filter rows (filters larger than the input), 0: share pixels
 };
+
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Tiles are renumbered so that an XCD
+// receives a contiguous range of them, and the range runs along the operand that is cheaper to duplicate: the
+// more expensive operand (filters at batch 1, activations at large batch) is then fetched into one L2 only.
+__device__ __forceinline__ void xcd_tile(const ConvKernelArgs &a, int block, int &tm, int &tn) {
+    const int total = a.tiles_m * a.tiles_n;
+    const int xcd = block & 7, slot = block >> 3;
+    const int q = total >> 3, r = total & 7;
+    const int t = xcd < r ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
+    if (a.weights_major) {
+        tm = t / a.tiles_n;
+        tn = t - tm * a.tiles_n;
+    } else {
+        tn = t / a.tiles_m;
+        tm = t - tn * a.tiles_m;
+    }
+}
 
 __device__ __forceinline__ float apply_act(float v, int act) {
     switch (act) {
@@ -137,8 +155,8 @@ struct ConvTiled {
     const int wm = (wave / WN) % WM;
     const int wk = wave / (WN * WM);
 
-    const int tm = tile % a.tiles_m;
-    const int tn = tile / a.tiles_m;
+    int tm, tn;
+    xcd_tile(a, tile, tm, tn);
     const int m0 = tm * BM;
     const int n0 = tn * BN;
     const int k_begin = z * a.k_chunk;
@@ -390,8 +408,8 @@ struct ConvWsplit {
     const int wave = tid >> 6;
     const int lk = lane / MT;
     const int lc = lane % MT;
-    const int tm = tile % a.tiles_m;
-    const int tn = tile / a.tiles_m;
+    int tm, tn;
+    xcd_tile(a, tile, tm, tn);
     const int m0 = tm * BM;
     const int n0 = tn * BN;
 
@@ -514,26 +532,29 @@ struct ConvWsplit {
 
 // ---- kernel configurations ------------------------------------------------------------------------------------------
 // X(index, name, BM, BN, BK, WM, WN, WK, MT, PD) for the LDS-tiled kernel
-#define IOS_TILED_VARIANTS(X)                                  \
-    X(0, "m64n64k32_w2x2x1_t32", 64, 64, 32, 2, 2, 1, 32, 3)   \
+#define IOS_TILED_VARIANTS(X)                                    \
+    X(0, "m64n64k32_w2x2x1_t32", 64, 64, 32, 2, 2, 1, 32, 3)     \
     X(1, "m128n128k16_w2x2x1_t32", 128, 128, 16, 2, 2, 1, 32, 3) \
-    X(2, "m32n32k64_w1x1x4_t32", 32, 32, 64, 1, 1, 4, 32, 4)   \
-    X(3, "m64n32k32_w2x1x2_t32", 64, 32, 32, 2, 1, 2, 32, 4)   \
-    X(4, "m32n64k32_w1x2x2_t32", 32, 64, 32, 1, 2, 2, 32, 4)   \
-    X(5, "m128n64k16_w2x2x1_t32", 128, 64, 16, 2, 2, 1, 32, 3) \
-    X(6, "m64n16k64_w4x1x1_t16", 64, 16, 64, 4, 1, 1, 16, 3)   \
-    X(7, "m32n16k64_w2x1x2_t16", 32, 16, 64, 2, 1, 2, 16, 4)   \
-    X(8, "m16n16k128_w1x1x4_t16", 16, 16, 128, 1, 1, 4, 16, 3)
+    X(2, "m32n32k64_w1x1x4_t32", 32, 32, 64, 1, 1, 4, 32, 4)     \
+    X(3, "m64n32k32_w2x1x2_t32", 64, 32, 32, 2, 1, 2, 32, 4)     \
+    X(4, "m32n64k32_w1x2x2_t32", 32, 64, 32, 1, 2, 2, 32, 4)     \
+    X(5, "m128n64k16_w2x2x1_t32", 128, 64, 16, 2, 2, 1, 32, 3)   \
+    X(6, "m64n16k64_w4x1x1_t16", 64, 16, 64, 4, 1, 1, 16, 3)     \
+    X(7, "m32n16k64_w2x1x2_t16", 32, 16, 64, 2, 1, 2, 16, 4)     \
+    X(8, "m16n16k128_w1x1x4_t16", 16, 16, 128, 1, 1, 4, 16, 3)   \
+    X(9, "m64n128k16_w2x2x1_t32", 64, 128, 16, 2, 2, 1, 32, 3)   \
+    X(10, "m64n64k16_w2x2x1_t32", 64, 64, 16, 2, 2, 1, 32, 4)    \
+    X(11, "m32n128k16_w1x4x1_t32", 32, 128, 16, 1, 4, 1, 32, 4)
 // X(index, name, MT, TM, TN, NW, U) for the wave-split kernel
 #define IOS_WSPLIT_VARIANTS(X)                     \
-    X(9, "ws_m32n16_w16_t16", 16, 2, 1, 16, 4)     \
-    X(10, "ws_m16n16_w16_t16", 16, 1, 1, 16, 8)    \
-    X(11, "ws_m32n32_w16_t16", 16, 2, 2, 16, 4)    \
-    X(12, "ws_m64n16_w16_t16", 16, 4, 1, 16, 4)    \
-    X(13, "ws_m32n16_w8_t16", 16, 2, 1, 8, 4)      \
-    X(14, "ws_m32n16_w4_t16", 16, 2, 1, 4, 8)      \
-    X(15, "ws_m32n32_w16_t32", 32, 1, 1, 16, 8)    \
-    X(16, "ws_m16n32_w16_t16", 16, 1, 2, 16, 4)
-constexpr int kNumConvVariants = 17;
+    X(12, "ws_m32n16_w16_t16", 16, 2, 1, 16, 4)    \
+    X(13, "ws_m16n16_w16_t16", 16, 1, 1, 16, 8)    \
+    X(14, "ws_m32n32_w16_t16", 16, 2, 2, 16, 4)    \
+    X(15, "ws_m64n16_w16_t16", 16, 4, 1, 16, 4)    \
+    X(16, "ws_m32n16_w8_t16", 16, 2, 1, 8, 4)      \
+    X(17, "ws_m32n16_w4_t16", 16, 2, 1, 4, 8)      \
+    X(18, "ws_m32n32_w16_t32", 32, 1, 1, 16, 8)    \
+    X(19, "ws_m16n32_w16_t16", 16, 1, 2, 16, 4)
+constexpr int kNumConvVariants = 20;
 
 }  // namespace ios

@@ -70,7 +70,7 @@ ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus) {
     // split K, keeping at least two K tiles per slice.
     const long long M = p.OCg(), N = p.Npix();
     const long long want = 2LL * num_cus;
-    static const int by_size[] = {1, 5, 0, 3, 4, 2, 7};   // large to small tiles
+    static const int by_size[] = {1, 5, 9, 0, 3, 4, 2, 7};   // large to small tiles
     ConvLaunch best;
     for (int idx : by_size) {
         const ConvVariant &v = kVariants[idx].v;
@@ -132,6 +132,7 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     a.split_k = effective_split(p, l);
     a.tiles_m = ceil_div(p.OCg(), e.v.BM);
     a.tiles_n = ceil_div(p.Npix(), e.v.BN);
+    a.weights_major = (double)p.OC * p.K() > (double)p.B * p.IC * p.H * p.W ? 1 : 0;
     if (a.split_k > 1 && workspace == nullptr) throw std::runtime_error("conv: split-K launch without workspace");
     if (p.groups > 65535 || a.split_k > 65535) throw std::runtime_error("conv: grid too large");
     d.variant = l.variant;
