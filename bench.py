@@ -129,6 +129,7 @@ def main():
     parser.add_argument('--no-sweep', action='store_true', help='skip the batch 16 / 64 sweep')
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     parser.add_argument('--no-configs', action='store_true', help='skip the other four configuration networks')
+    parser.add_argument('--option', action='append', default=[], metavar='KEY=VALUE', help='extra runtime option (repeatable)')
     parser.add_argument('--probe', choices=['copy', 'pass'], help='run a profiler probe instead of the benchmark')
     args = parser.parse_args()
     if args.gpus != 1:
@@ -150,6 +151,9 @@ def main():
 
     # schedule search with measured stage latencies (not part of the timed steps)
     rt.set_option('autotune', 1)        # measure kernel configurations on first sight of a shape
+    for item in args.option:
+        key, _, value = item.partition('=')
+        rt.set_option(key, value)
     rt.set_option('executor', args.search_executor)
     t0 = time.time()
     cost_model = ios.IOSCostModel() if args.search == 'measured' else ios.AnalyticCostModel()

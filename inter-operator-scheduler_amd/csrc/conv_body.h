@@ -36,6 +36,7 @@ struct ConvKernelArgs {
     const float *bias;
     float *y;
     float *ws;
+    unsigned *counters;               // split-K tickets, one per (group, tile), zero between launches; null: two-kernel split-K
     int H, W, OH, OW, sh, sw, ph, pw;
     int KW, taps;                     // taps = KH * KW
     unsigned magic_icgp, magic_kw;    // floor(2^32 / d) + 1: exact quotients for dividends < 2^16
@@ -320,41 +321,97 @@ struct ConvTiled {
         }
     }
 
-    // ---- epilogue -------------------------------------------------------------------------------------------
-    if (a.split_k == 1) {
+    // ---- split-K ----------------------------------------------------------------------------------------------
+    if (a.split_k > 1) {
+        if (a.counters == nullptr) {
+            // two-kernel form: store this slice's partial tile; splitk_reduce_kernel adds the slices, bias and activation
+            float *wsz = a.ws + ((size_t)z * a.groups + g) * a.OCg * (size_t)a.Npix;
+            if (wk == 0) {
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const int nn = n0 + wn * WTN + j * MT + lc;
+                    if (nn >= a.Npix) continue;
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int v = 0; v < M::ACC; v++) {
+                            const int m = m0 + wm * WTM + i * MT + M::row(v, lane);
+                            if (m < a.OCg) wsz[(size_t)m * a.Npix + nn] = acc[i][j][v];
+                        }
+                }
+            }
+            return;
+        }
+        // one-kernel form: every slice stores its partial tile in accumulator layout ([element][thread], so a
+        // wavefront writes 256 contiguous bytes), then takes a ticket on the tile's counter; the block that
+        // draws the last ticket adds all slices in slice order (its own included, so the sum does not depend
+        // on which block came last) and runs the epilogue.  Partials and tickets move with device-scope
+        // atomics, which are coherent across the per-XCD L2s without cache-wide write-backs or invalidations;
+        // the wait on the outstanding stores before the barrier orders a block's partials before its ticket.
+        constexpr int T0 = 64 * WM * WN;
+        constexpr int E = TM * TN * M::ACC;
+        static_assert(T0 * E == BM * BN, "accumulator layout covers the tile");
+        const size_t tiles = (size_t)a.tiles_m * a.tiles_n;
+        float *slices = a.ws + (((size_t)g * tiles + tile) * a.split_k) * (size_t)(BM * BN);
+        if (wk == 0) {
+            float *mine = slices + (size_t)z * (BM * BN) + tid;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int v = 0; v < M::ACC; v++)
+                        __hip_atomic_store(mine + ((i * TN + j) * M::ACC + v) * T0, acc[i][j][v], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        int *last_flag = reinterpret_cast<int *>(smem);
+        if (tid == 0) {
+            unsigned *counter = a.counters + (size_t)g * tiles + tile;
+            const unsigned ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int last = ticket == (unsigned)a.split_k - 1u ? 1 : 0;
+            if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+            *last_flag = last;
+        }
+        __syncthreads();
+        if (*last_flag == 0) return;
         if (wk == 0) {
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const int nn = n0 + wn * WTN + j * MT + lc;
-                if (nn >= a.Npix) continue;
-                const int b = nn / a.OHW;
-                const int r = nn - b * a.OHW;
-                float *yb = a.y + (long long)b * a.y_bs + (long long)g * a.OCg * a.OHW + r;
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int v = 0; v < M::ACC; v++) acc[i][j][v] = 0.f;
+            for (int s = 0; s < a.split_k; s++) {
+                const float *theirs = slices + (size_t)s * (BM * BN) + tid;
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
-                    for (int v = 0; v < M::ACC; v++) {
-                        const int m = m0 + wm * WTM + i * MT + M::row(v, lane);
-                        if (m < a.OCg) yb[(long long)m * a.OHW] = apply_act(acc[i][j][v] + a.bias[g * a.OCg + m], a.act);
-                    }
+                    for (int j = 0; j < TN; j++)
+#pragma unroll
+                        for (int v = 0; v < M::ACC; v++)
+                            acc[i][j][v] += __hip_atomic_load(theirs + ((i * TN + j) * M::ACC + v) * T0, __ATOMIC_RELAXED,
+                                                              __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        return;
     }
 
-    // split-K: store this slice's partial tile; splitk_reduce_kernel adds the slices, bias and activation
-    float *wsz = a.ws + ((size_t)z * a.groups + g) * a.OCg * (size_t)a.Npix;
+    // ---- epilogue -------------------------------------------------------------------------------------------
     if (wk == 0) {
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int nn = n0 + wn * WTN + j * MT + lc;
             if (nn >= a.Npix) continue;
+            const int b = nn / a.OHW;
+            const int r = nn - b * a.OHW;
+            float *yb = a.y + (long long)b * a.y_bs + (long long)g * a.OCg * a.OHW + r;
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int v = 0; v < M::ACC; v++) {
                     const int m = m0 + wm * WTM + i * MT + M::row(v, lane);
-                    if (m < a.OCg) wsz[(size_t)m * a.Npix + nn] = acc[i][j][v];
+                    if (m < a.OCg) yb[(long long)m * a.OHW] = apply_act(acc[i][j][v] + a.bias[g * a.OCg + m], a.act);
                 }
         }
     }
@@ -544,17 +601,21 @@ struct ConvWsplit {
     X(8, "m16n16k128_w1x1x4_t16", 16, 16, 128, 1, 1, 4, 16, 3)   \
     X(9, "m64n128k16_w2x2x1_t32", 64, 128, 16, 2, 2, 1, 32, 3)   \
     X(10, "m64n64k16_w2x2x1_t32", 64, 64, 16, 2, 2, 1, 32, 4)    \
-    X(11, "m32n128k16_w1x4x1_t32", 32, 128, 16, 1, 4, 1, 32, 4)
+    X(11, "m32n128k16_w1x4x1_t32", 32, 128, 16, 1, 4, 1, 32, 4)  \
+    X(12, "m192n64k16_w2x2x1_t32", 192, 64, 16, 2, 2, 1, 32, 3)  \
+    X(13, "m96n128k16_w1x4x1_t32", 96, 128, 16, 1, 4, 1, 32, 3)  \
+    X(14, "m192n128k16_w2x2x1_t32", 192, 128, 16, 2, 2, 1, 32, 3) \
+    X(15, "m160n128k16_w1x4x1_t32", 160, 128, 16, 1, 4, 1, 32, 3)
 // X(index, name, MT, TM, TN, NW, U) for the wave-split kernel
 #define IOS_WSPLIT_VARIANTS(X)                     \
-    X(12, "ws_m32n16_w16_t16", 16, 2, 1, 16, 4)    \
-    X(13, "ws_m16n16_w16_t16", 16, 1, 1, 16, 8)    \
-    X(14, "ws_m32n32_w16_t16", 16, 2, 2, 16, 4)    \
-    X(15, "ws_m64n16_w16_t16", 16, 4, 1, 16, 4)    \
-    X(16, "ws_m32n16_w8_t16", 16, 2, 1, 8, 4)      \
-    X(17, "ws_m32n16_w4_t16", 16, 2, 1, 4, 8)      \
-    X(18, "ws_m32n32_w16_t32", 32, 1, 1, 16, 8)    \
-    X(19, "ws_m16n32_w16_t16", 16, 1, 2, 16, 4)
-constexpr int kNumConvVariants = 20;
+    X(16, "ws_m32n16_w16_t16", 16, 2, 1, 16, 4)    \
+    X(17, "ws_m16n16_w16_t16", 16, 1, 1, 16, 8)    \
+    X(18, "ws_m32n32_w16_t16", 16, 2, 2, 16, 4)    \
+    X(19, "ws_m64n16_w16_t16", 16, 4, 1, 16, 4)    \
+    X(20, "ws_m32n16_w8_t16", 16, 2, 1, 8, 4)      \
+    X(21, "ws_m32n16_w4_t16", 16, 2, 1, 4, 8)      \
+    X(22, "ws_m32n32_w16_t32", 32, 1, 1, 16, 8)    \
+    X(23, "ws_m16n32_w16_t16", 16, 1, 2, 16, 4)
+constexpr int kNumConvVariants = 24;
 
 }  // namespace ios

@@ -61,7 +61,17 @@ static int effective_split(const ConvProblem &p, const ConvLaunch &l) {
 
 size_t conv_workspace_floats(const ConvProblem &p, const ConvLaunch &l) {
     const int s = effective_split(p, l);
-    return s > 1 ? (size_t)s * p.OC * (size_t)p.Npix() : 0;
+    if (s <= 1) return 0;
+    // two-kernel form: [slice][OC][pixels]; one-kernel form: [group][tile][slice][BM * BN]
+    const ConvVariant &v = kVariants[l.variant].v;
+    const size_t padded = (size_t)p.groups * ceil_div(p.OCg(), v.BM) * (size_t)ceil_div(p.Npix(), v.BN) * v.BM * v.BN;
+    return (size_t)s * std::max((size_t)p.OC * (size_t)p.Npix(), padded);
+}
+
+size_t conv_counter_count(const ConvProblem &p, const ConvLaunch &l) {
+    if (effective_split(p, l) <= 1) return 0;
+    const ConvVariant &v = kVariants[l.variant].v;
+    return (size_t)p.groups * ceil_div(p.OCg(), v.BM) * (size_t)ceil_div(p.Npix(), v.BN);
 }
 
 ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus) {
@@ -99,7 +109,7 @@ bool conv_matrix_path_supported(const ConvProblem &p) {
 }
 
 ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
-                                const float *bias, const TensorView &y, float *workspace) {
+                                const float *bias, const TensorView &y, float *workspace, unsigned *counters) {
     if (l.variant < 0 || l.variant >= kNumVariants) throw std::runtime_error("conv: bad variant");
     const VariantEntry &e = kVariants[l.variant];
     if (x.C != p.IC || x.H != p.H || x.W != p.W || y.C != p.OC || y.H != p.OH || y.W != p.OW)
@@ -113,6 +123,7 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     a.bias = bias;
     a.y = y.ptr;
     a.ws = workspace;
+    a.counters = counters;
     a.H = p.H; a.W = p.W; a.OH = p.OH; a.OW = p.OW;
     a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw;
     a.KW = p.KW; a.taps = p.KH * p.KW;
@@ -141,7 +152,8 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     d.tiles = a.tiles_m * a.tiles_n;
     d.groups = p.groups;
     d.slices = a.split_k;
-    d.has_reduce = a.split_k > 1;
+    if (a.split_k <= 1) a.counters = nullptr;
+    d.has_reduce = a.split_k > 1 && a.counters == nullptr;
     d.reduce_blocks = 0;
     if (d.has_reduce) {
         ReduceArgs &r = d.reduce;
@@ -161,8 +173,8 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
 }
 
 void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
-                      const float *bias, const TensorView &y, float *workspace, hipStream_t stream) {
-    const ConvDispatch d = make_conv_dispatch(p, l, x, packed, bias, y, workspace);
+                      const float *bias, const TensorView &y, float *workspace, unsigned *counters, hipStream_t stream) {
+    const ConvDispatch d = make_conv_dispatch(p, l, x, packed, bias, y, workspace, counters);
     const VariantEntry &e = kVariants[d.variant];
     const dim3 grid((unsigned)d.tiles, (unsigned)d.groups, (unsigned)d.slices);
     hipLaunchKernelGGL(e.kernel, grid, dim3(d.threads), d.smem_bytes, stream, d.args);

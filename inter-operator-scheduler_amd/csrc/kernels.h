@@ -57,8 +57,11 @@ struct ConvLaunch {
     int split_k = 1;  // number of grid slices along K; > 1 needs workspace
 };
 
-// Floats of workspace a launch configuration needs (split_k partial outputs).
+// Floats of workspace a launch configuration needs (split_k partial outputs; large enough for both split-K forms).
 size_t conv_workspace_floats(const ConvProblem &p, const ConvLaunch &l);
+// Ticket counters the one-kernel split-K form needs: one unsigned per (group, output tile), zero before the
+// first launch (the kernel leaves them zero); 0 when the configuration does not split K.
+size_t conv_counter_count(const ConvProblem &p, const ConvLaunch &l);
 // The matrix path indexes packed filter rows with 16 bits and pixels / input offsets with 31 bits.
 bool conv_matrix_path_supported(const ConvProblem &p);
 
@@ -72,9 +75,11 @@ size_t conv_packed_floats_max(const ConvProblem &p);   // over all configuration
 void launch_pack_filters(const ConvProblem &p, const ConvLaunch &l, const float *w, float *packed, hipStream_t stream);
 
 // y = act(conv(x, w) + bias).  `packed` comes from launch_pack_filters.  `workspace` holds the split_k
-// partial outputs (conv_workspace_floats); with split_k > 1 a second kernel reduces them on the same stream.
+// partial outputs (conv_workspace_floats).  With split_k > 1 and `counters` (conv_counter_count) the block that
+// finishes a tile last adds the slices inside the kernel; without counters a second kernel adds them on the
+// same stream.  Both forms add in slice order.
 void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
-                      const float *bias, const TensorView &y, float *workspace, hipStream_t stream);
+                      const float *bias, const TensorView &y, float *workspace, unsigned *counters, hipStream_t stream);
 
 // Depth-wise convolution (groups == IC == OC), filters in their original [C][1][KH][KW] layout.
 void launch_dwconv(const ConvProblem &p, const TensorView &x, const float *w, const float *bias,

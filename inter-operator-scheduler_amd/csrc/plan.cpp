@@ -603,6 +603,8 @@ private:
             conv.packed_off = reserve(conv_packed_floats(conv.problem, conv.launch));
             conv.ws_floats = conv_workspace_floats(conv.problem, conv.launch);
             if (conv.ws_floats > 0) conv.ws_off = reserve(conv.ws_floats);
+            conv.ctr_count = conv_counter_count(conv.problem, conv.launch);
+            if (conv.ctr_count > 0) conv.ctr_off = reserve(conv.ctr_count);
         }
     }
 

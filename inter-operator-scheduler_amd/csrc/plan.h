@@ -45,6 +45,7 @@ struct PlanConv {
     size_t weight_off = 0, bias_off = 0;       // original layouts
     size_t packed_off = 0;                     // matrix path only
     size_t ws_off = 0, ws_floats = 0;          // split-K only
+    size_t ctr_off = 0, ctr_count = 0;         // split-K ticket counters (32-bit words at float offsets), zeroed at session setup
     ConvLaunch launch;
     bool matrix_path = false;
 };

@@ -31,8 +31,18 @@ PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorV
     a.x_bs = x.bstride;
     a.y_bs = y.bstride;
     a.p = p;
-    if (global) *blocks = blocks_for((long long)p.B * p.C, 4, 4096);
-    else *blocks = blocks_for((long long)p.B * p.C * p.OH * p.OW, 256, 8192);
+    a.strip_rows = 0;
+    if (global) {
+        *blocks = blocks_for((long long)p.B * p.C, 4, 4096);
+    } else if (p.KH == 3 && p.KW == 3 && (p.sh == 1 || p.sh == 2)) {
+        // one thread per strip of output rows; the longest strip that still leaves a million threads
+        int rows = kPoolStripRows;
+        while (rows > 1 && (long long)p.B * p.C * ((p.OH + rows - 1) / rows) * p.OW < (1LL << 20)) rows >>= 1;
+        a.strip_rows = rows;
+        *blocks = blocks_for((long long)p.B * p.C * ((p.OH + rows - 1) / rows) * p.OW, 256, 16384);
+    } else {
+        *blocks = blocks_for((long long)p.B * p.C * p.OH * p.OW, 256, 8192);
+    }
     return a;
 }
 

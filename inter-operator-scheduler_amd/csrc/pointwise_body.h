@@ -24,9 +24,10 @@ struct PoolArgs {
     float *y;
     long long x_bs, y_bs;
     PoolProblem p;
+    int strip_rows;   // 3 x 3 windows: output rows per thread (see pool3x3_body); 0 selects the generic body
 };
 
-__device__ __forceinline__ void pool_body(const PoolArgs &a, int block, int num_blocks) {
+__device__ __forceinline__ void pool_generic_body(const PoolArgs &a, int block, int num_blocks) {
     const PoolProblem &p = a.p;
     // 32-bit index arithmetic: the host side rejects tensors with 2^31 or more elements
     const unsigned plane = (unsigned)(p.OH * p.OW);
@@ -53,6 +54,71 @@ __device__ __forceinline__ void pool_body(const PoolArgs &a, int block, int num_
             }
         a.y[(long long)b * a.y_bs + o] = p.is_max ? best : sum * inv;
     }
+}
+
+// Most rows of outputs a thread of the 3 x 3 pooling body produces: a thread walks down one output column and keeps
+// the horizontal partial results of the input rows two consecutive windows share.  Small problems use shorter
+// strips (down to one row) so that the launch still fills the device.
+constexpr int kPoolStripRows = 8;
+
+// 3 x 3 windows, stride 1 or 2 in h (any stride in w).  Consecutive lanes take consecutive output columns, so the
+// three loads of an input row are contiguous (stride 1) or interleaved (stride 2) across a wavefront.  Per output
+// this reads 3 * (1 + 2 / 8) (stride 1) or 3 * (2 + 1 / 8) (stride 2) elements instead of 9.
+__device__ __forceinline__ void pool3x3_body(const PoolArgs &a, int block, int num_blocks) {
+    const PoolProblem &p = a.p;
+    const int R = a.strip_rows;
+    const unsigned strips = (unsigned)((p.OH + R - 1) / R);
+    const unsigned per_plane = strips * (unsigned)p.OW;
+    const unsigned total = per_plane * (unsigned)(p.C * p.B);
+    const bool is_max = p.is_max != 0;
+    const float neutral = is_max ? -INFINITY : 0.f;
+    for (unsigned i = block * blockDim.x + threadIdx.x; i < total; i += num_blocks * blockDim.x) {
+        const unsigned pc = i / per_plane;
+        const unsigned rest = i - pc * per_plane;
+        const unsigned strip = rest / (unsigned)p.OW;
+        const int ow = (int)(rest - strip * (unsigned)p.OW);
+        const unsigned b = pc / (unsigned)p.C;
+        const unsigned c = pc - b * (unsigned)p.C;
+        const float *xc = a.x + (long long)b * a.x_bs + (long long)c * p.H * p.W;
+        float *yc = a.y + (long long)b * a.y_bs + (long long)c * p.OH * p.OW + ow;
+        const int w0 = ow * p.sw - p.pw;
+        const bool c0 = (unsigned)w0 < (unsigned)p.W, c1 = (unsigned)(w0 + 1) < (unsigned)p.W, c2 = (unsigned)(w0 + 2) < (unsigned)p.W;
+        auto row = [&](int h) -> float {
+            if ((unsigned)h >= (unsigned)p.H) return neutral;
+            const float *xr = xc + h * p.W + w0;
+            const float v0 = c0 ? xr[0] : neutral;
+            const float v1 = c1 ? xr[1] : neutral;
+            const float v2 = c2 ? xr[2] : neutral;
+            return is_max ? fmaxf(fmaxf(v0, v1), v2) : (v0 + v1) + v2;
+        };
+        auto combine = [&](float r0, float r1, float r2) -> float {
+            return is_max ? fmaxf(fmaxf(r0, r1), r2) : ((r0 + r1) + r2) * (1.0f / 9.0f);
+        };
+        const int oh_begin = (int)strip * R;
+        const int oh_end = min(p.OH, oh_begin + R);
+        if (p.sh == 1) {
+            float r0 = row(oh_begin - p.ph), r1 = row(oh_begin - p.ph + 1);
+            for (int oh = oh_begin; oh < oh_end; oh++) {
+                const float r2 = row(oh - p.ph + 2);
+                yc[oh * p.OW] = combine(r0, r1, r2);
+                r0 = r1;
+                r1 = r2;
+            }
+        } else {
+            float r0 = row(oh_begin * 2 - p.ph);
+            for (int oh = oh_begin; oh < oh_end; oh++) {
+                const float r1 = row(oh * 2 - p.ph + 1);
+                const float r2 = row(oh * 2 - p.ph + 2);
+                yc[oh * p.OW] = combine(r0, r1, r2);
+                r0 = r2;
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ void pool_body(const PoolArgs &a, int block, int num_blocks) {
+    if (a.strip_rows > 0) pool3x3_body(a, block, num_blocks);
+    else pool_generic_body(a, block, num_blocks);
 }
 
 // window == whole map: one wavefront reduces one (image, channel) plane

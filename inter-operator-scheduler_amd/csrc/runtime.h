@@ -37,6 +37,9 @@ public:
     void set_option(const std::string &key, const std::string &value);
     ExecMode exec_mode() const { return exec_mode_; }
     bool autotune() const { return autotune_; }
+    // split-K partial sums are added by the last block of a tile inside the convolution kernel (true) or by a
+    // second kernel (false)
+    bool inline_reduce() const { return inline_reduce_; }
     // testing aid: force one kernel configuration for every matrix-path convolution (-1 / 0 = off)
     int forced_variant() const { return forced_variant_; }
     int forced_split_k() const { return forced_split_k_; }
@@ -57,6 +60,10 @@ private:
     DeviceContext();
     TunedConv tune_conv(const ConvProblem &p);
     float *tuning_buffer(int which, size_t floats);
+    unsigned *tuning_counters(size_t count);
+    unsigned *tune_counters_ = nullptr;
+    size_t tune_counter_count_ = 0;
+    bool inline_reduce_ = true;
     void load_tune_cache();
     float *tune_buf_[4] = {nullptr, nullptr, nullptr, nullptr};
     size_t tune_floats_[4] = {0, 0, 0, 0};
@@ -102,6 +109,7 @@ private:
     void setup();
     void tune_convs();
     void launch_op(const PlanOp &op, hipStream_t stream);
+    unsigned *counters_of(const PlanConv &c) const;
     void enqueue(bool stage_events);   // issue one forward pass according to the execution mode
     void enqueue_streams(bool stage_events);
     void enqueue_fused(bool stage_events);

@@ -106,6 +106,22 @@ float *DeviceContext::tuning_buffer(int which, size_t floats) {
     return tune_buf_[which];
 }
 
+unsigned *DeviceContext::tuning_counters(size_t count) {
+    if (count == 0) return nullptr;
+    if (count > tune_counter_count_) {
+        IOS_HIP(hipDeviceSynchronize());
+        if (tune_counters_ != nullptr) IOS_HIP(hipFree(tune_counters_));
+        tune_counters_ = nullptr;
+        tune_counter_count_ = 0;
+        const size_t want = count * 2 + 1024;
+        IOS_HIP(hipMalloc(reinterpret_cast<void **>(&tune_counters_), want * sizeof(unsigned)));
+        tune_counter_count_ = want;
+        launch_fill_u32(tune_counters_, want, 0u, streams_[0]);
+        IOS_HIP(hipStreamSynchronize(streams_[0]));
+    }
+    return tune_counters_;
+}
+
 DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     // Like the reference's exhaustive algorithm search on first sight of a shape: run every kernel
     // configuration on scratch tensors of the real shape and keep the fastest.
@@ -147,10 +163,11 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
             last_effective = effective;
             if (ws > kMaxWorkspace) break;
             float *workspace = ws ? tuning_buffer(3, ws) : nullptr;
-            launch_conv_mfma(p, l, x, packed, bias, y, workspace, stream);   // warm-up
+            unsigned *counters = inline_reduce_ ? tuning_counters(conv_counter_count(p, l)) : nullptr;
+            launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream);   // warm-up
             IOS_HIP(hipEventRecord(start, stream));
             const int reps = 4;
-            for (int r = 0; r < reps; r++) launch_conv_mfma(p, l, x, packed, bias, y, workspace, stream);
+            for (int r = 0; r < reps; r++) launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream);
             IOS_HIP(hipEventRecord(stop, stream));
             IOS_HIP(hipEventSynchronize(stop));
             float ms = 0.f;
@@ -250,6 +267,10 @@ void DeviceContext::set_option(const std::string &key, const std::string &value)
         const int v = atoi(value.c_str());
         if (v < 0 || v > 64) throw std::runtime_error("option conv_split_k: expected 0..64");
         forced_split_k_ = v;
+    } else if (key == "split_k_reduce") {
+        if (value == "inline") inline_reduce_ = true;
+        else if (value == "kernel") inline_reduce_ = false;
+        else throw std::runtime_error("option split_k_reduce: expected inline or kernel, got '" + value + "'");
     } else if (key == "clear_tuning") {
         tuned.clear();
     } else {
@@ -261,6 +282,7 @@ std::string DeviceContext::info_json() const {
     std::ostringstream os;
     os << "{\"name\":\"" << name_ << "\",\"arch\":\"" << arch_ << "\",\"compute_units\":" << num_cus_
        << ",\"executor\":\"" << (exec_mode_ == ExecMode::Graph ? "graph" : exec_mode_ == ExecMode::Fused ? "fused" : exec_mode_ == ExecMode::FusedGraph ? "fused_graph" : "streams") << "\",\"autotune\":" << (autotune_ ? "true" : "false")
+       << ",\"split_k_reduce\":\"" << (inline_reduce_ ? "inline" : "kernel") << "\""
        << ",\"max_groups\":" << kMaxGroups << ",\"conv_variants\":[";
     for (int i = 0; i < conv_num_variants(); i++) os << (i ? "," : "") << '"' << conv_variant(i).name << '"';
     os << "]}";
@@ -317,6 +339,8 @@ void Session::setup() {
         // the probes never upload filters: pack whatever the filter region holds so that the matrix
         // path reads initialised memory
         launch_pack_filters(conv.problem, conv.launch, base_ + conv.weight_off, base_ + conv.packed_off, main);
+        // split-K tickets start at zero; every launch leaves them at zero again
+        if (conv.ctr_count > 0) launch_fill_u32(reinterpret_cast<unsigned *>(base_ + conv.ctr_off), conv.ctr_count, 0u, main);
     }
     const size_t num_stages = plan_.stages.size();
     fork_events_.assign(num_stages, nullptr);
@@ -383,12 +407,17 @@ void Session::get_tensor(const std::string &name, float *host) {
     copy_out(it->second, host);
 }
 
+unsigned *Session::counters_of(const PlanConv &c) const {
+    if (c.ctr_count == 0 || !ctx_.inline_reduce()) return nullptr;
+    return reinterpret_cast<unsigned *>(base_ + c.ctr_off);
+}
+
 void Session::launch_op(const PlanOp &op, hipStream_t stream) {
     switch (op.kind) {
         case OpKind::ConvMfma: {
             const PlanConv &c = plan_.convs[op.conv];
             launch_conv_mfma(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off, tv(op.out),
-                             c.ws_floats ? base_ + c.ws_off : nullptr, stream);
+                             c.ws_floats ? base_ + c.ws_off : nullptr, counters_of(c), stream);
             break;
         }
         case OpKind::ConvDepthwise: {
@@ -473,7 +502,7 @@ void Session::build_fused() {
                     case OpKind::ConvMfma: {
                         const PlanConv &c = plan_.convs[op.conv];
                         const ConvDispatch d = make_conv_dispatch(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off,
-                                                                  tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr);
+                                                                  tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr, counters_of(c));
                         pend.item.kind = WORK_CONV;
                         pend.item.variant = d.variant;
                         pend.item.tiles = d.tiles;

@@ -33,10 +33,12 @@ def default_options():
     rt.set_option('conv_variant', -1)
     rt.set_option('conv_split_k', 0)
     rt.set_option('executor', 'streams')
+    rt.set_option('split_k_reduce', 'inline')
     yield
     rt.set_option('conv_variant', -1)
     rt.set_option('conv_split_k', 0)
     rt.set_option('executor', 'streams')
+    rt.set_option('split_k_reduce', 'inline')
 
 
 def single_op_graph(in_shape, build):
@@ -107,6 +109,35 @@ def test_every_conv_kernel_variant(variant, split_k):
         np.testing.assert_array_equal(got, got2)      # split-K reduction order is fixed
 
 
+@pytest.mark.parametrize('variant_name', ['m64n64k32_w2x2x1_t32', 'm32n32k64_w1x1x4_t32', 'm64n16k64_w4x1x1_t16',
+                                          'm32n16k64_w2x1x2_t16', 'm128n64k16_w2x2x1_t32'])
+def test_split_k_reduction_inside_the_kernel_equals_the_reduction_kernel(variant_name):
+    """Both forms add the same partial tiles in slice order, so they must agree bit for bit, launch after launch."""
+    names = rt.device_info()['conv_variants']
+    rt.set_option('conv_variant', names.index(variant_name))
+    for in_shape, oc, k, p, batch, split in [((200, 8, 8), 136, (1, 1), (0, 0), 1, 6), ((72, 19, 19), 88, (3, 3), (1, 1), 2, 3),
+                                             ((96, 17, 17), 40, (1, 7), (0, 3), 1, 4)]:
+        rt.set_option('conv_split_k', split)
+        graph = single_op_graph(in_shape, lambda b, v: ios.conv2d(b, [[v]], oc, k, (1, 1), p, 1, 'relu', is_exit=True))
+        x = np.random.default_rng(5).standard_normal((batch, *in_shape)).astype(np.float32)
+        want = ios_oracle.run(graph, x)
+        results = {}
+        for form in ('kernel', 'inline'):
+            rt.set_option('split_k_reduce', form)
+            with rt.Session(graph, batch) as session:
+                session.load_weights()
+                session.set_input(x)
+                outs = []
+                for _ in range(4):          # the tickets must be back at zero after every launch
+                    session.run()
+                    outs.append(session.output())
+                for out in outs[1:]:
+                    np.testing.assert_array_equal(outs[0], out)
+                results[form] = outs[0]
+        assert_close(results['inline'], want, f'{variant_name} split {split} {in_shape}')
+        np.testing.assert_array_equal(results['inline'], results['kernel'])
+
+
 def test_split_k_is_repeatable_in_a_session():
     rt.set_option('conv_split_k', 4)
     graph = single_op_graph((64, 12, 12), lambda b, v: ios.conv2d(b, [[v]], 40, (3, 3), (1, 1), (1, 1), 1, 'relu', is_exit=True))
@@ -128,6 +159,12 @@ POOLS = [
     ((6, 8, 8), 'max', (2, 2), (2, 2), (0, 0), 3),
     ((40, 8, 8), 'global_avg', (1, 1), (1, 1), (0, 0), 2),
     ((9, 13, 13), 'global_max', (1, 1), (1, 1), (0, 0), 1),
+    # large enough for the 3 x 3 kernel to give every thread a strip of 8, 8, 8, 4 and 2 output rows
+    ((64, 147, 147), 'avg', (3, 3), (1, 1), (1, 1), 8),
+    ((64, 147, 147), 'max', (3, 3), (1, 1), (1, 1), 8),
+    ((128, 149, 149), 'max', (3, 3), (2, 2), (0, 0), 16),
+    ((96, 75, 75), 'avg', (3, 3), (2, 2), (1, 1), 32),
+    ((64, 75, 75), 'max', (3, 3), (1, 2), (1, 0), 8),
 ]
 
 
