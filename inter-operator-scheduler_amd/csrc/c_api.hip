@@ -120,7 +120,7 @@ int ios_plan_describe(const char *graph_json, int batch_size, char *buf, int cap
         const ios::Json doc = ios::Json::parse(graph_json);
         // host-only: the closed-form configuration model for a 256-CU device, no device is touched
         ios::Plan plan = ios::build_plan(ios::PlanMode::Graph, doc, nullptr, batch_size,
-                                         [](const ios::ConvProblem &p, int share) { return ios::conv_pick_launch(p, 256 / (share > 0 ? share : 1)); });
+                                         [](const ios::ConvProblem &p, int share) { return ios::conv_pick_launch(p, 256 / (share > 0 ? share : 1), share > 1); });
         const std::string text = ios::describe_plan(plan);
         needed = (int)text.size();
         if (buf != nullptr && cap > needed) memcpy(buf, text.c_str(), text.size() + 1);

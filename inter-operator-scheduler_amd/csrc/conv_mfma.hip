@@ -74,7 +74,7 @@ size_t conv_counter_count(const ConvProblem &p, const ConvLaunch &l) {
     return (size_t)p.groups * ceil_div(p.OCg(), v.BM) * (size_t)ceil_div(p.Npix(), v.BN);
 }
 
-ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus) {
+ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only) {
     // Occupancy model: a launch should offer about two blocks per compute unit.  Prefer the largest tile
     // that still does so without splitting K; otherwise take a small tile, sized to the pixel count, and
     // split K, keeping at least two K tiles per slice.
@@ -84,6 +84,7 @@ ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus) {
     ConvLaunch best;
     for (int idx : by_size) {
         const ConvVariant &v = kVariants[idx].v;
+        if (fusable_only && !v.fusable()) continue;
         const long long blocks = (long long)ceil_div(M, v.BM) * ceil_div(N, v.BN) * p.groups;
         if (blocks >= want) {
             best.variant = idx;

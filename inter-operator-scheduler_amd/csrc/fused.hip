@@ -6,7 +6,7 @@
 namespace ios {
 
 template <int T>
-__global__ __launch_bounds__(T) void fused_kernel(const WorkItem *__restrict__ items, int num_items) {
+__global__ __launch_bounds__(T, 1024 / T) void fused_kernel(const WorkItem *__restrict__ items, int num_items) {
     extern __shared__ floatx4 fused_smem[];
     float *smem = reinterpret_cast<float *>(fused_smem);
     const int bid = blockIdx.x;
@@ -25,7 +25,7 @@ __global__ __launch_bounds__(T) void fused_kernel(const WorkItem *__restrict__ i
             switch (item.variant) {
 #define IOS_CASE_TILED(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                          \
     case IDX:                                                                                              \
-        if constexpr (64 * WM * WN * WK == T) ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::run(a, smem, tile, g, z); \
+        if constexpr (64 * WM * WN * WK == T && BM * BN <= 8192) ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::run(a, smem, tile, g, z); \
         break;
 #define IOS_CASE_WSPLIT(IDX, NAME, MT, TM, TN, NW, U)                                        \
     case IDX:                                                                                \

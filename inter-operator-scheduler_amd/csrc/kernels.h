@@ -47,6 +47,9 @@ struct ConvVariant {
     bool wave_split;
     int cpad;   // channel padding of the packed filters this configuration reads
     int threads() const { return 64 * WM * WN * WK; }
+    // Tiles of more than 8192 outputs need so many registers that they would lower the occupancy of every other
+    // operator inside a fused stage launch; they only run as stand-alone kernels.
+    bool fusable() const { return BM * BN <= 8192; }
 };
 
 int conv_num_variants();
@@ -65,8 +68,9 @@ size_t conv_counter_count(const ConvProblem &p, const ConvLaunch &l);
 // The matrix path indexes packed filter rows with 16 bits and pixels / input offsets with 31 bits.
 bool conv_matrix_path_supported(const ConvProblem &p);
 
-// Default configuration from a closed-form occupancy model (num_cus = compute units of the device).
-ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus);
+// Default configuration from a closed-form occupancy model (num_cus = compute units of the device);
+// fusable_only restricts the choice to configurations that can run inside a fused stage launch.
+ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only = false);
 
 // Filter packing for a kernel configuration: w[OC][ICg][KH][KW] -> packed[g][(kh*KW + kw)*ICgP + c][OCgP],
 // ICgP = ICg rounded up to the configuration's channel padding (zero rows), OCgP = OCg rounded up to 4.

@@ -144,7 +144,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     TunedConv result;
     float best_ms[kShareClasses];
     for (int c = 0; c < kShareClasses; c++) {
-        result.best[c] = conv_pick_launch(p, std::max(1, num_cus_ >> c));
+        result.best[c] = conv_pick_launch(p, std::max(1, num_cus_ >> c), c > 0);
         best_ms[c] = 1e30f;
     }
     float fastest = 1e30f;
@@ -176,8 +176,9 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
             const double footprint = (double)cv.threads() * ((p.OCg() + cv.BM - 1) / cv.BM) * (double)((p.Npix() + cv.BN - 1) / cv.BN) *
                                      p.groups * effective;
             for (int c = 0; c < kShareClasses; c++) {
-                // class 0 is unconstrained; the others accept kernels that fit their share of the device
-                if (c > 0 && footprint > capacity / (1 << c)) continue;
+                // class 0 is unconstrained; the others accept kernels that fit their share of the device and can
+                // run inside a fused stage launch
+                if (c > 0 && (footprint > capacity / (1 << c) || !cv.fusable())) continue;
                 if (ms < best_ms[c]) {
                     best_ms[c] = ms;
                     result.best[c] = l;
@@ -214,7 +215,7 @@ ConvLaunch DeviceContext::choose_launch(const ConvProblem &p, int share) {
         if (it == tuned.end()) it = tuned.emplace(key, tune_conv(p)).first;
         launch = it->second.best[cls];
     } else {
-        launch = conv_pick_launch(p, std::max(1, num_cus_ >> cls));
+        launch = conv_pick_launch(p, std::max(1, num_cus_ >> cls), cls > 0);
     }
     if (forced_variant_ >= 0) launch.variant = forced_variant_;
     if (forced_split_k_ > 0) launch.split_k = forced_split_k_;
@@ -503,6 +504,9 @@ void Session::build_fused() {
                         const PlanConv &c = plan_.convs[op.conv];
                         const ConvDispatch d = make_conv_dispatch(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off,
                                                                   tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr, counters_of(c));
+                        if (!conv_variant(d.variant).fusable())
+                            throw std::runtime_error(std::string("convolution kernel configuration ") + conv_variant(d.variant).name +
+                                                     " cannot run inside a fused stage launch");
                         pend.item.kind = WORK_CONV;
                         pend.item.variant = d.variant;
                         pend.item.tiles = d.tiles;
