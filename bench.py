@@ -21,6 +21,10 @@ for path in (ROOT, os.path.join(ROOT, 'inter-operator-scheduler_amd')):
 
 PEAK_FP32_MATRIX_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per convolution launch of a batch-1 Inception-v3 pass, from FETCH_SIZE / WRITE_SIZE counter runs scaled by a
+# copy kernel of known size (profiles/conv_kernel_hbm_traffic_inception_v3.md); counters cannot be read from inside this
+# script, so the figure is the offline measurement of the same kernels.
+MEASURED_CONV_TRAFFIC_BYTES_PER_LAUNCH = {1: 5.86e6, 64: 132.4e6}
 
 
 def op_bound_ms(op):
@@ -54,13 +58,19 @@ def timed_latency(rt, np, graph, batch, x, steps, warmup):
                 'events_std': float(np.std(events))}, session.output()
 
 
-def conv_roofline(rt, graph, batch, x):
-    """Per-kernel HIP-event timing of one pass; returns (ops, ms per op, conv summary, memory-bound GB/s)."""
+def conv_roofline(rt, graph, batch, x, stages=False):
+    """Per-kernel HIP-event timing of one pass; returns (ops, ms per op, conv summary, memory-bound GB/s[, stage ms])."""
     with rt.Session(graph, batch) as session:
         session.load_weights()
         session.set_input(x)
         ops = session.describe()
         op_ms = session.profile_ops(warmup=3, repeat=20)
+        stage_ms = None
+        if stages:
+            repeat = 6
+            _, per_stage = session.measure(warmup=2, number=6, repeat=repeat, profile_stage=True)
+            count = len(per_stage) // repeat
+            stage_ms = [sum(per_stage[r * count + i] for r in range(repeat)) / repeat for i in range(count)]
     conv = [(op, ms) for op, ms in zip(ops, op_ms) if op['kind'] == 'conv_mfma']
     flops = sum(op['flops'] for op, _ in conv)
     ms = sum(t for _, t in conv)
@@ -69,9 +79,30 @@ def conv_roofline(rt, graph, batch, x):
     achieved = flops / (ms * 1e-3) / 1e12
     summary = {'bound': 'mfma', 'kernel': f'conv_kernel<...> ({len(conv)} convolution launches of one pass)',
                'achieved': achieved, 'peak': PEAK_FP32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
-               'frac': achieved / PEAK_FP32_MATRIX_TFLOPS, 'traffic': None,
+               'frac': achieved / PEAK_FP32_MATRIX_TFLOPS, 'traffic': MEASURED_CONV_TRAFFIC_BYTES_PER_LAUNCH.get(batch),
+               'traffic_unit': 'bytes per launch (offline counter runs)',
+               'algorithmic_bytes_per_launch': sum(op['bytes'] for op, _ in conv) / len(conv),
+               'algorithmic_flops_per_launch': flops / len(conv), 'avg_launch_us': ms / len(conv) * 1e3,
                'flops_per_pass': flops, 'kernel_ms_per_pass': ms, 'launches': len(conv)}
+    if stages:
+        return ops, op_ms, summary, mem_gbs, stage_ms
     return ops, op_ms, summary, mem_gbs
+
+
+def stage_overlap(ops, op_ms, stage_ms):
+    """Multi-group stages: time of their operators launched one by one against the measured time of the stage."""
+    groups, alone = {}, {}
+    for op, ms in zip(ops, op_ms):
+        if op['stage'] < 0:
+            continue
+        groups.setdefault(op['stage'], set()).add(op['group'])
+        alone[op['stage']] = alone.get(op['stage'], 0.0) + ms
+    multi = [s for s, g in groups.items() if len(g) > 1 and s < len(stage_ms)]
+    if not multi:
+        return None
+    return {'multi_group_stages': len(multi), 'operators_one_by_one_ms': sum(alone[s] for s in multi),
+            'stages_measured_ms': sum(stage_ms[s] for s in multi),
+            'single_group_stages_ms': sum(ms for s, ms in enumerate(stage_ms) if s not in multi)}
 
 
 def probe(args, np, ios, rt):
@@ -166,7 +197,7 @@ def main():
     seq, seq_out = timed_latency(rt, np, graph, batch, x, args.steps, args.warmup)
     opt, opt_out = timed_latency(rt, np, optimized, batch, x, args.steps, args.warmup)
 
-    ops, op_ms, roofline, mem_gbs = conv_roofline(rt, optimized, batch, x)
+    ops, op_ms, roofline, mem_gbs, stage_ms = conv_roofline(rt, optimized, batch, x, stages=True)
     roof_seq = network_roofline_ms(ops, parallel=False)
     roof_par = network_roofline_ms(ops, parallel=True)
 
@@ -195,6 +226,7 @@ def main():
                                 'fraction_of_sequential_roofline': roof_seq / opt['wall']},
         'roofline': roofline,
         'memory_bound_ops_gbs': mem_gbs,
+        'stage_overlap': stage_overlap(ops, op_ms, stage_ms),
         'device': {k: device[k] for k in ('name', 'arch', 'compute_units')},
     }
 
@@ -247,7 +279,7 @@ def main():
         config, weights = graph.export_config(), ios_oracle.graph_weights(graph)
         ios_oracle.run_graph(config, weights, x)
         runs, t = 0, time.perf_counter()
-        while runs < 6 or (time.perf_counter() - t < 10.0 and runs < 200):
+        while runs < 6 or (time.perf_counter() - t < 10.0 and runs < 2000):
             cpu_out = ios_oracle.run_graph(config, weights, x)
             runs += 1
         cpu_ms = (time.perf_counter() - t) / runs * 1e3

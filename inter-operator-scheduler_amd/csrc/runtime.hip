@@ -147,7 +147,8 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
         result.best[c] = conv_pick_launch(p, std::max(1, num_cus_ >> c), c > 0);
         best_ms[c] = 1e30f;
     }
-    float fastest = 1e30f;
+    float fastest = 1e30f, fastest_fusable_ms = 1e30f;
+    ConvLaunch fastest_fusable = conv_pick_launch(p, num_cus_, true);
     for (int v = 0; v < conv_num_variants(); v++) {
         const ConvVariant &cv = conv_variant(v);
         // tiles more than twice as tall / wide as the problem only waste lanes
@@ -184,15 +185,20 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
                     result.best[c] = l;
                 }
             }
+            if (cv.fusable() && ms < fastest_fusable_ms) {
+                fastest_fusable_ms = ms;
+                fastest_fusable = l;
+            }
             fastest = std::min(fastest, ms);
             if (ms > 3.f * fastest) break;   // more slices only add reduction work from here on
         }
     }
     IOS_HIP(hipEventDestroy(start));
     IOS_HIP(hipEventDestroy(stop));
-    // a budget nobody fits falls back to the next larger one
+    // a budget nobody fits falls back to the next larger one, the largest to the fastest configuration that
+    // can run inside a fused stage launch
     for (int c = 1; c < kShareClasses; c++)
-        if (best_ms[c] > 1e29f) result.best[c] = result.best[c - 1];
+        if (best_ms[c] > 1e29f) result.best[c] = c > 1 ? result.best[c - 1] : fastest_fusable;
     if (!tune_cache_path_.empty()) {
         FILE *f = fopen(tune_cache_path_.c_str(), "a");
         if (f != nullptr) {

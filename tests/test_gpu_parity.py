@@ -330,6 +330,29 @@ def test_network_matches_oracle_under_every_schedule_and_executor(name, make, ba
         np.testing.assert_array_equal(value, first, err_msg=str(key))
 
 
+def test_large_batch_parallel_stages_with_measured_kernel_configurations():
+    """
+    At batch 32 no kernel configuration fits the share of the device a group of a parallel stage is budgeted,
+    so the tuner falls back; whatever it picks must be able to run inside the fused stage launch.
+    """
+    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    graph.greedy_schedule(8)
+    batch = 32
+    x = np.random.default_rng(4).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
+    want = ios_oracle.run(graph, x)
+    rt.set_option('autotune', 1)
+    try:
+        for executor in ('fused', 'streams'):
+            rt.set_option('executor', executor)
+            with rt.Session(graph, batch) as session:
+                session.load_weights()
+                session.set_input(x)
+                session.run()
+                assert_close(session.output(), want, f'inception batch {batch} {executor}')
+    finally:
+        rt.set_option('autotune', 0)
+
+
 def test_merged_convolutions_match_unmerged():
     graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
     merged = ios.optimize(graph, 1, ios.AnalyticCostModel(launch=1.0, rate=2e7, sync=1.5), 'dp_parallel_merge',
