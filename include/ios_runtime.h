@@ -57,11 +57,15 @@ int graph_inference(const char *graph_json, int batch_size, float *input, int nu
 /* Message of the most recent failure (valid until the next failing call). */
 const char *ios_last_error(void);
 
-/* Options: "executor" = "streams" (one HIP stream per group, event fork/join) | "graph" (the same, captured into a
- * hipGraph and replayed) | "fused" (the groups of a stage share one kernel launch per level) | "fused_graph"; "autotune" = "0" | "1" (measure convolution
- * kernel configurations on first use, like the reference's cudnnFind-based selection,
- * src/ios/ios_runtime.cu:150-205); "clear_tuning" = anything;
- * "conv_variant" = index or -1 and "conv_split_k" = count or 0 force one convolution kernel configuration (testing). */
+/* Options (set them before sessions are created):
+ *   "executor" = "streams" (one HIP stream per group, event fork/join) | "graph" (the same, captured into a hipGraph
+ *       and replayed) | "fused" (the groups of a stage share one kernel launch per level) | "fused_graph" (fused
+ *       launches inside a hipGraph);
+ *   "autotune" = "0" | "1": measure convolution kernel configurations on first use, like the reference's
+ *       cudnnFind-based selection (src/ios/ios_runtime.cu:150-205); "clear_tuning" = anything forgets them;
+ *   "split_k_reduce" = "inline" (the last block of a tile adds the split-K slices inside the convolution kernel)
+ *       | "kernel" (a second kernel adds them); same results bit for bit;
+ *   "conv_variant" = index or -1 and "conv_split_k" = count or 0 force one convolution kernel configuration (testing). */
 int ios_set_option(const char *key, const char *value);
 
 /* JSON description of device 0 ({"name", "arch", "compute_units", ...}) into buf. */

@@ -15,8 +15,9 @@
 //
 // Parallelism for small problems comes from three places: WK wavefronts of a block split each K tile
 // and add their accumulators through LDS at the end; split_k grid slices along K write partial tiles
-// to a workspace that a second small kernel sums in slice order (fixed order, so results do not depend
-// on scheduling; no device-scope fences inside the main kernel); everything else is M x N tiling.
+// to a workspace, and the block that finishes a tile last (or a second small kernel) sums them in slice
+// order (fixed order, so results do not depend on scheduling; no device-scope fences, which would write
+// back and invalidate whole L2s); everything else is M x N tiling.
 // The epilogue adds the bias, applies the activation and stores through the output view, i.e. directly
 // into the consumer's channel window when the output lives inside a concat buffer.
 // Device-side bodies of the convolution kernels; included by the translation units that instantiate them
