@@ -450,14 +450,21 @@ __device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int bloc
 // inside the K loop, two register batches of U k-steps keep dozens of loads in flight per lane, and the NW partial
 // tiles meet once in LDS, where the wavefronts share the bias + activation + store work.  The sum order is fixed
 // (k ascending inside a wavefront, wavefronts ascending), so results are reproducible.
-template <int MT, int TM, int TN, int NW, int U>
+//
+// QUAD: within a batch of U k-steps (U * KSTEP consecutive k) the lane group lk supplies k = U * lk + u in step u
+// instead of KSTEP * u + lk.  The MFMA only needs A and B to agree on k, and this assignment gives a lane U
+// consecutive filter rows, which the quad-packed filter layout [k / 4][m][4] delivers as 16-byte loads: a quarter
+// of the filter load instructions.  Channels are padded to the batch (U * KSTEP), so a batch lies inside one tap.
+template <int MT, int TM, int TN, int NW, int U, bool QUAD = false>
 struct ConvWsplit {
     using M = Mfma<MT>;
     static constexpr int BM = TM * MT, BN = TN * MT;
     static constexpr int E = TM * TN * M::ACC;
     static constexpr int THREADS = 64 * NW;
     static constexpr int SMEM_FLOATS = NW * E * 64;
-    static constexpr int CPAD = 8;   // channel padding of the packed filters this kernel expects
+    static constexpr int CPAD = QUAD ? U * M::KSTEP : 8;   // channel padding of the packed filters this kernel expects
+    static constexpr bool KQUAD = QUAD;                    // packed filters are [k / 4][m][4] instead of [k][m]
+    static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
 
     __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *red, int tile, int g, int /*z*/) {
 
@@ -471,8 +478,8 @@ struct ConvWsplit {
     const int m0 = tm * BM;
     const int n0 = tn * BN;
 
-    const int steps_total = a.Kq / M::KSTEP;   // Kq is a multiple of 8
-    const int steps_per_wave = (steps_total + NW - 1) / NW;
+    const int steps_total = a.Kq / M::KSTEP;   // Kq is a multiple of 8 (of U * KSTEP with QUAD)
+    const int steps_per_wave = QUAD ? (steps_total / U + NW - 1) / NW * U : (steps_total + NW - 1) / NW;
     const int s_begin = wave * steps_per_wave;
     const int s_end = min(steps_total, s_begin + steps_per_wave);
 
@@ -490,7 +497,8 @@ struct ConvWsplit {
         const int ow = r - oh * a.OW;
         ih0[j] = oh * a.sh - a.ph;
         iw0[j] = ow * a.sw - a.pw;
-        x_lane[j] = (unsigned)(((long long)b * a.x_bs + ((long long)g * a.ICg + lk) * a.HW + (long long)ih0[j] * a.W + iw0[j]) * 4);
+        const int lane_channel = QUAD ? U * lk : lk;   // first channel of this lane inside a step / batch
+        x_lane[j] = (unsigned)(((long long)b * a.x_bs + ((long long)g * a.ICg + lane_channel) * a.HW + (long long)ih0[j] * a.W + iw0[j]) * 4);
     }
     const __amdgpu_buffer_rsrc_t xr = buffer_of(a.x, a.x_bytes);
     const __amdgpu_buffer_rsrc_t wr = buffer_of(a.wp, a.w_bytes);
@@ -498,7 +506,10 @@ struct ConvWsplit {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         w_kill[i] = m0 + i * MT + lc < a.OCgP ? 0u : kOutOfRange;
-        w_lane[i] = (unsigned)(((size_t)g * a.Kq * a.OCgP + (size_t)lk * a.OCgP + m0 + i * MT + lc) * 4);
+        if (QUAD)   // [g][k / 4][m][4]: this lane's first quad of a batch is row (U / 4) * lk
+            w_lane[i] = (unsigned)((((size_t)g * (a.Kq / 4) + (size_t)(U / 4) * lk) * a.OCgP + m0 + i * MT + lc) * 16);
+        else
+            w_lane[i] = (unsigned)(((size_t)g * a.Kq * a.OCgP + (size_t)lk * a.OCgP + m0 + i * MT + lc) * 4);
     }
 #pragma unroll
     for (int j = 0; j < TN; j++) n_kill[j] = n_ok[j] ? 0u : kOutOfRange;
@@ -516,6 +527,43 @@ struct ConvWsplit {
     // k-step s covers rows k = s * KSTEP + lk of the tap-major packed filters; ICgP is a multiple of KSTEP, so a
     // step lies inside one filter tap and (tap, kh, kw, first channel) are wavefront-uniform
     auto load_batch = [&](int s0, float(&A)[U][TM], float(&B)[U][TN]) {
+        if constexpr (QUAD) {
+            // the whole batch lies inside one tap; batches start at multiples of U steps and ranges end at one
+            const int kb = s0 * M::KSTEP;
+            const int tap = (int)__umulhi((unsigned)kb, a.magic_icgp);
+            const int cb = kb - tap * a.ICgP;
+            const int kh = a.KW == 1 ? tap : (int)__umulhi((unsigned)tap, a.magic_kw);
+            const int kw = tap - kh * a.KW;
+            const unsigned batch_kill = s0 < s_end ? 0u : kOutOfRange;   // wavefront-uniform
+            const unsigned w_batch = (unsigned)((kb / 4) * a.OCgP) * 16u;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int q = 0; q < U / 4; q++) {
+                    const floatx4 w4 = buffer_load_f32x4(wr, (w_lane[i] + w_batch + (unsigned)(q * a.OCgP) * 16u) | w_kill[i] | batch_kill);
+                    A[q * 4 + 0][i] = w4.x;
+                    A[q * 4 + 1][i] = w4.y;
+                    A[q * 4 + 2][i] = w4.z;
+                    A[q * 4 + 3][i] = w4.w;
+                }
+            const unsigned x_batch = (unsigned)(cb * a.HW + kh * a.W + kw) * 4u;
+            const int c_left = a.ICg - 1 - cb - U * lk;   // channels of this lane beyond c_left are padding
+            unsigned kill[TN];
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const unsigned in_h = (unsigned)(ih0[j] + kh) < (unsigned)a.H ? 1u : 0u;
+                const unsigned in_w = (unsigned)(iw0[j] + kw) < (unsigned)a.W ? 1u : 0u;
+                kill[j] = (((in_h & in_w) ^ 1u) << 31) | n_kill[j] | batch_kill;
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const unsigned c_kill = (unsigned)(c_left - u) & kOutOfRange;   // sign bit
+                const unsigned x_step = x_batch + (unsigned)(u * a.HW) * 4u;
+#pragma unroll
+                for (int j = 0; j < TN; j++) B[u][j] = buffer_load_f32(xr, (x_lane[j] + x_step) | kill[j] | c_kill);
+            }
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const bool s_ok = (s0 + u) < s_end;
@@ -607,16 +655,21 @@ struct ConvWsplit {
     X(13, "m96n128k16_w1x4x1_t32", 96, 128, 16, 1, 4, 1, 32, 3)  \
     X(14, "m192n128k16_w2x2x1_t32", 192, 128, 16, 2, 2, 1, 32, 3) \
     X(15, "m160n128k16_w1x4x1_t32", 160, 128, 16, 1, 4, 1, 32, 3)
-// X(index, name, MT, TM, TN, NW, U) for the wave-split kernel
+// X(index, name, MT, TM, TN, NW, U, QUAD) for the wave-split kernel
 #define IOS_WSPLIT_VARIANTS(X)                     \
-    X(16, "ws_m32n16_w16_t16", 16, 2, 1, 16, 4)    \
-    X(17, "ws_m16n16_w16_t16", 16, 1, 1, 16, 8)    \
-    X(18, "ws_m32n32_w16_t16", 16, 2, 2, 16, 4)    \
-    X(19, "ws_m64n16_w16_t16", 16, 4, 1, 16, 4)    \
-    X(20, "ws_m32n16_w8_t16", 16, 2, 1, 8, 4)      \
-    X(21, "ws_m32n16_w4_t16", 16, 2, 1, 4, 8)      \
-    X(22, "ws_m32n32_w16_t32", 32, 1, 1, 16, 8)    \
-    X(23, "ws_m16n32_w16_t16", 16, 1, 2, 16, 4)
-constexpr int kNumConvVariants = 24;
+    X(16, "ws_m32n16_w16_t16", 16, 2, 1, 16, 4, false)    \
+    X(17, "ws_m16n16_w16_t16", 16, 1, 1, 16, 8, false)    \
+    X(18, "ws_m32n32_w16_t16", 16, 2, 2, 16, 4, false)    \
+    X(19, "ws_m64n16_w16_t16", 16, 4, 1, 16, 4, false)    \
+    X(20, "ws_m32n16_w8_t16", 16, 2, 1, 8, 4, false)      \
+    X(21, "ws_m32n16_w4_t16", 16, 2, 1, 4, 8, false)      \
+    X(22, "ws_m32n32_w16_t32", 32, 1, 1, 16, 8, false)    \
+    X(23, "ws_m16n32_w16_t16", 16, 1, 2, 16, 4, false)    \
+    X(24, "wq_m32n16_w16_t16", 16, 2, 1, 16, 4, true)     \
+    X(25, "wq_m32n16_w8_t16", 16, 2, 1, 8, 4, true)       \
+    X(26, "wq_m32n32_w16_t16", 16, 2, 2, 16, 4, true)     \
+    X(27, "wq_m16n16_w16_t16", 16, 1, 1, 16, 4, true)     \
+    X(28, "wq_m64n16_w8_t16", 16, 4, 1, 8, 4, true)
+constexpr int kNumConvVariants = 29;
 
 }  // namespace ios

@@ -27,11 +27,11 @@ struct VariantEntry {
 };
 
 #define IOS_TILED_ENTRY(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                        \
-    {{NAME, BM, BN, BK, WM, WN, WK, MT, false, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::CPAD},           \
+    {{NAME, BM, BN, BK, WM, WN, WK, MT, false, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::CPAD, false},    \
      conv_kernel<ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>>, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::SMEM_FLOATS},
-#define IOS_WSPLIT_ENTRY(IDX, NAME, MT, TM, TN, NW, U)                                                                \
-    {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U>::CPAD},         \
-     conv_kernel<ConvWsplit<MT, TM, TN, NW, U>>, ConvWsplit<MT, TM, TN, NW, U>::SMEM_FLOATS},
+#define IOS_WSPLIT_ENTRY(IDX, NAME, MT, TM, TN, NW, U, QUAD)                                                                  \
+    {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U, QUAD>::CPAD, QUAD},      \
+     conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD>>, ConvWsplit<MT, TM, TN, NW, U, QUAD>::SMEM_FLOATS},
 
 static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)};
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -183,12 +183,21 @@ void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorVie
 }
 
 // ---- filter packing ------------------------------------------------------------------------
-__global__ void pack_filters_kernel(const float *w, float *packed, int OCg, int OCgP, int ICg, int ICgP, int taps, int groups) {
-    // packed[g][tap * ICgP + c][m] = w[g * OCg + m][c][tap];  rows with c >= ICg and columns with m >= OCg are zero
+__global__ void pack_filters_kernel(const float *w, float *packed, int OCg, int OCgP, int ICg, int ICgP, int taps, int groups, int kquad) {
+    // packed[g][k][m] = w[g * OCg + m][c][tap] with k = tap * ICgP + c;  rows with c >= ICg and columns with m >= OCg are zero.
+    // kquad: packed[g][k / 4][m][k % 4] instead (ICgP is a multiple of 4)
     const size_t total = (size_t)groups * taps * ICgP * OCgP;
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const int m = (int)(i % OCgP);
-        const size_t gk = i / OCgP;
+        int m;
+        size_t gk;
+        if (kquad) {
+            const size_t quad = i / 4;                 // (g, k / 4, m)
+            m = (int)(quad % OCgP);
+            gk = (quad / OCgP) * 4 + (i & 3);          // (g, k)
+        } else {
+            m = (int)(i % OCgP);
+            gk = i / OCgP;
+        }
         const int c = (int)(gk % ICgP);
         const size_t gt = gk / ICgP;
         const int tap = (int)(gt % taps);
@@ -213,7 +222,7 @@ void launch_pack_filters(const ConvProblem &p, const ConvLaunch &l, const float 
     const int cpad = kVariants[l.variant].v.cpad;
     const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 65535);
     hipLaunchKernelGGL(pack_filters_kernel, dim3(blocks), dim3(256), 0, stream, w, packed, p.OCg(), p.OCgP(), p.ICg(), p.ICgP(cpad),
-                       p.KH * p.KW, p.groups);
+                       p.KH * p.KW, p.groups, kVariants[l.variant].v.kquad ? 1 : 0);
 }
 
 }  // namespace ios

@@ -46,6 +46,7 @@ struct ConvVariant {
     int BM, BN, BK, WM, WN, WK, MT;
     bool wave_split;
     int cpad;   // channel padding of the packed filters this configuration reads
+    bool kquad; // packed filters are [k / 4][m][4] (16-byte loads along k) instead of [k][m]
     int threads() const { return 64 * WM * WN * WK; }
     // Tiles of more than 8192 outputs need so many registers that they would lower the occupancy of every other
     // operator inside a fused stage launch; they only run as stand-alone kernels.
@@ -72,8 +73,9 @@ bool conv_matrix_path_supported(const ConvProblem &p);
 // fusable_only restricts the choice to configurations that can run inside a fused stage launch.
 ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only = false);
 
-// Filter packing for a kernel configuration: w[OC][ICg][KH][KW] -> packed[g][(kh*KW + kw)*ICgP + c][OCgP],
-// ICgP = ICg rounded up to the configuration's channel padding (zero rows), OCgP = OCg rounded up to 4.
+// Filter packing for a kernel configuration: w[OC][ICg][KH][KW] -> packed[g][k = (kh*KW + kw)*ICgP + c][OCgP]
+// (or [g][k / 4][OCgP][k % 4] for kquad configurations), ICgP = ICg rounded up to the configuration's channel
+// padding (zero rows), OCgP = OCg rounded up to 4.
 size_t conv_packed_floats(const ConvProblem &p, const ConvLaunch &l);
 size_t conv_packed_floats_max(const ConvProblem &p);   // over all configurations
 void launch_pack_filters(const ConvProblem &p, const ConvLaunch &l, const float *w, float *packed, hipStream_t stream);

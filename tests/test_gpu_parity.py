@@ -95,7 +95,7 @@ def test_every_conv_kernel_variant(variant, split_k):
     names = rt.device_info()['conv_variants']
     if variant >= len(names):
         pytest.skip('no such kernel variant')
-    if names[variant].startswith('ws_') and split_k > 1:
+    if names[variant].startswith(('ws_', 'wq_')) and split_k > 1:
         pytest.skip('wave-split kernels divide K inside the block')
     rt.set_option('conv_variant', variant)
     rt.set_option('conv_split_k', split_k)
