@@ -466,7 +466,7 @@ struct ConvWsplit {
     static constexpr bool KQUAD = QUAD;                    // packed filters are [k / 4][m][4] instead of [k][m]
     static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
 
-    __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *red, int tile, int g, int /*z*/) {
+    __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *red, int tile, int g, int z) {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -478,10 +478,13 @@ struct ConvWsplit {
     const int m0 = tm * BM;
     const int n0 = tn * BN;
 
-    const int steps_total = a.Kq / M::KSTEP;   // Kq is a multiple of 8 (of U * KSTEP with QUAD)
-    const int steps_per_wave = QUAD ? (steps_total / U + NW - 1) / NW * U : (steps_total + NW - 1) / NW;
-    const int s_begin = wave * steps_per_wave;
-    const int s_end = min(steps_total, s_begin + steps_per_wave);
+    // K slice z of the grid (k_chunk is a multiple of the batch U * KSTEP), divided among the wavefronts
+    const int s_lo = z * (a.k_chunk / M::KSTEP);
+    const int s_hi = min(a.Kq / M::KSTEP, s_lo + a.k_chunk / M::KSTEP);   // Kq is a multiple of 8 (of U * KSTEP with QUAD)
+    const int steps_slice = s_hi - s_lo;
+    const int steps_per_wave = QUAD ? ((steps_slice + U - 1) / U + NW - 1) / NW * U : (steps_slice + NW - 1) / NW;
+    const int s_begin = s_lo + wave * steps_per_wave;
+    const int s_end = min(s_hi, s_begin + steps_per_wave);
 
     int ih0[TN], iw0[TN];
     unsigned x_lane[TN];   // byte offset of (image, group channel lk, ih0, iw0); wraps like x_thread above
@@ -618,10 +621,54 @@ struct ConvWsplit {
 #pragma unroll
             for (int v = 0; v < M::ACC; v++) red[(wave * E + (i * TN + j) * M::ACC + v) * 64 + lane] = acc[i][j][v];
     __syncthreads();
+    if (a.split_k > 1 && a.counters == nullptr) {
+        // two-kernel split-K: this slice's partial outputs as [slice][group][m][pixel] for splitk_reduce_kernel
+        float *wsz = a.ws + ((size_t)z * a.groups + g) * a.OCg * (size_t)a.Npix;
+        for (int e = wave; e < E; e += NW) {
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; w++) sum += red[(w * E + e) * 64 + lane];
+            const int m = m0 + (e / (M::ACC * TN)) * MT + M::row(e % M::ACC, lane);
+            const int nn = n0 + ((e / M::ACC) % TN) * MT + lc;
+            if (m < a.OCg && nn < a.Npix) wsz[(size_t)m * a.Npix + nn] = sum;
+        }
+        return;
+    }
+    float *slices = nullptr;
+    if (a.split_k > 1) {
+        // one-kernel split-K, as in the LDS-tiled kernel: partial tiles in [element][lane] order, a ticket per
+        // tile, the block drawing the last ticket adds the slices in slice order
+        const size_t tiles = (size_t)a.tiles_m * a.tiles_n;
+        slices = a.ws + (((size_t)g * tiles + tile) * a.split_k) * (size_t)(BM * BN);
+        float *mine = slices + (size_t)z * (BM * BN) + lane;
+        for (int e = wave; e < E; e += NW) {
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; w++) sum += red[(w * E + e) * 64 + lane];
+            __hip_atomic_store(mine + e * 64, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        int *last_flag = reinterpret_cast<int *>(red);
+        if (tid == 0) {
+            unsigned *counter = a.counters + (size_t)g * tiles + tile;
+            const unsigned ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int last = ticket == (unsigned)a.split_k - 1u ? 1 : 0;
+            if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *last_flag = last;
+        }
+        __syncthreads();
+        if (*last_flag == 0) return;
+    }
     for (int e = wave; e < E; e += NW) {
         float sum = 0.f;
+        if (a.split_k > 1) {
+            for (int s2 = 0; s2 < a.split_k; s2++)
+                sum += __hip_atomic_load(slices + (size_t)s2 * (BM * BN) + e * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
 #pragma unroll
-        for (int w = 0; w < NW; w++) sum += red[(w * E + e) * 64 + lane];
+            for (int w = 0; w < NW; w++) sum += red[(w * E + e) * 64 + lane];
+        }
         const int v = e % M::ACC;
         const int j = (e / M::ACC) % TN;
         const int i = e / (M::ACC * TN);
@@ -669,7 +716,12 @@ struct ConvWsplit {
     X(25, "wq_m32n16_w8_t16", 16, 2, 1, 8, 4, true)       \
     X(26, "wq_m32n32_w16_t16", 16, 2, 2, 16, 4, true)     \
     X(27, "wq_m16n16_w16_t16", 16, 1, 1, 16, 4, true)     \
-    X(28, "wq_m64n16_w8_t16", 16, 4, 1, 8, 4, true)
-constexpr int kNumConvVariants = 29;
+    X(28, "wq_m64n16_w8_t16", 16, 4, 1, 8, 4, true)       \
+    X(29, "wq_m64n32_w8_t16", 16, 4, 2, 8, 4, true)       \
+    X(30, "wq_m64n64_w4_t16", 16, 4, 4, 4, 4, true)       \
+    X(31, "wq_m64n32_w4_t16", 16, 4, 2, 4, 4, true)       \
+    X(32, "wq_m32n32_w8_t16", 16, 2, 2, 8, 4, true)       \
+    X(33, "wq_m64n64_w4_t32", 32, 2, 2, 4, 8, true)
+constexpr int kNumConvVariants = 34;
 
 }  // namespace ios

@@ -49,9 +49,9 @@ static int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 static int k_chunk_of(const ConvProblem &p, const ConvLaunch &l) {
     const ConvVariant &v = kVariants[l.variant].v;
     const int kq = p.Kq(v.cpad);
-    if (v.wave_split) return kq;   // one slice: K is divided inside the block
-    const int tiles_k = kq / v.BK;
-    return ceil_div(tiles_k, l.split_k) * v.BK;
+    // for the wave-split kernels BK is the K extent of one register batch, which may not divide kq
+    const int tiles_k = ceil_div(kq, v.BK);
+    return ceil_div(tiles_k, std::max(1, l.split_k)) * v.BK;
 }
 
 // split_k may ask for more slices than there are K tiles; the effective count leaves no slice empty

@@ -40,7 +40,7 @@ struct ConvProblem {
 
 // One implicit-GEMM kernel configuration: block tile BM (output channels) x BN (pixels) x BK, a grid of
 // WM x WN x WK wavefronts (WK wavefronts split K) built from MT x MT fp32 MFMA tiles.  `wave_split` selects
-// the kernel without LDS staging whose WK wavefronts each own a contiguous range of K (split_k is ignored).
+// the kernel without LDS staging whose WK wavefronts each own a contiguous range of K (of the block's K slice).
 struct ConvVariant {
     const char *name;
     int BM, BN, BK, WM, WN, WK, MT;

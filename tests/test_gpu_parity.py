@@ -89,14 +89,12 @@ def test_conv_matches_oracle(case):
     assert_close(got, want, f'conv {case}')
 
 
-@pytest.mark.parametrize('variant', range(32))
+@pytest.mark.parametrize('variant', range(48))
 @pytest.mark.parametrize('split_k', [1, 3])
 def test_every_conv_kernel_variant(variant, split_k):
     names = rt.device_info()['conv_variants']
     if variant >= len(names):
         pytest.skip('no such kernel variant')
-    if names[variant].startswith(('ws_', 'wq_')) and split_k > 1:
-        pytest.skip('wave-split kernels divide K inside the block')
     rt.set_option('conv_variant', variant)
     rt.set_option('conv_split_k', split_k)
     for in_shape, oc, k, s, p, batch in [((72, 19, 19), 88, (3, 3), (1, 1), (1, 1), 2),
@@ -110,7 +108,8 @@ def test_every_conv_kernel_variant(variant, split_k):
 
 
 @pytest.mark.parametrize('variant_name', ['m64n64k32_w2x2x1_t32', 'm32n32k64_w1x1x4_t32', 'm64n16k64_w4x1x1_t16',
-                                          'm32n16k64_w2x1x2_t16', 'm128n64k16_w2x2x1_t32'])
+                                          'm32n16k64_w2x1x2_t16', 'm128n64k16_w2x2x1_t32', 'ws_m32n16_w8_t16',
+                                          'wq_m16n16_w16_t16', 'wq_m32n32_w16_t16', 'ws_m32n32_w16_t32'])
 def test_split_k_reduction_inside_the_kernel_equals_the_reduction_kernel(variant_name):
     """Both forms add the same partial tiles in slice order, so they must agree bit for bit, launch after launch."""
     names = rt.device_info()['conv_variants']
