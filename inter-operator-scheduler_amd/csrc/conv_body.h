@@ -455,7 +455,7 @@ __device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int bloc
 // instead of KSTEP * u + lk.  The MFMA only needs A and B to agree on k, and this assignment gives a lane U
 // consecutive filter rows, which the quad-packed filter layout [k / 4][m][4] delivers as 16-byte loads: a quarter
 // of the filter load instructions.  Channels are padded to the batch (U * KSTEP), so a batch lies inside one tap.
-template <int MT, int TM, int TN, int NW, int U, bool QUAD = false>
+template <int MT, int TM, int TN, int NW, int U, bool QUAD = false, int D = 2>
 struct ConvWsplit {
     using M = Mfma<MT>;
     static constexpr int BM = TM * MT, BN = TN * MT;
@@ -525,7 +525,7 @@ struct ConvWsplit {
 #pragma unroll
             for (int v = 0; v < M::ACC; v++) acc[i][j][v] = 0.f;
 
-    float av[2][U][TM], bv[2][U][TN];
+    float av[D][U][TM], bv[D][U][TN];   // D register batches in flight
 
     // k-step s covers rows k = s * KSTEP + lk of the tap-major packed filters; ICgP is a multiple of KSTEP, so a
     // step lies inside one filter tap and (tap, kh, kw, first channel) are wavefront-uniform
@@ -603,13 +603,28 @@ struct ConvWsplit {
     };
 
     const int batches = (s_end - s_begin + U - 1) / U;   // <= 0 for wavefronts beyond the end of K
-    if (batches > 0) load_batch(s_begin, av[0], bv[0]);
-    for (int b = 0; b < batches; b += 2) {
-        if (b + 1 < batches) load_batch(s_begin + (b + 1) * U, av[1], bv[1]);
-        compute(av[0], bv[0]);
-        if (b + 1 < batches) {
-            if (b + 2 < batches) load_batch(s_begin + (b + 2) * U, av[0], bv[0]);
-            compute(av[1], bv[1]);
+    if constexpr (D == 2) {
+        if (batches > 0) load_batch(s_begin, av[0], bv[0]);
+        for (int b = 0; b < batches; b += 2) {
+            if (b + 1 < batches) load_batch(s_begin + (b + 1) * U, av[1], bv[1]);
+            compute(av[0], bv[0]);
+            if (b + 1 < batches) {
+                if (b + 2 < batches) load_batch(s_begin + (b + 2) * U, av[0], bv[0]);
+                compute(av[1], bv[1]);
+            }
+        }
+    } else {
+        // deeper pipeline: D batches requested before the first one is consumed (wavefront-uniform guards only)
+#pragma unroll
+        for (int st = 0; st < D; st++)
+            if (st < batches) load_batch(s_begin + st * U, av[st], bv[st]);
+        for (int b = 0; b < batches; b += D) {
+#pragma unroll
+            for (int st = 0; st < D; st++)
+                if (b + st < batches) {
+                    compute(av[st], bv[st]);
+                    if (b + st + D < batches) load_batch(s_begin + (b + st + D) * U, av[st], bv[st]);
+                }
         }
     }
 
@@ -702,26 +717,30 @@ struct ConvWsplit {
     X(13, "m96n128k16_w1x4x1_t32", 96, 128, 16, 1, 4, 1, 32, 3)  \
     X(14, "m192n128k16_w2x2x1_t32", 192, 128, 16, 2, 2, 1, 32, 3) \
     X(15, "m160n128k16_w1x4x1_t32", 160, 128, 16, 1, 4, 1, 32, 3)
-// X(index, name, MT, TM, TN, NW, U, QUAD) for the wave-split kernel
+// X(index, name, MT, TM, TN, NW, U, QUAD, D) for the wave-split kernel
 #define IOS_WSPLIT_VARIANTS(X)                     \
-    X(16, "ws_m32n16_w16_t16", 16, 2, 1, 16, 4, false)    \
-    X(17, "ws_m16n16_w16_t16", 16, 1, 1, 16, 8, false)    \
-    X(18, "ws_m32n32_w16_t16", 16, 2, 2, 16, 4, false)    \
-    X(19, "ws_m64n16_w16_t16", 16, 4, 1, 16, 4, false)    \
-    X(20, "ws_m32n16_w8_t16", 16, 2, 1, 8, 4, false)      \
-    X(21, "ws_m32n16_w4_t16", 16, 2, 1, 4, 8, false)      \
-    X(22, "ws_m32n32_w16_t32", 32, 1, 1, 16, 8, false)    \
-    X(23, "ws_m16n32_w16_t16", 16, 1, 2, 16, 4, false)    \
-    X(24, "wq_m32n16_w16_t16", 16, 2, 1, 16, 4, true)     \
-    X(25, "wq_m32n16_w8_t16", 16, 2, 1, 8, 4, true)       \
-    X(26, "wq_m32n32_w16_t16", 16, 2, 2, 16, 4, true)     \
-    X(27, "wq_m16n16_w16_t16", 16, 1, 1, 16, 4, true)     \
-    X(28, "wq_m64n16_w8_t16", 16, 4, 1, 8, 4, true)       \
-    X(29, "wq_m64n32_w8_t16", 16, 4, 2, 8, 4, true)       \
-    X(30, "wq_m64n64_w4_t16", 16, 4, 4, 4, 4, true)       \
-    X(31, "wq_m64n32_w4_t16", 16, 4, 2, 4, 4, true)       \
-    X(32, "wq_m32n32_w8_t16", 16, 2, 2, 8, 4, true)       \
-    X(33, "wq_m64n64_w4_t32", 32, 2, 2, 4, 8, true)
-constexpr int kNumConvVariants = 34;
+    X(16, "ws_m32n16_w16_t16", 16, 2, 1, 16, 4, false, 2)    \
+    X(17, "ws_m16n16_w16_t16", 16, 1, 1, 16, 8, false, 2)    \
+    X(18, "ws_m32n32_w16_t16", 16, 2, 2, 16, 4, false, 2)    \
+    X(19, "ws_m64n16_w16_t16", 16, 4, 1, 16, 4, false, 2)    \
+    X(20, "ws_m32n16_w8_t16", 16, 2, 1, 8, 4, false, 2)      \
+    X(21, "ws_m32n16_w4_t16", 16, 2, 1, 4, 8, false, 2)      \
+    X(22, "ws_m32n32_w16_t32", 32, 1, 1, 16, 8, false, 2)    \
+    X(23, "ws_m16n32_w16_t16", 16, 1, 2, 16, 4, false, 2)    \
+    X(24, "wq_m32n16_w16_t16", 16, 2, 1, 16, 4, true, 2)     \
+    X(25, "wq_m32n16_w8_t16", 16, 2, 1, 8, 4, true, 2)       \
+    X(26, "wq_m32n32_w16_t16", 16, 2, 2, 16, 4, true, 2)     \
+    X(27, "wq_m16n16_w16_t16", 16, 1, 1, 16, 4, true, 2)     \
+    X(28, "wq_m64n16_w8_t16", 16, 4, 1, 8, 4, true, 2)       \
+    X(29, "wq_m64n32_w8_t16", 16, 4, 2, 8, 4, true, 2)       \
+    X(30, "wq_m64n64_w4_t16", 16, 4, 4, 4, 4, true, 2)       \
+    X(31, "wq_m64n32_w4_t16", 16, 4, 2, 4, 4, true, 2)       \
+    X(32, "wq_m32n32_w8_t16", 16, 2, 2, 8, 4, true, 2)       \
+    X(33, "wq_m64n64_w4_t32", 32, 2, 2, 4, 8, true, 2)       \
+    X(34, "wq_m16n16_w16_t16_d4", 16, 1, 1, 16, 4, true, 4) \
+    X(35, "wq_m32n16_w8_t16_d4", 16, 2, 1, 8, 4, true, 4)   \
+    X(36, "wq_m32n16_w16_t16_d4", 16, 2, 1, 16, 4, true, 4) \
+    X(37, "wq_m16n16_w8_t16_d4", 16, 1, 1, 8, 4, true, 4)
+constexpr int kNumConvVariants = 38;
 
 }  // namespace ios

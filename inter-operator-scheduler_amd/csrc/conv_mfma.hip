@@ -29,9 +29,9 @@ struct VariantEntry {
 #define IOS_TILED_ENTRY(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                        \
     {{NAME, BM, BN, BK, WM, WN, WK, MT, false, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::CPAD, false},    \
      conv_kernel<ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>>, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::SMEM_FLOATS},
-#define IOS_WSPLIT_ENTRY(IDX, NAME, MT, TM, TN, NW, U, QUAD)                                                                  \
-    {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U, QUAD>::CPAD, QUAD},      \
-     conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD>>, ConvWsplit<MT, TM, TN, NW, U, QUAD>::SMEM_FLOATS},
+#define IOS_WSPLIT_ENTRY(IDX, NAME, MT, TM, TN, NW, U, QUAD, D)                                                                  \
+    {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::CPAD, QUAD},      \
+     conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD, D>>, ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::SMEM_FLOATS},
 
 static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)};
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -74,31 +74,50 @@ size_t conv_counter_count(const ConvProblem &p, const ConvLaunch &l) {
     return (size_t)p.groups * ceil_div(p.OCg(), v.BM) * (size_t)ceil_div(p.Npix(), v.BN);
 }
 
+static int variant_by_name(const char *name) {
+    for (int i = 0; i < kNumVariants; i++)
+        if (std::string(kVariants[i].v.name) == name) return i;
+    throw std::runtime_error(std::string("conv: no kernel configuration named ") + name);
+}
+
 ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only) {
-    // Occupancy model: a launch should offer about two blocks per compute unit.  Prefer the largest tile
-    // that still does so without splitting K; otherwise take a small tile, sized to the pixel count, and
-    // split K, keeping at least two K tiles per slice.
+    // Closed-form model distilled from measured choices on Inception-v3 at batch 1, 16 and 64: problems that fill
+    // the device several times over with 64 x 64 tiles take the LDS-tiled kernel (the largest tile that still
+    // offers two blocks per compute unit); smaller ones take the wave-split kernel with the largest tile that
+    // still offers a block per compute unit; the smallest split K over the grid as well.
     const long long M = p.OCg(), N = p.Npix();
-    const long long want = 2LL * num_cus;
-    static const int by_size[] = {1, 5, 9, 0, 3, 4, 2, 7};   // large to small tiles
-    ConvLaunch best;
-    for (int idx : by_size) {
+    auto blocks_of = [&](int idx) {
         const ConvVariant &v = kVariants[idx].v;
-        if (fusable_only && !v.fusable()) continue;
-        const long long blocks = (long long)ceil_div(M, v.BM) * ceil_div(N, v.BN) * p.groups;
-        if (blocks >= want) {
+        return (long long)ceil_div(M, v.BM) * ceil_div(N, v.BN) * p.groups;
+    };
+    ConvLaunch best;
+    static const int tiled_mid = variant_by_name("m64n64k16_w2x2x1_t32");
+    if (blocks_of(tiled_mid) >= 4LL * num_cus) {
+        static const int by_size[] = {variant_by_name("m128n128k16_w2x2x1_t32"), variant_by_name("m128n64k16_w2x2x1_t32"),
+                                      variant_by_name("m64n128k16_w2x2x1_t32")};
+        best.variant = tiled_mid;
+        for (int idx : by_size) {
+            if (fusable_only && !kVariants[idx].v.fusable()) continue;
+            if (blocks_of(idx) >= 2LL * num_cus) {
+                best.variant = idx;
+                break;
+            }
+        }
+        return best;
+    }
+    static const int split_large_to_small[] = {variant_by_name("wq_m64n32_w8_t16"), variant_by_name("wq_m32n16_w8_t16")};
+    for (int idx : split_large_to_small)
+        if (blocks_of(idx) >= num_cus) {
             best.variant = idx;
-            best.split_k = 1;
             return best;
         }
-    }
-    const int pick = 7;   // 32 x 16 tile, four wavefronts
-    const ConvVariant &v = kVariants[pick].v;
-    const long long blocks = (long long)ceil_div(M, v.BM) * ceil_div(N, v.BN) * p.groups;
-    const int tiles_k = p.Kq(v.cpad) / v.BK;
-    int split = (int)std::min<long long>((want + blocks - 1) / blocks, std::max(1, tiles_k / 2));
-    best.variant = pick;
-    best.split_k = std::max(1, std::min(split, 32));
+    best.variant = variant_by_name("wq_m16n16_w16_t16");
+    const ConvVariant &v = kVariants[best.variant].v;
+    const long long blocks = blocks_of(best.variant);
+    const int batches = ceil_div(p.Kq(v.cpad), v.BK);          // register batches along K
+    const int per_slice = 2 * v.WK;                            // leave every wavefront two batches
+    const long long split = std::min<long long>((num_cus + blocks - 1) / blocks, std::max(1, batches / per_slice));
+    best.split_k = (int)std::max<long long>(1, std::min<long long>(split, 16));
     return best;
 }
 
