@@ -59,6 +59,8 @@ static int effective_split(const ConvProblem &p, const ConvLaunch &l) {
     return std::max(1, ceil_div(p.Kq(kVariants[l.variant].v.cpad), k_chunk_of(p, l)));
 }
 
+int conv_effective_split(const ConvProblem &p, const ConvLaunch &l) { return effective_split(p, l); }
+
 size_t conv_workspace_floats(const ConvProblem &p, const ConvLaunch &l) {
     const int s = effective_split(p, l);
     if (s <= 1) return 0;

@@ -61,6 +61,8 @@ struct ConvLaunch {
     int split_k = 1;  // number of grid slices along K; > 1 needs workspace
 };
 
+// Grid slices along K a launch configuration really uses (split_k may ask for more than there are K tiles).
+int conv_effective_split(const ConvProblem &p, const ConvLaunch &l);
 // Floats of workspace a launch configuration needs (split_k partial outputs; large enough for both split-K forms).
 size_t conv_workspace_floats(const ConvProblem &p, const ConvLaunch &l);
 // Ticket counters the one-kernel split-K form needs: one unsigned per (group, output tile), zero before the

@@ -14,6 +14,7 @@
 
 #include "fused.h"
 
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
 #include <sstream>
@@ -141,14 +142,28 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     // one winner per footprint budget: the whole device, a half, a quarter, an eighth (threads in flight);
     // a convolution that shares its stage with other groups uses the winner of the matching budget
     const double capacity = (double)num_cus_ * 2048.0;
-    TunedConv result;
-    float best_ms[kShareClasses];
-    for (int c = 0; c < kShareClasses; c++) {
-        result.best[c] = conv_pick_launch(p, std::max(1, num_cus_ >> c), c > 0);
-        best_ms[c] = 1e30f;
-    }
-    float fastest = 1e30f, fastest_fusable_ms = 1e30f;
-    ConvLaunch fastest_fusable = conv_pick_launch(p, num_cus_, true);
+    struct Candidate {
+        ConvLaunch launch;
+        float ms;
+        double footprint;
+        bool fusable;
+    };
+    auto measure = [&](const ConvLaunch &l, int reps) {
+        const size_t ws = conv_workspace_floats(p, l);
+        float *workspace = ws ? tuning_buffer(3, ws) : nullptr;
+        unsigned *counters = inline_reduce_ ? tuning_counters(conv_counter_count(p, l)) : nullptr;
+        launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream);   // warm-up
+        IOS_HIP(hipEventRecord(start, stream));
+        for (int r = 0; r < reps; r++) launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream);
+        IOS_HIP(hipEventRecord(stop, stream));
+        IOS_HIP(hipEventSynchronize(stop));
+        float ms = 0.f;
+        IOS_HIP(hipEventElapsedTime(&ms, start, stop));
+        return ms / reps;
+    };
+    // first pass: every configuration and split factor, a few launches each
+    std::vector<Candidate> candidates;
+    float fastest = 1e30f;
     for (int v = 0; v < conv_num_variants(); v++) {
         const ConvVariant &cv = conv_variant(v);
         // tiles more than twice as tall / wide as the problem only waste lanes
@@ -158,47 +173,52 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
             ConvLaunch l;
             l.variant = v;
             l.split_k = split;
-            const size_t ws = conv_workspace_floats(p, l);
-            const int effective = ws == 0 ? 1 : (int)(ws / ((size_t)p.OC * p.Npix()));
+            const int effective = conv_effective_split(p, l);
             if (effective == last_effective) continue;   // asks for more slices than there are K tiles
             last_effective = effective;
-            if (ws > kMaxWorkspace) break;
-            float *workspace = ws ? tuning_buffer(3, ws) : nullptr;
-            unsigned *counters = inline_reduce_ ? tuning_counters(conv_counter_count(p, l)) : nullptr;
-            launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream);   // warm-up
-            IOS_HIP(hipEventRecord(start, stream));
-            const int reps = 4;
-            for (int r = 0; r < reps; r++) launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream);
-            IOS_HIP(hipEventRecord(stop, stream));
-            IOS_HIP(hipEventSynchronize(stop));
-            float ms = 0.f;
-            IOS_HIP(hipEventElapsedTime(&ms, start, stop));
-            ms /= reps;
+            if (conv_workspace_floats(p, l) > kMaxWorkspace) break;
+            const float ms = measure(l, 4);
             const double footprint = (double)cv.threads() * ((p.OCg() + cv.BM - 1) / cv.BM) * (double)((p.Npix() + cv.BN - 1) / cv.BN) *
                                      p.groups * effective;
-            for (int c = 0; c < kShareClasses; c++) {
-                // class 0 is unconstrained; the others accept kernels that fit their share of the device and can
-                // run inside a fused stage launch
-                if (c > 0 && (footprint > capacity / (1 << c) || !cv.fusable())) continue;
-                if (ms < best_ms[c]) {
-                    best_ms[c] = ms;
-                    result.best[c] = l;
-                }
-            }
-            if (cv.fusable() && ms < fastest_fusable_ms) {
-                fastest_fusable_ms = ms;
-                fastest_fusable = l;
-            }
+            candidates.push_back({l, ms, footprint, cv.fusable()});
             fastest = std::min(fastest, ms);
             if (ms > 3.f * fastest) break;   // more slices only add reduction work from here on
         }
     }
+    // second pass: the three fastest of every class again with more launches (the first pass is noisy at 5-10 us)
+    std::sort(candidates.begin(), candidates.end(), [](const Candidate &a, const Candidate &b) { return a.ms < b.ms; });
+    std::vector<char> refined(candidates.size(), 0);
+    TunedConv result;
+    bool found[kShareClasses];
+    for (int c = 0; c < kShareClasses; c++) {
+        // class 0 is unconstrained; the others accept kernels that fit their share of the device and can run inside
+        // a fused stage launch; a budget nobody fits takes the fastest fusable configuration
+        auto eligible = [&](const Candidate &cand, bool fit) {
+            if (c == 0) return true;
+            return cand.fusable && (!fit || cand.footprint <= capacity / (1 << c));
+        };
+        found[c] = false;
+        for (int pass = 0; pass < 2 && !found[c]; pass++) {
+            int taken = 0;
+            float best = 1e30f;
+            for (size_t i = 0; i < candidates.size() && taken < 3; i++) {
+                if (!eligible(candidates[i], pass == 0)) continue;
+                taken++;
+                if (!refined[i]) {
+                    candidates[i].ms = std::min(candidates[i].ms, measure(candidates[i].launch, 16));
+                    refined[i] = 1;
+                }
+                if (candidates[i].ms < best) {
+                    best = candidates[i].ms;
+                    result.best[c] = candidates[i].launch;
+                    found[c] = true;
+                }
+            }
+        }
+        if (!found[c]) result.best[c] = conv_pick_launch(p, std::max(1, num_cus_ >> c), c > 0);
+    }
     IOS_HIP(hipEventDestroy(start));
     IOS_HIP(hipEventDestroy(stop));
-    // a budget nobody fits falls back to the next larger one, the largest to the fastest configuration that
-    // can run inside a fused stage launch
-    for (int c = 1; c < kShareClasses; c++)
-        if (best_ms[c] > 1e29f) result.best[c] = c > 1 ? result.best[c - 1] : fastest_fusable;
     if (!tune_cache_path_.empty()) {
         FILE *f = fopen(tune_cache_path_.c_str(), "a");
         if (f != nullptr) {
