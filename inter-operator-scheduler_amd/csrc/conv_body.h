@@ -152,7 +152,7 @@ struct ConvTiled {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: keeps per-wavefront K ranges and loop control on the SALU
     const int wn = wave % WN;
     const int wm = (wave / WN) % WM;
     const int wk = wave / (WN * WM);
@@ -228,6 +228,7 @@ struct ConvTiled {
         }
     };
 
+    const int relu_floor = a.pre_relu ? 0 : (int)0x80000000;
     auto store_tile = [&](int buf, const floatx4(&ar)[A_ITERS], const float(&br)[B_ITERS]) {
         float *Ab = As + buf * BK * LDA;
         float *Bb = Bs + buf * BK * LDB;
@@ -242,9 +243,8 @@ struct ConvTiled {
         }
 #pragma unroll
         for (int i = 0; i < B_ITERS; i++) {
-            float v = br[i];
-            if (a.pre_relu) v = fmaxf(v, 0.f);
-            Bb[(bk_l + i * B_ROWS_PER_PASS) * LDB + bn_l] = v;
+            // folded ReLU of the producer as one integer max (negative floats are negative integers)
+            Bb[(bk_l + i * B_ROWS_PER_PASS) * LDB + bn_l] = __int_as_float(max(__float_as_int(br[i]), relu_floor));
         }
     };
 
@@ -470,7 +470,7 @@ struct ConvWsplit {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: keeps per-wavefront K ranges and loop control on the SALU
     const int lk = lane / MT;
     const int lc = lane % MT;
     int tm, tn;
@@ -590,6 +590,8 @@ struct ConvWsplit {
             }
         }
     };
+    // folded ReLU of the producer: as integers, negative floats are below 0 and everything is above INT_MIN
+    const int relu_floor = a.pre_relu ? 0 : (int)0x80000000;
     auto compute = [&](const float(&A)[U][TM], const float(&B)[U][TN]) {
 #pragma unroll
         for (int u = 0; u < U; u++)
@@ -597,7 +599,7 @@ struct ConvWsplit {
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
-                    const float bval = a.pre_relu ? fmaxf(B[u][j], 0.f) : B[u][j];
+                    const float bval = __int_as_float(max(__float_as_int(B[u][j]), relu_floor));   // one integer max
                     acc[i][j] = M::run(A[u][i], bval, acc[i][j]);
                 }
     };
