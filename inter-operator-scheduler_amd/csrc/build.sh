@@ -6,11 +6,21 @@ mkdir -p build
 FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclang -packed-fp32-ops -mllvm -amdgpu-mfma-vgpr-form=1 -Wno-unused-result"
 pids=()
 for src in conv_mfma.hip pointwise.hip fused.hip runtime.hip c_api.hip; do
-    hipcc $FLAGS -c "$src" -o "build/${src%.hip}.o" &
+    # the resource remarks go to a log: a kernel that spills registers to scratch memory is reported below
+    hipcc $FLAGS -Rpass-analysis=kernel-resource-usage -c "$src" -o "build/${src%.hip}.o" 2> "build/${src%.hip}.log" &
     pids+=($!)
 done
 hipcc $FLAGS -x hip -c plan.cpp -o build/plan.o &
 pids+=($!)
-for pid in "${pids[@]}"; do wait "$pid"; done
+status=0
+for pid in "${pids[@]}"; do wait "$pid" || status=1; done
+if [ "$status" -ne 0 ]; then
+    grep -h -B2 -A8 "error" build/*.log >&2 || cat build/*.log >&2
+    exit 1
+fi
+if grep -h "ScratchSize \[bytes/lane\]: [1-9]" build/*.log > /dev/null; then
+    echo "warning: kernels spilling to scratch memory:" >&2
+    grep -h -B4 "ScratchSize \[bytes/lane\]: [1-9]" build/*.log | grep "Function Name" | sed 's/.*Function Name: /  /; s/ \[-R.*//' >&2
+fi
 hipcc --offload-arch=gfx950 -shared -fPIC -o build/libios_runtime.so build/conv_mfma.o build/pointwise.o build/fused.o build/runtime.o build/c_api.o build/plan.o
 echo "built $(pwd)/build/libios_runtime.so"

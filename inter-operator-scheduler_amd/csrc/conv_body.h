@@ -31,6 +31,27 @@ namespace ios {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// Division of a 32-bit unsigned by a divisor fixed at launch time (Granlund-Montgomery): exact for every dividend,
+// five instructions instead of the ~20 of a hardware-less integer division.
+struct FastDiv {
+    unsigned m, s1, s2;
+};
+
+inline FastDiv make_fast_div(unsigned d) {   // d >= 1
+    unsigned l = 0;
+    while ((1ull << l) < d) l++;   // ceil(log2(d))
+    FastDiv f;
+    f.m = (unsigned)((((1ull << l) - d) << 32) / d + 1);
+    f.s1 = l < 1 ? l : 1;
+    f.s2 = l > 0 ? l - 1 : 0;
+    return f;
+}
+
+__device__ __forceinline__ unsigned fast_div(unsigned n, const FastDiv &f) {
+    const unsigned t = __umulhi(f.m, n);
+    return (t + ((n - t) >> f.s1)) >> f.s2;
+}
+
 struct ConvKernelArgs {
     const float *x;
     const float *wp;
@@ -49,6 +70,8 @@ struct ConvKernelArgs {
     int split_k, k_chunk;
     int tiles_m, tiles_n;
     int weights_major;   // 1: consecutive tiles share filter rows (filters larger than the input), 0: share pixels
+    FastDiv div_tile;    // by tiles_n (weights_major) or tiles_m
+    FastDiv div_ohw, div_ow;
 };
 
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Tiles are renumbered so that an XCD
@@ -59,11 +82,12 @@ __device__ __forceinline__ void xcd_tile(const ConvKernelArgs &a, int block, int
     const int xcd = block & 7, slot = block >> 3;
     const int q = total >> 3, r = total & 7;
     const int t = xcd < r ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
+    const int q2 = (int)fast_div((unsigned)t, a.div_tile);
     if (a.weights_major) {
-        tm = t / a.tiles_n;
+        tm = q2;
         tn = t - tm * a.tiles_n;
     } else {
-        tn = t / a.tiles_m;
+        tn = q2;
         tm = t - tn * a.tiles_m;
     }
 }
@@ -87,11 +111,12 @@ constexpr unsigned kOutOfRange = 0x80000000u;
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const float *base, unsigned bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, bytes, 0x00020000);
 }
-__device__ __forceinline__ float buffer_load_f32(__amdgpu_buffer_rsrc_t r, unsigned byte_offset) {
-    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_offset, 0, 0));
+// `scalar_offset` must be wavefront-uniform; it is added to the address after the range check of `byte_offset`.
+__device__ __forceinline__ float buffer_load_f32(__amdgpu_buffer_rsrc_t r, unsigned byte_offset, unsigned scalar_offset = 0) {
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_offset, scalar_offset, 0));
 }
-__device__ __forceinline__ floatx4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, unsigned byte_offset) {
-    const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, 0, 0);
+__device__ __forceinline__ floatx4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, unsigned byte_offset, unsigned scalar_offset = 0) {
+    const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, scalar_offset, 0);
     floatx4 f = {__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
     return f;
 }
@@ -132,6 +157,9 @@ struct ConvTiled {
     static constexpr int LDA = BM + PAD, LDB = BN + PAD;
     static constexpr int TILE_FLOATS = 2 * BK * (LDA + LDB);
     static constexpr int RED_FLOATS = (WK - 1) * BM * BN;
+    // Tiles of more than 8192 outputs need so many registers that they would lower the occupancy of every other
+    // operator inside a fused stage launch; they only run as stand-alone kernels.
+    static constexpr bool FUSABLE = BM * BN <= 8192;
     static constexpr int SMEM_FLOATS = TILE_FLOATS > RED_FLOATS ? TILE_FLOATS : RED_FLOATS;
 
     // one block: output tile `tile` of group `g`, K slice `z`; smem holds SMEM_FLOATS floats, 16-byte aligned
@@ -174,9 +202,9 @@ struct ConvTiled {
     unsigned x_thread = 0;   // byte offset of (image, group, ih0, iw0); may wrap below zero, the tap offset brings it back
     {
         const int nn = n_ok ? n : 0;
-        const int b = nn / a.OHW;
+        const int b = (int)fast_div((unsigned)nn, a.div_ohw);
         const int r = nn - b * a.OHW;
-        const int oh = r / a.OW;
+        const int oh = (int)fast_div((unsigned)r, a.div_ow);
         const int ow = r - oh * a.OW;
         ih0 = oh * a.sh - a.ph;
         iw0 = ow * a.sw - a.pw;
@@ -404,7 +432,7 @@ struct ConvTiled {
         for (int j = 0; j < TN; j++) {
             const int nn = n0 + wn * WTN + j * MT + lc;
             if (nn >= a.Npix) continue;
-            const int b = nn / a.OHW;
+            const int b = (int)fast_div((unsigned)nn, a.div_ohw);
             const int r = nn - b * a.OHW;
             float *yb = a.y + (long long)b * a.y_bs + (long long)g * a.OCg * a.OHW + r;
 #pragma unroll
@@ -464,6 +492,8 @@ struct ConvWsplit {
     static constexpr int SMEM_FLOATS = NW * E * 64;
     static constexpr int CPAD = QUAD ? U * M::KSTEP : 8;   // channel padding of the packed filters this kernel expects
     static constexpr bool KQUAD = QUAD;                    // packed filters are [k / 4][m][4] instead of [k][m]
+    // accumulators + staged operands per lane decide whether the body fits the register budget of a fused launch
+    static constexpr bool FUSABLE = E + D * U * (TM + TN) <= 88;
     static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
 
     __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *red, int tile, int g, int z) {
@@ -494,9 +524,9 @@ struct ConvWsplit {
         const int n = n0 + j * MT + lc;
         n_ok[j] = n < a.Npix;
         const int nn = n_ok[j] ? n : 0;
-        const int b = nn / a.OHW;
+        const int b = (int)fast_div((unsigned)nn, a.div_ohw);
         const int r = nn - b * a.OHW;
-        const int oh = r / a.OW;
+        const int oh = (int)fast_div((unsigned)r, a.div_ow);
         const int ow = r - oh * a.OW;
         ih0[j] = oh * a.sh - a.ph;
         iw0[j] = ow * a.sw - a.pw;
@@ -529,41 +559,67 @@ struct ConvWsplit {
 
     // k-step s covers rows k = s * KSTEP + lk of the tap-major packed filters; ICgP is a multiple of KSTEP, so a
     // step lies inside one filter tap and (tap, kh, kw, first channel) are wavefront-uniform
+    // QUAD: scalar state of the next batch to request (batches are requested in K order starting at s_begin)
+    int q_cb = 0, q_kh = 0, q_kw = 0;
+    unsigned q_w = 0;
+    if constexpr (QUAD) {
+        const int kb = s_begin * M::KSTEP;
+        const int tap = (int)__umulhi((unsigned)kb, a.magic_icgp);
+        q_cb = kb - tap * a.ICgP;
+        q_kh = a.KW == 1 ? tap : (int)__umulhi((unsigned)tap, a.magic_kw);
+        q_kw = tap - q_kh * a.KW;
+        q_w = (unsigned)((kb / 4) * a.OCgP) * 16u;
+    }
     auto load_batch = [&](int s0, float(&A)[U][TM], float(&B)[U][TN]) {
         if constexpr (QUAD) {
-            // the whole batch lies inside one tap; batches start at multiples of U steps and ranges end at one
-            const int kb = s0 * M::KSTEP;
-            const int tap = (int)__umulhi((unsigned)kb, a.magic_icgp);
-            const int cb = kb - tap * a.ICgP;
-            const int kh = a.KW == 1 ? tap : (int)__umulhi((unsigned)tap, a.magic_kw);
-            const int kw = tap - kh * a.KW;
-            const unsigned batch_kill = s0 < s_end ? 0u : kOutOfRange;   // wavefront-uniform
-            const unsigned w_batch = (unsigned)((kb / 4) * a.OCgP) * 16u;
+            // The whole batch lies inside one tap (channels are padded to the batch).  Batches are requested in K
+            // order, so (first channel, kh, kw) and the filter offset advance incrementally on the SALU.  Lane-constant
+            // offsets go into the vector operand of the buffer loads, the per-batch / per-step parts into the scalar
+            // operand: a filter load costs no VALU instruction, an input load one add + one or per batch and tile.
+            (void)s0;
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int q = 0; q < U / 4; q++) {
-                    const floatx4 w4 = buffer_load_f32x4(wr, (w_lane[i] + w_batch + (unsigned)(q * a.OCgP) * 16u) | w_kill[i] | batch_kill);
+                    const floatx4 w4 = buffer_load_f32x4(wr, w_lane[i] | w_kill[i], q_w + (unsigned)(q * a.OCgP) * 16u);
                     A[q * 4 + 0][i] = w4.x;
                     A[q * 4 + 1][i] = w4.y;
                     A[q * 4 + 2][i] = w4.z;
                     A[q * 4 + 3][i] = w4.w;
                 }
-            const unsigned x_batch = (unsigned)(cb * a.HW + kh * a.W + kw) * 4u;
-            const int c_left = a.ICg - 1 - cb - U * lk;   // channels of this lane beyond c_left are padding
-            unsigned kill[TN];
+            const unsigned x_tap = (unsigned)(q_kh * a.W + q_kw) * 4u;
+            const unsigned x_chan = (unsigned)(q_cb * a.HW) * 4u;
+            unsigned voff[TN];
 #pragma unroll
             for (int j = 0; j < TN; j++) {
-                const unsigned in_h = (unsigned)(ih0[j] + kh) < (unsigned)a.H ? 1u : 0u;
-                const unsigned in_w = (unsigned)(iw0[j] + kw) < (unsigned)a.W ? 1u : 0u;
-                kill[j] = (((in_h & in_w) ^ 1u) << 31) | n_kill[j] | batch_kill;
+                const unsigned in_h = (unsigned)(ih0[j] + q_kh) < (unsigned)a.H ? 1u : 0u;
+                const unsigned in_w = (unsigned)(iw0[j] + q_kw) < (unsigned)a.W ? 1u : 0u;
+                voff[j] = (x_lane[j] + x_tap) | (((in_h & in_w) ^ 1u) << 31);
             }
+            if (q_cb + U * M::KSTEP > a.ICg) {   // wavefront-uniform: the last batch of a tap when channels are padded
+                const int c_left = a.ICg - 1 - q_cb - U * lk;   // channels of this lane beyond c_left are padding
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                const unsigned c_kill = (unsigned)(c_left - u) & kOutOfRange;   // sign bit
-                const unsigned x_step = x_batch + (unsigned)(u * a.HW) * 4u;
+                for (int u = 0; u < U; u++) {
+                    const unsigned c_kill = (unsigned)(c_left - u) & kOutOfRange;   // sign bit
 #pragma unroll
-                for (int j = 0; j < TN; j++) B[u][j] = buffer_load_f32(xr, (x_lane[j] + x_step) | kill[j] | c_kill);
+                    for (int j = 0; j < TN; j++) B[u][j] = buffer_load_f32(xr, voff[j] | c_kill, x_chan + (unsigned)(u * a.HW) * 4u);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; u++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) B[u][j] = buffer_load_f32(xr, voff[j], x_chan + (unsigned)(u * a.HW) * 4u);
+            }
+            // next batch
+            q_w += (unsigned)((U * M::KSTEP / 4) * a.OCgP) * 16u;
+            q_cb += U * M::KSTEP;
+            if (q_cb >= a.ICgP) {
+                q_cb = 0;
+                q_kw++;
+                if (q_kw == a.KW) {
+                    q_kw = 0;
+                    q_kh++;
+                }
             }
             return;
         }
@@ -692,7 +748,7 @@ struct ConvWsplit {
         const int m = m0 + i * MT + M::row(v, lane);
         const int nn = n0 + j * MT + lc;
         if (m < a.OCg && nn < a.Npix) {
-            const int b = nn / a.OHW;
+            const int b = (int)fast_div((unsigned)nn, a.div_ohw);
             const int r = nn - b * a.OHW;
             a.y[(long long)b * a.y_bs + ((long long)g * a.OCg + m) * a.OHW + r] = apply_act(sum + a.bias[g * a.OCg + m], a.act);
         }

@@ -27,10 +27,12 @@ struct VariantEntry {
 };
 
 #define IOS_TILED_ENTRY(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                        \
-    {{NAME, BM, BN, BK, WM, WN, WK, MT, false, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::CPAD, false},    \
+    {{NAME, BM, BN, BK, WM, WN, WK, MT, false, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::CPAD, false, \
+      ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::FUSABLE},    \
      conv_kernel<ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>>, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::SMEM_FLOATS},
 #define IOS_WSPLIT_ENTRY(IDX, NAME, MT, TM, TN, NW, U, QUAD, D)                                                                  \
-    {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::CPAD, QUAD},      \
+    {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::CPAD, QUAD, \
+      ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::FUSABLE},      \
      conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD, D>>, ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::SMEM_FLOATS},
 
 static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)};
@@ -166,6 +168,9 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     a.tiles_m = ceil_div(p.OCg(), e.v.BM);
     a.tiles_n = ceil_div(p.Npix(), e.v.BN);
     a.weights_major = (double)p.OC * p.K() > (double)p.B * p.IC * p.H * p.W ? 1 : 0;
+    a.div_tile = make_fast_div((unsigned)(a.weights_major ? a.tiles_n : a.tiles_m));
+    a.div_ohw = make_fast_div((unsigned)a.OHW);
+    a.div_ow = make_fast_div((unsigned)a.OW);
     if (a.split_k > 1 && workspace == nullptr) throw std::runtime_error("conv: split-K launch without workspace");
     if (p.groups > 65535 || a.split_k > 65535) throw std::runtime_error("conv: grid too large");
     d.variant = l.variant;

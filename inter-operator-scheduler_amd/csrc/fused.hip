@@ -25,11 +25,13 @@ __global__ __launch_bounds__(T, 1024 / T) void fused_kernel(const WorkItem *__re
             switch (item.variant) {
 #define IOS_CASE_TILED(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                          \
     case IDX:                                                                                              \
-        if constexpr (64 * WM * WN * WK == T && BM * BN <= 8192) ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::run(a, smem, tile, g, z); \
+        if constexpr (64 * WM * WN * WK == T && ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::FUSABLE)                   \
+            ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::run(a, smem, tile, g, z);                                      \
         break;
 #define IOS_CASE_WSPLIT(IDX, NAME, MT, TM, TN, NW, U, QUAD, D)                                        \
     case IDX:                                                                                      \
-        if constexpr (64 * NW == T) ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::run(a, smem, tile, g, z); \
+        if constexpr (64 * NW == T && ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::FUSABLE)              \
+            ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::run(a, smem, tile, g, z);                       \
         break;
                 IOS_TILED_VARIANTS(IOS_CASE_TILED)
                 IOS_WSPLIT_VARIANTS(IOS_CASE_WSPLIT)

@@ -48,9 +48,8 @@ struct ConvVariant {
     int cpad;   // channel padding of the packed filters this configuration reads
     bool kquad; // packed filters are [k / 4][m][4] (16-byte loads along k) instead of [k][m]
     int threads() const { return 64 * WM * WN * WK; }
-    // Tiles of more than 8192 outputs need so many registers that they would lower the occupancy of every other
-    // operator inside a fused stage launch; they only run as stand-alone kernels.
-    bool fusable() const { return BM * BN <= 8192; }
+    bool fusable_;   // light enough on registers to run inside a fused stage launch
+    bool fusable() const { return fusable_; }
 };
 
 int conv_num_variants();
