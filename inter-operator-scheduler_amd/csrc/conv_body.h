@@ -157,9 +157,10 @@ struct ConvTiled {
     static constexpr int LDA = BM + PAD, LDB = BN + PAD;
     static constexpr int TILE_FLOATS = 2 * BK * (LDA + LDB);
     static constexpr int RED_FLOATS = (WK - 1) * BM * BN;
-    // Tiles of more than 8192 outputs need so many registers that they would lower the occupancy of every other
-    // operator inside a fused stage launch; they only run as stand-alone kernels.
-    static constexpr bool FUSABLE = BM * BN <= 8192;
+    // Accumulators + prefetched operands per lane: bodies above the budget would lower the occupancy of every
+    // other operator inside a fused stage launch; they only run as stand-alone kernels.
+    static constexpr int LANE_REGS = BM * BN / (64 * WM * WN) + PD * (4 * ((BK * BM / 4 + T - 1) / T) + BK * BN / T);
+    static constexpr bool FUSABLE = LANE_REGS <= 56;
     static constexpr int SMEM_FLOATS = TILE_FLOATS > RED_FLOATS ? TILE_FLOATS : RED_FLOATS;
 
     // one block: output tile `tile` of group `g`, K slice `z`; smem holds SMEM_FLOATS floats, 16-byte aligned
@@ -493,7 +494,7 @@ struct ConvWsplit {
     static constexpr int CPAD = QUAD ? U * M::KSTEP : 8;   // channel padding of the packed filters this kernel expects
     static constexpr bool KQUAD = QUAD;                    // packed filters are [k / 4][m][4] instead of [k][m]
     // accumulators + staged operands per lane decide whether the body fits the register budget of a fused launch
-    static constexpr bool FUSABLE = E + D * U * (TM + TN) <= 88;
+    static constexpr bool FUSABLE = E + D * U * (TM + TN) <= 56;
     static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
 
     __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *red, int tile, int g, int z) {

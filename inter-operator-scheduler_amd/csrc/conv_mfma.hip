@@ -109,9 +109,10 @@ ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only
         }
         return best;
     }
-    static const int split_large_to_small[] = {variant_by_name("wq_m64n32_w8_t16"), variant_by_name("wq_m32n16_w8_t16")};
+    static const int split_large_to_small[] = {variant_by_name("wq_m64n32_w8_t16"), variant_by_name("wq_m32n32_w8_t16"),
+                                               variant_by_name("wq_m32n16_w8_t16")};
     for (int idx : split_large_to_small)
-        if (blocks_of(idx) >= num_cus) {
+        if ((!fusable_only || kVariants[idx].v.fusable()) && blocks_of(idx) >= num_cus) {
             best.variant = idx;
             return best;
         }

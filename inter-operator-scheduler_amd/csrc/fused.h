@@ -15,7 +15,7 @@ enum WorkKind : int { WORK_CONV = 0, WORK_REDUCE, WORK_POOL, WORK_GLOBAL_POOL, W
 
 struct WorkItem {
     int kind;
-    int variant, reserved0;        // convolution kernel configuration
+    int variant, threads;          // convolution kernel configuration and the threads its body uses (<= block size)
     int tiles, groups;             // convolution grid decomposition: block = (tile, group, K slice)
     int first_block, num_blocks;   // range of this item inside the fused grid
     int reserved;
@@ -28,7 +28,9 @@ struct WorkItem {
     };
 };
 
-// thread-block sizes the fused kernel is instantiated for
+// Thread-block sizes the fused kernel is instantiated for.  A launch uses the size of its widest convolution body;
+// bodies that need fewer wavefronts let the surplus wavefronts of their blocks end at once (barriers only count
+// wavefronts that have not ended), the memory-bound bodies adapt to any block size.
 constexpr int kFusedThreadClasses[] = {256, 512, 1024};
 
 // Launch `num_items` items (device pointer) as one grid of `total_blocks` blocks of `threads` threads.

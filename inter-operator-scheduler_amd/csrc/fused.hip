@@ -17,6 +17,7 @@ __global__ __launch_bounds__(T, 1024 / T) void fused_kernel(const WorkItem *__re
     const int num_blocks = item.num_blocks;
     switch (item.kind) {
         case WORK_CONV: {
+            if ((int)threadIdx.x >= item.threads) return;   // surplus wavefronts of a narrower body
             const ConvKernelArgs a = item.conv;
             const int tile = local % item.tiles;
             const int rest = local / item.tiles;
@@ -25,12 +26,12 @@ __global__ __launch_bounds__(T, 1024 / T) void fused_kernel(const WorkItem *__re
             switch (item.variant) {
 #define IOS_CASE_TILED(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                          \
     case IDX:                                                                                              \
-        if constexpr (64 * WM * WN * WK == T && ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::FUSABLE)                   \
+        if constexpr (64 * WM * WN * WK <= T && ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::FUSABLE)                   \
             ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::run(a, smem, tile, g, z);                                      \
         break;
 #define IOS_CASE_WSPLIT(IDX, NAME, MT, TM, TN, NW, U, QUAD, D)                                        \
     case IDX:                                                                                      \
-        if constexpr (64 * NW == T && ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::FUSABLE)              \
+        if constexpr (64 * NW <= T && ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::FUSABLE)              \
             ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::run(a, smem, tile, g, z);                       \
         break;
                 IOS_TILED_VARIANTS(IOS_CASE_TILED)

@@ -503,7 +503,7 @@ void Session::enqueue(bool stage_events) {
 // ---- fused stage launches -----------------------------------------------------------------------------------------
 // A multi-group stage is cut into levels: level l holds the l-th kernel of every group (a split-K convolution
 // contributes its main kernel and, one level later, its reduction).  The kernels of one level are independent
-// and become work items of one fused launch per thread-block size; levels follow each other on the main stream.
+// and become work items of one fused launch; levels follow each other on the main stream.
 void Session::build_fused() {
     if (fused_built_) return;
     std::vector<WorkItem> items;
@@ -601,21 +601,19 @@ void Session::build_fused() {
                     widest = std::max(widest, chain[level].threads);
                 }
             if (widest == 0) widest = 256;
-            for (int threads : kFusedThreadClasses) {
-                FusedLaunch launch{threads, (int)items.size(), 0, 0, 0};
-                for (Pending *pend : here) {
-                    const int wants = pend->threads == 0 ? widest : pend->threads;
-                    if (wants != threads) continue;
-                    WorkItem item = pend->item;
-                    if (pend->threads == 0) item.num_blocks = std::max(1, (item.num_blocks * 256 + threads - 1) / threads);
-                    item.first_block = launch.total_blocks;
-                    launch.total_blocks += item.num_blocks;
-                    launch.smem_bytes = std::max(launch.smem_bytes, pend->smem_bytes);
-                    launch.num_items++;
-                    items.push_back(item);
-                }
-                if (launch.num_items > 0) fused_stages_[s].push_back(launch);
+            // one launch per level, as wide as its widest convolution body
+            FusedLaunch launch{widest, (int)items.size(), 0, 0, 0};
+            for (Pending *pend : here) {
+                WorkItem item = pend->item;
+                item.threads = pend->threads == 0 ? widest : pend->threads;
+                if (pend->threads == 0) item.num_blocks = std::max(1, (item.num_blocks * 256 + widest - 1) / widest);
+                item.first_block = launch.total_blocks;
+                launch.total_blocks += item.num_blocks;
+                launch.smem_bytes = std::max(launch.smem_bytes, pend->smem_bytes);
+                launch.num_items++;
+                items.push_back(item);
             }
+            fused_stages_[s].push_back(launch);
         }
     }
     if (!items.empty()) {

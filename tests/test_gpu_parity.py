@@ -224,7 +224,7 @@ def test_fused_stage_launch_covers_every_operator_kind():
     for split in (0, 3):
         rt.set_option('conv_split_k', split)
         names = rt.device_info()['conv_variants']
-        for variant in (-1, names.index('m64n64k32_w2x2x1_t32'), names.index('ws_m32n16_w16_t16')):
+        for variant in (-1, names.index('m64n64k16_w2x2x1_t32'), names.index('wq_m32n16_w8_t16'), names.index('ws_m32n16_w16_t16')):
             rt.set_option('conv_variant', variant)
             for batch in (1, 2):
                 x = np.random.default_rng(5).standard_normal((batch, 16, 14, 14)).astype(np.float32)
