@@ -18,7 +18,7 @@ __global__ __launch_bounds__(T, 1024 / T) void fused_kernel(const WorkItem *__re
     switch (item.kind) {
         case WORK_CONV: {
             if ((int)threadIdx.x >= item.threads) return;   // surplus wavefronts of a narrower body
-            const ConvKernelArgs a = item.conv;
+            const ConvKernelArgs &a = item.conv;   // fields are fetched with scalar loads where they are used
             const int tile = local % item.tiles;
             const int rest = local / item.tiles;
             const int g = rest % item.groups;
