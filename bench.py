@@ -3,7 +3,9 @@ Benchmark of the north-star path: Inception-v3 at batch 1 under the dp_parallel 
 dynamic-programming search with on-device stage measurements, on one MI355X.
 
 A step is one forward pass over one synthetic batch (weights and input already resident in HBM).  Prints one
-JSON line; DESIGN.md section 5 defines `roofline` and `cpu_baseline`.
+JSON line.  `roofline`: the convolution kernels of one pass, achieved = algorithmic FLOPs / HIP-event time of
+their launches on the launch stream, against the fp32 matrix peak.  `cpu_baseline`: the CPU oracle on the same
+graph, weights and input, timed on the host cores for about ten seconds.
 
 Probe modes for the profiler (`--probe copy`, `--probe pass`) run a fixed small workload and print what the
 counters should be compared with; they are used by the commands recorded under profiles/.
