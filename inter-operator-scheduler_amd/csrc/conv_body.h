@@ -799,7 +799,12 @@ struct ConvWsplit {
     X(34, "wq_m16n16_w16_t16_d4", 16, 1, 1, 16, 4, true, 4) \
     X(35, "wq_m32n16_w8_t16_d4", 16, 2, 1, 8, 4, true, 4)   \
     X(36, "wq_m32n16_w16_t16_d4", 16, 2, 1, 16, 4, true, 4) \
-    X(37, "wq_m16n16_w8_t16_d4", 16, 1, 1, 8, 4, true, 4)
-constexpr int kNumConvVariants = 38;
+    X(37, "wq_m16n16_w8_t16_d4", 16, 1, 1, 8, 4, true, 4)   \
+    X(38, "wq_m32n32_w4_t16", 16, 2, 2, 4, 4, true, 2)      \
+    X(39, "wq_m32n32_w2_t16_d4", 16, 2, 2, 2, 4, true, 4)   \
+    X(40, "wq_m64n32_w2_t16", 16, 4, 2, 2, 4, true, 2)      \
+    X(41, "wq_m32n64_w4_t16", 16, 2, 4, 4, 4, true, 2)      \
+    X(42, "wq_m64n32_w4_t16_d4", 16, 4, 2, 4, 4, true, 4)
+constexpr int kNumConvVariants = 43;
 
 }  // namespace ios

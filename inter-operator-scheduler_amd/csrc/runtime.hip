@@ -600,7 +600,7 @@ void Session::build_fused() {
                     here.push_back(&chain[level]);
                     widest = std::max(widest, chain[level].threads);
                 }
-            if (widest == 0) widest = 256;
+            widest = std::max(widest, 256);   // narrowest instantiation of the fused kernel
             // one launch per level, as wide as its widest convolution body
             FusedLaunch launch{widest, (int)items.size(), 0, 0, 0};
             for (Pending *pend : here) {
