@@ -162,6 +162,8 @@ def main():
     parser.add_argument('--no-sweep', action='store_true', help='skip the batch 16 / 64 sweep')
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     parser.add_argument('--no-configs', action='store_true', help='skip the other four configuration networks')
+    parser.add_argument('--search-all', action='store_true',
+                        help='run the measured schedule search on RandWire and NASNet too (minutes each) instead of the greedy schedule')
     parser.add_argument('--option', action='append', default=[], metavar='KEY=VALUE', help='extra runtime option (repeatable)')
     parser.add_argument('--probe', choices=['copy', 'pass'], help='run a profiler probe instead of the benchmark')
     args = parser.parse_args()
@@ -248,6 +250,18 @@ def main():
                              'fraction_of_network_roofline': network_roofline_ms(ops_b, parallel=False) / best,
                              'conv_tflops': roof_b['achieved'], 'conv_frac_of_fp32_matrix_peak': roof_b['frac']}
         result['batch_sweep'] = sweep
+        # reduced-precision mode (bfloat16 operands, fp32 accumulation): not the headline metric, reported beside it
+        rt.set_option('precision', 'bf16')
+        reduced = {}
+        for b in (1, 64):
+            xb = np.random.default_rng(1).standard_normal((b, 3, 299, 299)).astype(np.float32)
+            r_seq, out_b = timed_latency(rt, np, graph, b, xb, max(10, args.steps // (b * 2)), 3)
+            reduced[str(b)] = {'sequential_ms': r_seq['wall'], 'images_per_s': b / (r_seq['wall'] * 1e-3)}
+            if b == 1:
+                reduced[str(b)]['max_abs_diff_to_fp32'] = float(np.abs(out_b - seq_out).max())
+                reduced[str(b)]['fp32_output_scale'] = float(np.abs(seq_out).max())
+        rt.set_option('precision', 'fp32')
+        result['reduced_precision_bf16'] = reduced
 
     if not args.no_configs:
         configs = {}
@@ -257,12 +271,12 @@ def main():
                                    ('nasnet_mobile', ios.models.nasnet_mobile, False)):
             g = make(init_seed=0, init_scheme='he_normal')
             xc = np.random.default_rng(1).standard_normal((1, *g.enter_node.output_shape)).astype(np.float32)
-            if search:
+            if search or args.search_all:
                 rt.set_option('executor', args.search_executor)
                 scheduled = ios.optimize(g, batch_size=1, opt_type='dp_parallel', compute_weight=True, warmup=2, number=6, repeat=3)
                 label = 'dp_parallel'
                 rt.set_option('executor', args.executor)
-            else:   # the pure-Python search takes tens of minutes on these graphs: use the greedy schedule
+            else:   # the measured search takes minutes on these graphs (--search-all): use the greedy schedule
                 scheduled = make(init_seed=0, init_scheme='he_normal')
                 scheduled.greedy_schedule(4)
                 label = 'greedy'

@@ -26,6 +26,8 @@
 
 #include "kernels.h"
 
+#include <type_traits>
+
 namespace ios {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -119,6 +121,13 @@ __device__ __forceinline__ floatx4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, u
     const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, scalar_offset, 0);
     floatx4 f = {__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
     return f;
+}
+
+typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uintx2 buffer_load_u32x2(__amdgpu_buffer_rsrc_t r, unsigned byte_offset, unsigned scalar_offset = 0) {
+    return __builtin_amdgcn_raw_buffer_load_b64(r, byte_offset, scalar_offset, 0);
 }
 
 template <int MT>
@@ -484,7 +493,11 @@ __device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int bloc
 // instead of KSTEP * u + lk.  The MFMA only needs A and B to agree on k, and this assignment gives a lane U
 // consecutive filter rows, which the quad-packed filter layout [k / 4][m][4] delivers as 16-byte loads: a quarter
 // of the filter load instructions.  Channels are padded to the batch (U * KSTEP), so a batch lies inside one tap.
-template <int MT, int TM, int TN, int NW, int U, bool QUAD = false, int D = 2>
+//
+// BF16 (reduced-precision mode): filters are packed as bfloat16 in the quad layout (a lane's four k are one 8-byte
+// load), inputs are rounded to bfloat16 (nearest even) after loading, and one v_mfma_f32_16x16x16_bf16 consumes
+// the four k of a lane group at once - the same k assignment as QUAD; accumulation stays fp32.
+template <int MT, int TM, int TN, int NW, int U, bool QUAD = false, int D = 2, bool BF16 = false>
 struct ConvWsplit {
     using M = Mfma<MT>;
     static constexpr int BM = TM * MT, BN = TN * MT;
@@ -495,7 +508,9 @@ struct ConvWsplit {
     static constexpr bool KQUAD = QUAD;                    // packed filters are [k / 4][m][4] instead of [k][m]
     // accumulators + staged operands per lane decide whether the body fits the register budget of a fused launch
     static constexpr bool FUSABLE = E + D * U * (TM + TN) <= 56;
+    static constexpr bool KBF16 = BF16;                    // packed filters hold bfloat16
     static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
+    static_assert(!BF16 || (QUAD && MT == 16 && U == 4), "the bfloat16 path is the 16 x 16 x 16 form of the quad layout");
 
     __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *red, int tile, int g, int z) {
 
@@ -541,7 +556,7 @@ struct ConvWsplit {
     for (int i = 0; i < TM; i++) {
         w_kill[i] = m0 + i * MT + lc < a.OCgP ? 0u : kOutOfRange;
         if (QUAD)   // [g][k / 4][m][4]: this lane's first quad of a batch is row (U / 4) * lk
-            w_lane[i] = (unsigned)((((size_t)g * (a.Kq / 4) + (size_t)(U / 4) * lk) * a.OCgP + m0 + i * MT + lc) * 16);
+            w_lane[i] = (unsigned)((((size_t)g * (a.Kq / 4) + (size_t)(U / 4) * lk) * a.OCgP + m0 + i * MT + lc) * (BF16 ? 8 : 16));
         else
             w_lane[i] = (unsigned)(((size_t)g * a.Kq * a.OCgP + (size_t)lk * a.OCgP + m0 + i * MT + lc) * 4);
     }
@@ -556,7 +571,16 @@ struct ConvWsplit {
 #pragma unroll
             for (int v = 0; v < M::ACC; v++) acc[i][j][v] = 0.f;
 
-    float av[D][U][TM], bv[D][U][TN];   // D register batches in flight
+    // D register batches in flight: filter operands (fp32: U steps x TM tiles; bf16: four packed k per tile) and inputs
+    struct FilterStageF32 {
+        float v[U][TM];
+    };
+    struct FilterStageBf16 {
+        uintx2 v[TM];
+    };
+    using FilterStage = std::conditional_t<BF16, FilterStageBf16, FilterStageF32>;
+    FilterStage av[D];
+    float bv[D][U][TN];
 
     // k-step s covers rows k = s * KSTEP + lk of the tap-major packed filters; ICgP is a multiple of KSTEP, so a
     // step lies inside one filter tap and (tap, kh, kw, first channel) are wavefront-uniform
@@ -569,25 +593,32 @@ struct ConvWsplit {
         q_cb = kb - tap * a.ICgP;
         q_kh = a.KW == 1 ? tap : (int)__umulhi((unsigned)tap, a.magic_kw);
         q_kw = tap - q_kh * a.KW;
-        q_w = (unsigned)((kb / 4) * a.OCgP) * 16u;
+        q_w = (unsigned)((kb / 4) * a.OCgP) * (BF16 ? 8u : 16u);
     }
-    auto load_batch = [&](int s0, float(&A)[U][TM], float(&B)[U][TN]) {
+    auto load_batch = [&](int s0, FilterStage &A, float(&B)[U][TN]) {
         if constexpr (QUAD) {
             // The whole batch lies inside one tap (channels are padded to the batch).  Batches are requested in K
             // order, so (first channel, kh, kw) and the filter offset advance incrementally on the SALU.  Lane-constant
             // offsets go into the vector operand of the buffer loads, the per-batch / per-step parts into the scalar
             // operand: a filter load costs no VALU instruction, an input load one add + one or per batch and tile.
             (void)s0;
+            if constexpr (BF16) {
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int q = 0; q < U / 4; q++) {
-                    const floatx4 w4 = buffer_load_f32x4(wr, w_lane[i] | w_kill[i], q_w + (unsigned)(q * a.OCgP) * 16u);
-                    A[q * 4 + 0][i] = w4.x;
-                    A[q * 4 + 1][i] = w4.y;
-                    A[q * 4 + 2][i] = w4.z;
-                    A[q * 4 + 3][i] = w4.w;
+                for (int i = 0; i < TM; i++) {   // four bfloat16 = the lane's four k of this batch
+                    A.v[i] = buffer_load_u32x2(wr, w_lane[i] | w_kill[i], q_w);
                 }
+            } else {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int q = 0; q < U / 4; q++) {
+                        const floatx4 w4 = buffer_load_f32x4(wr, w_lane[i] | w_kill[i], q_w + (unsigned)(q * a.OCgP) * 16u);
+                        A.v[q * 4 + 0][i] = w4.x;
+                        A.v[q * 4 + 1][i] = w4.y;
+                        A.v[q * 4 + 2][i] = w4.z;
+                        A.v[q * 4 + 3][i] = w4.w;
+                    }
+            }
             const unsigned x_tap = (unsigned)(q_kh * a.W + q_kw) * 4u;
             const unsigned x_chan = (unsigned)(q_cb * a.HW) * 4u;
             unsigned voff[TN];
@@ -612,7 +643,7 @@ struct ConvWsplit {
                     for (int j = 0; j < TN; j++) B[u][j] = buffer_load_f32(xr, voff[j], x_chan + (unsigned)(u * a.HW) * 4u);
             }
             // next batch
-            q_w += (unsigned)((U * M::KSTEP / 4) * a.OCgP) * 16u;
+            q_w += (unsigned)((U * M::KSTEP / 4) * a.OCgP) * (BF16 ? 8u : 16u);
             q_cb += U * M::KSTEP;
             if (q_cb >= a.ICgP) {
                 q_cb = 0;
@@ -635,7 +666,7 @@ struct ConvWsplit {
             const unsigned w_step = (unsigned)(kb * a.OCgP) * 4u;
             const unsigned step_kill = s_ok ? 0u : kOutOfRange;   // wavefront-uniform
 #pragma unroll
-            for (int i = 0; i < TM; i++) A[u][i] = buffer_load_f32(wr, (w_lane[i] + w_step) | w_kill[i] | step_kill);
+            for (int i = 0; i < TM; i++) A.v[u][i] = buffer_load_f32(wr, (w_lane[i] + w_step) | w_kill[i] | step_kill);
             const unsigned x_step = (unsigned)(cb * a.HW + kh * a.W + kw) * 4u;
             const unsigned c_kill = (unsigned)(a.ICg - 1 - cb - lk) & kOutOfRange;   // sign bit: channel padding
 #pragma unroll
@@ -649,7 +680,20 @@ struct ConvWsplit {
     };
     // folded ReLU of the producer: as integers, negative floats are below 0 and everything is above INT_MIN
     const int relu_floor = a.pre_relu ? 0 : (int)0x80000000;
-    auto compute = [&](const float(&A)[U][TM], const float(&B)[U][TN]) {
+    auto compute = [&](const FilterStage &A, const float(&B)[U][TN]) {
+        if constexpr (BF16) {
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const floatx4 b32 = {__int_as_float(max(__float_as_int(B[0][j]), relu_floor)), __int_as_float(max(__float_as_int(B[1][j]), relu_floor)),
+                                     __int_as_float(max(__float_as_int(B[2][j]), relu_floor)), __int_as_float(max(__float_as_int(B[3][j]), relu_floor))};
+                const bf16x4 b4 = __builtin_convertvector(b32, bf16x4);   // round to nearest even
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(bf16x4, A.v[i]), b4, acc[i][j], 0, 0, 0);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < U; u++)
 #pragma unroll
@@ -657,7 +701,7 @@ struct ConvWsplit {
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
                     const float bval = __int_as_float(max(__float_as_int(B[u][j]), relu_floor));   // one integer max
-                    acc[i][j] = M::run(A[u][i], bval, acc[i][j]);
+                    acc[i][j] = M::run(A.v[u][i], bval, acc[i][j]);
                 }
     };
 
@@ -776,35 +820,45 @@ struct ConvWsplit {
     X(13, "m96n128k16_w1x4x1_t32", 96, 128, 16, 1, 4, 1, 32, 3)  \
     X(14, "m192n128k16_w2x2x1_t32", 192, 128, 16, 2, 2, 1, 32, 3) \
     X(15, "m160n128k16_w1x4x1_t32", 160, 128, 16, 1, 4, 1, 32, 3)
-// X(index, name, MT, TM, TN, NW, U, QUAD, D) for the wave-split kernel
+// X(index, name, MT, TM, TN, NW, U, QUAD, D, BF16) for the wave-split kernel
 #define IOS_WSPLIT_VARIANTS(X)                     \
-    X(16, "ws_m32n16_w16_t16", 16, 2, 1, 16, 4, false, 2)    \
-    X(17, "ws_m16n16_w16_t16", 16, 1, 1, 16, 8, false, 2)    \
-    X(18, "ws_m32n32_w16_t16", 16, 2, 2, 16, 4, false, 2)    \
-    X(19, "ws_m64n16_w16_t16", 16, 4, 1, 16, 4, false, 2)    \
-    X(20, "ws_m32n16_w8_t16", 16, 2, 1, 8, 4, false, 2)      \
-    X(21, "ws_m32n16_w4_t16", 16, 2, 1, 4, 8, false, 2)      \
-    X(22, "ws_m32n32_w16_t32", 32, 1, 1, 16, 8, false, 2)    \
-    X(23, "ws_m16n32_w16_t16", 16, 1, 2, 16, 4, false, 2)    \
-    X(24, "wq_m32n16_w16_t16", 16, 2, 1, 16, 4, true, 2)     \
-    X(25, "wq_m32n16_w8_t16", 16, 2, 1, 8, 4, true, 2)       \
-    X(26, "wq_m32n32_w16_t16", 16, 2, 2, 16, 4, true, 2)     \
-    X(27, "wq_m16n16_w16_t16", 16, 1, 1, 16, 4, true, 2)     \
-    X(28, "wq_m64n16_w8_t16", 16, 4, 1, 8, 4, true, 2)       \
-    X(29, "wq_m64n32_w8_t16", 16, 4, 2, 8, 4, true, 2)       \
-    X(30, "wq_m64n64_w4_t16", 16, 4, 4, 4, 4, true, 2)       \
-    X(31, "wq_m64n32_w4_t16", 16, 4, 2, 4, 4, true, 2)       \
-    X(32, "wq_m32n32_w8_t16", 16, 2, 2, 8, 4, true, 2)       \
-    X(33, "wq_m64n64_w4_t32", 32, 2, 2, 4, 8, true, 2)       \
-    X(34, "wq_m16n16_w16_t16_d4", 16, 1, 1, 16, 4, true, 4) \
-    X(35, "wq_m32n16_w8_t16_d4", 16, 2, 1, 8, 4, true, 4)   \
-    X(36, "wq_m32n16_w16_t16_d4", 16, 2, 1, 16, 4, true, 4) \
-    X(37, "wq_m16n16_w8_t16_d4", 16, 1, 1, 8, 4, true, 4)   \
-    X(38, "wq_m32n32_w4_t16", 16, 2, 2, 4, 4, true, 2)      \
-    X(39, "wq_m32n32_w2_t16_d4", 16, 2, 2, 2, 4, true, 4)   \
-    X(40, "wq_m64n32_w2_t16", 16, 4, 2, 2, 4, true, 2)      \
-    X(41, "wq_m32n64_w4_t16", 16, 2, 4, 4, 4, true, 2)      \
-    X(42, "wq_m64n32_w4_t16_d4", 16, 4, 2, 4, 4, true, 4)
-constexpr int kNumConvVariants = 43;
+    X(16, "ws_m32n16_w16_t16", 16, 2, 1, 16, 4, false, 2, false)    \
+    X(17, "ws_m16n16_w16_t16", 16, 1, 1, 16, 8, false, 2, false)    \
+    X(18, "ws_m32n32_w16_t16", 16, 2, 2, 16, 4, false, 2, false)    \
+    X(19, "ws_m64n16_w16_t16", 16, 4, 1, 16, 4, false, 2, false)    \
+    X(20, "ws_m32n16_w8_t16", 16, 2, 1, 8, 4, false, 2, false)      \
+    X(21, "ws_m32n16_w4_t16", 16, 2, 1, 4, 8, false, 2, false)      \
+    X(22, "ws_m32n32_w16_t32", 32, 1, 1, 16, 8, false, 2, false)    \
+    X(23, "ws_m16n32_w16_t16", 16, 1, 2, 16, 4, false, 2, false)    \
+    X(24, "wq_m32n16_w16_t16", 16, 2, 1, 16, 4, true, 2, false)     \
+    X(25, "wq_m32n16_w8_t16", 16, 2, 1, 8, 4, true, 2, false)       \
+    X(26, "wq_m32n32_w16_t16", 16, 2, 2, 16, 4, true, 2, false)     \
+    X(27, "wq_m16n16_w16_t16", 16, 1, 1, 16, 4, true, 2, false)     \
+    X(28, "wq_m64n16_w8_t16", 16, 4, 1, 8, 4, true, 2, false)       \
+    X(29, "wq_m64n32_w8_t16", 16, 4, 2, 8, 4, true, 2, false)       \
+    X(30, "wq_m64n64_w4_t16", 16, 4, 4, 4, 4, true, 2, false)       \
+    X(31, "wq_m64n32_w4_t16", 16, 4, 2, 4, 4, true, 2, false)       \
+    X(32, "wq_m32n32_w8_t16", 16, 2, 2, 8, 4, true, 2, false)       \
+    X(33, "wq_m64n64_w4_t32", 32, 2, 2, 4, 8, true, 2, false)       \
+    X(34, "wq_m16n16_w16_t16_d4", 16, 1, 1, 16, 4, true, 4, false) \
+    X(35, "wq_m32n16_w8_t16_d4", 16, 2, 1, 8, 4, true, 4, false)   \
+    X(36, "wq_m32n16_w16_t16_d4", 16, 2, 1, 16, 4, true, 4, false) \
+    X(37, "wq_m16n16_w8_t16_d4", 16, 1, 1, 8, 4, true, 4, false)   \
+    X(38, "wq_m32n32_w4_t16", 16, 2, 2, 4, 4, true, 2, false)      \
+    X(39, "wq_m32n32_w2_t16_d4", 16, 2, 2, 2, 4, true, 4, false)   \
+    X(40, "wq_m64n32_w2_t16", 16, 4, 2, 2, 4, true, 2, false)      \
+    X(41, "wq_m32n64_w4_t16", 16, 2, 4, 4, 4, true, 2, false)      \
+    X(42, "wq_m64n32_w4_t16_d4", 16, 4, 2, 4, 4, true, 4, false) \
+    X(43, "wb_m16n16_w16", 16, 1, 1, 16, 4, true, 2, true)    \
+    X(44, "wb_m16n16_w8_d4", 16, 1, 1, 8, 4, true, 4, true)   \
+    X(45, "wb_m32n16_w8", 16, 2, 1, 8, 4, true, 2, true)      \
+    X(46, "wb_m32n16_w16", 16, 2, 1, 16, 4, true, 2, true)    \
+    X(47, "wb_m32n32_w8", 16, 2, 2, 8, 4, true, 2, true)      \
+    X(48, "wb_m32n32_w4_d4", 16, 2, 2, 4, 4, true, 4, true)   \
+    X(49, "wb_m64n16_w8", 16, 4, 1, 8, 4, true, 2, true)      \
+    X(50, "wb_m64n32_w8", 16, 4, 2, 8, 4, true, 2, true)      \
+    X(51, "wb_m64n32_w4_d4", 16, 4, 2, 4, 4, true, 4, true)   \
+    X(52, "wb_m64n64_w4", 16, 4, 4, 4, 4, true, 2, true)
+constexpr int kNumConvVariants = 53;
 
 }  // namespace ios

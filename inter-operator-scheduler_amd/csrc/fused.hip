@@ -29,10 +29,10 @@ __global__ __launch_bounds__(T, 1024 / T) void fused_kernel(const WorkItem *__re
         if constexpr (64 * WM * WN * WK <= T && ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::FUSABLE)                   \
             ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::run(a, smem, tile, g, z);                                      \
         break;
-#define IOS_CASE_WSPLIT(IDX, NAME, MT, TM, TN, NW, U, QUAD, D)                                        \
+#define IOS_CASE_WSPLIT(IDX, NAME, MT, TM, TN, NW, U, QUAD, D, BF16)                                        \
     case IDX:                                                                                      \
-        if constexpr (64 * NW <= T && ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::FUSABLE)              \
-            ConvWsplit<MT, TM, TN, NW, U, QUAD, D>::run(a, smem, tile, g, z);                       \
+        if constexpr (64 * NW <= T && ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::FUSABLE)              \
+            ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::run(a, smem, tile, g, z);                       \
         break;
                 IOS_TILED_VARIANTS(IOS_CASE_TILED)
                 IOS_WSPLIT_VARIANTS(IOS_CASE_WSPLIT)

@@ -49,6 +49,7 @@ struct ConvVariant {
     bool kquad; // packed filters are [k / 4][m][4] (16-byte loads along k) instead of [k][m]
     int threads() const { return 64 * WM * WN * WK; }
     bool fusable_;   // light enough on registers to run inside a fused stage launch
+    bool bf16;       // reduced-precision mode: bfloat16 filters and inputs, fp32 accumulation
     bool fusable() const { return fusable_; }
 };
 
@@ -72,11 +73,13 @@ bool conv_matrix_path_supported(const ConvProblem &p);
 
 // Default configuration from a closed-form occupancy model (num_cus = compute units of the device);
 // fusable_only restricts the choice to configurations that can run inside a fused stage launch.
-ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only = false);
+// bf16 selects among the reduced-precision configurations.
+ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only = false, bool bf16 = false);
 
 // Filter packing for a kernel configuration: w[OC][ICg][KH][KW] -> packed[g][k = (kh*KW + kw)*ICgP + c][OCgP]
 // (or [g][k / 4][OCgP][k % 4] for kquad configurations), ICgP = ICg rounded up to the configuration's channel
-// padding (zero rows), OCgP = OCg rounded up to 4.
+// padding (zero rows), OCgP = OCg rounded up to 4.  bf16 configurations pack bfloat16 (round to nearest even), two
+// per float of the returned size.
 size_t conv_packed_floats(const ConvProblem &p, const ConvLaunch &l);
 size_t conv_packed_floats_max(const ConvProblem &p);   // over all configurations
 void launch_pack_filters(const ConvProblem &p, const ConvLaunch &l, const float *w, float *packed, hipStream_t stream);

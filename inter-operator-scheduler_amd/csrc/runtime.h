@@ -64,6 +64,7 @@ private:
     unsigned *tune_counters_ = nullptr;
     size_t tune_counter_count_ = 0;
     bool inline_reduce_ = true;
+    bool bf16_ = false;   // reduced-precision mode for matrix-path convolutions
     void load_tune_cache();
     float *tune_buf_[4] = {nullptr, nullptr, nullptr, nullptr};
     size_t tune_floats_[4] = {0, 0, 0, 0};

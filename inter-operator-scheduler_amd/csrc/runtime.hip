@@ -87,6 +87,7 @@ void DeviceContext::load_tune_cache() {
         if (!ok) break;
         std::ostringstream os;
         for (int i = 0; i < 12; i++) os << (i ? " " : "") << v[i];
+        if (conv_variant(entry.best[0].variant).bf16) os << " bf16";   // reduced-precision entries have their own keys
         tuned[os.str()] = entry;
     }
     fclose(f);
@@ -166,6 +167,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     float fastest = 1e30f;
     for (int v = 0; v < conv_num_variants(); v++) {
         const ConvVariant &cv = conv_variant(v);
+        if (cv.bf16 != bf16_) continue;   // the precision mode decides which family of configurations competes
         // tiles more than twice as tall / wide as the problem only waste lanes
         if (cv.BM >= 2 * p.OCg() + 32 || cv.BN >= 2 * p.Npix() + 32) continue;
         int last_effective = -1;
@@ -215,7 +217,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
                 }
             }
         }
-        if (!found[c]) result.best[c] = conv_pick_launch(p, std::max(1, num_cus_ >> c), c > 0);
+        if (!found[c]) result.best[c] = conv_pick_launch(p, std::max(1, num_cus_ >> c), c > 0, bf16_);
     }
     IOS_HIP(hipEventDestroy(start));
     IOS_HIP(hipEventDestroy(stop));
@@ -236,12 +238,12 @@ ConvLaunch DeviceContext::choose_launch(const ConvProblem &p, int share) {
     while (cls + 1 < kShareClasses && (1 << (cls + 1)) <= share) cls++;   // floor(log2(share)), capped
     ConvLaunch launch;
     if (autotune_) {
-        const std::string key = conv_signature(p);
+        const std::string key = conv_signature(p) + (bf16_ ? " bf16" : "");
         auto it = tuned.find(key);
         if (it == tuned.end()) it = tuned.emplace(key, tune_conv(p)).first;
         launch = it->second.best[cls];
     } else {
-        launch = conv_pick_launch(p, std::max(1, num_cus_ >> cls), cls > 0);
+        launch = conv_pick_launch(p, std::max(1, num_cus_ >> cls), cls > 0, bf16_);
     }
     if (forced_variant_ >= 0) launch.variant = forced_variant_;
     if (forced_split_k_ > 0) launch.split_k = forced_split_k_;
@@ -294,6 +296,10 @@ void DeviceContext::set_option(const std::string &key, const std::string &value)
         const int v = atoi(value.c_str());
         if (v < 0 || v > 64) throw std::runtime_error("option conv_split_k: expected 0..64");
         forced_split_k_ = v;
+    } else if (key == "precision") {
+        if (value == "fp32") bf16_ = false;
+        else if (value == "bf16") bf16_ = true;
+        else throw std::runtime_error("option precision: expected fp32 or bf16, got '" + value + "'");
     } else if (key == "split_k_reduce") {
         if (value == "inline") inline_reduce_ = true;
         else if (value == "kernel") inline_reduce_ = false;
@@ -310,6 +316,7 @@ std::string DeviceContext::info_json() const {
     os << "{\"name\":\"" << name_ << "\",\"arch\":\"" << arch_ << "\",\"compute_units\":" << num_cus_
        << ",\"executor\":\"" << (exec_mode_ == ExecMode::Graph ? "graph" : exec_mode_ == ExecMode::Fused ? "fused" : exec_mode_ == ExecMode::FusedGraph ? "fused_graph" : "streams") << "\",\"autotune\":" << (autotune_ ? "true" : "false")
        << ",\"split_k_reduce\":\"" << (inline_reduce_ ? "inline" : "kernel") << "\""
+       << ",\"precision\":\"" << (bf16_ ? "bf16" : "fp32") << "\""
        << ",\"max_groups\":" << kMaxGroups << ",\"conv_variants\":[";
     for (int i = 0; i < conv_num_variants(); i++) os << (i ? "," : "") << '"' << conv_variant(i).name << '"';
     os << "]}";

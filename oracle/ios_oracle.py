@@ -69,18 +69,26 @@ def gather_input(inputs, outputs, multiply=False):
     return terms[0] if len(terms) == 1 else torch.cat(terms, dim=1)
 
 
-def eval_node(config, outputs, weights: Weights):
+def to_bf16(t):
+    """Round to bfloat16 (nearest even) and back: the reduced-precision mode's view of a convolution operand."""
+    return t.to(torch.bfloat16).to(torch.float32)
+
+
+def eval_node(config, outputs, weights: Weights, bf16_convs=frozenset()):
     kind = config['type']
     if kind == 'sequential':
         out = None
         for child in config['nodes']:
-            out = eval_node(child, outputs, weights)
+            out = eval_node(child, outputs, weights, bf16_convs)
             outputs[child['name']] = out
         return out
     x = gather_input(config['inputs'], outputs, multiply=(kind == 'element' and config['op_type'] == 'mul'))
     if kind == 'conv':
         w, b = weights[config['name']]
-        return conv2d(x, torch.from_numpy(np.ascontiguousarray(w, dtype=np.float32)),
+        w = torch.from_numpy(np.ascontiguousarray(w, dtype=np.float32))
+        if config['name'] in bf16_convs:   # bfloat16 operands, fp32 accumulation
+            x, w = to_bf16(x), to_bf16(w)
+        return conv2d(x, w,
                       torch.from_numpy(np.ascontiguousarray(b, dtype=np.float32)),
                       config['stride'], config['padding'], config['groups'], config['act'])
     if kind == 'pool':
@@ -94,10 +102,12 @@ def eval_node(config, outputs, weights: Weights):
     raise ValueError(f'unrecognized node type {kind}')
 
 
-def run_graph(graph_config: dict, weights: Weights, x: np.ndarray, keep_all=False, num_threads: Optional[int] = None):
+def run_graph(graph_config: dict, weights: Weights, x: np.ndarray, keep_all=False, num_threads: Optional[int] = None,
+              bf16_convs=frozenset()):
     """
     Evaluate an exported graph on input ``x`` (batch, C, H, W).  Returns the exit operator's output as a
-    float32 array, or a dict name -> array of every operator when ``keep_all``.
+    float32 array, or a dict name -> array of every operator when ``keep_all``.  Convolutions named in
+    ``bf16_convs`` see their input and filters rounded to bfloat16 (the runtime's reduced-precision mode).
     """
     if num_threads is not None:
         torch.set_num_threads(num_threads)
@@ -106,7 +116,7 @@ def run_graph(graph_config: dict, weights: Weights, x: np.ndarray, keep_all=Fals
     with torch.no_grad():
         for block in graph_config['blocks']:
             for config in block['inner_nodes'] + [block['exit_node']]:
-                outputs[config['name']] = eval_node(config, outputs, weights)
+                outputs[config['name']] = eval_node(config, outputs, weights, bf16_convs)
                 last = config['name']
     if keep_all:
         return {name: t.numpy() for name, t in outputs.items()}
@@ -118,6 +128,6 @@ def graph_weights(graph) -> Weights:
     return {conv.name: (conv.weight, conv.bias) for conv in graph.conv_nodes()}
 
 
-def run(graph, x: np.ndarray, keep_all=False, num_threads=None):
+def run(graph, x: np.ndarray, keep_all=False, num_threads=None, bf16_convs=frozenset()):
     """Evaluate an ``ios.Graph`` object with the weights stored in its convolutions."""
-    return run_graph(graph.export_config(), graph_weights(graph), x, keep_all, num_threads)
+    return run_graph(graph.export_config(), graph_weights(graph), x, keep_all, num_threads, bf16_convs)

@@ -34,7 +34,9 @@ def default_options():
     rt.set_option('conv_split_k', 0)
     rt.set_option('executor', 'streams')
     rt.set_option('split_k_reduce', 'inline')
+    rt.set_option('precision', 'fp32')
     yield
+    rt.set_option('precision', 'fp32')
     rt.set_option('conv_variant', -1)
     rt.set_option('conv_split_k', 0)
     rt.set_option('executor', 'streams')
@@ -89,12 +91,14 @@ def test_conv_matches_oracle(case):
     assert_close(got, want, f'conv {case}')
 
 
-@pytest.mark.parametrize('variant', range(48))
+@pytest.mark.parametrize('variant', range(64))
 @pytest.mark.parametrize('split_k', [1, 3])
 def test_every_conv_kernel_variant(variant, split_k):
     names = rt.device_info()['conv_variants']
     if variant >= len(names):
         pytest.skip('no such kernel variant')
+    if names[variant].startswith('wb_'):
+        pytest.skip('reduced-precision configuration: see test_every_reduced_precision_kernel_configuration')
     rt.set_option('conv_variant', variant)
     rt.set_option('conv_split_k', split_k)
     for in_shape, oc, k, s, p, batch in [((72, 19, 19), 88, (3, 3), (1, 1), (1, 1), 2),
@@ -350,6 +354,83 @@ def test_large_batch_parallel_stages_with_measured_kernel_configurations():
                 assert_close(session.output(), want, f'inception batch {batch} {executor}')
     finally:
         rt.set_option('autotune', 0)
+
+
+def matrix_path_convs(graph, batch):
+    return frozenset(op['node'] for op in rt.plan_describe(graph, batch) if op['kind'] == 'conv_mfma')
+
+
+def assert_close_reduced(got, want, what=''):
+    """bfloat16 operands carry 8 bits of mantissa: 2^-8 per operand against the fp32 result, taken at the tensor's scale."""
+    scale = max(1.0, float(np.abs(want).max()))
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    assert err.max() <= 3e-2 * scale, f'{what}: max abs err {err.max():.3e} at scale {scale:.3e}'
+
+
+@pytest.mark.parametrize('case', [c for c in CONVS if c[5] == 1])
+def test_reduced_precision_conv_matches_the_bfloat16_oracle(case):
+    """precision=bf16: bit-level agreement is not expected (summation order), but against an oracle that rounds the
+    same operands to bfloat16 the fp32 tolerance holds; against the fp32 oracle the error is that of the rounding."""
+    in_shape, oc, k, s, p, g, act, batch = case
+    graph = single_op_graph(in_shape, lambda b, v: ios.conv2d(b, [[v]], oc, k, s, p, g, act, is_exit=True))
+    x = np.random.default_rng(1).standard_normal((batch, *in_shape)).astype(np.float32)
+    rt.set_option('precision', 'bf16')
+    convs = matrix_path_convs(graph, batch)
+    assert convs, 'expected a matrix-path convolution'
+    got = rt.graph_inference(graph, batch, x)
+    assert_close(got, ios_oracle.run(graph, x, bf16_convs=convs), f'bf16 conv {case}')
+    assert_close_reduced(got, ios_oracle.run(graph, x), f'bf16 conv {case} against fp32')
+    rt.set_option('precision', 'fp32')
+    assert not np.array_equal(got, rt.graph_inference(graph, batch, x))     # the mode really changes the arithmetic
+
+
+def test_every_reduced_precision_kernel_configuration():
+    names = rt.device_info()['conv_variants']
+    rt.set_option('precision', 'bf16')
+    tried = 0
+    for index, name in enumerate(names):
+        if not name.startswith('wb_'):
+            continue
+        tried += 1
+        rt.set_option('conv_variant', index)
+        for split in (1, 3):
+            rt.set_option('conv_split_k', split)
+            for in_shape, oc, k, s, p, batch in [((72, 19, 19), 88, (3, 3), (1, 1), (1, 1), 2),
+                                                  ((200, 8, 8), 136, (1, 1), (1, 1), (0, 0), 1),
+                                                  ((20, 37, 37), 24, (5, 5), (2, 2), (2, 2), 1)]:
+                graph = single_op_graph(in_shape, lambda b, v: ios.conv2d(b, [[v]], oc, k, s, p, 1, 'relu', is_exit=True))
+                x = np.random.default_rng(1).standard_normal((batch, *in_shape)).astype(np.float32)
+                got = rt.graph_inference(graph, batch, x)
+                want = ios_oracle.run(graph, x, bf16_convs=matrix_path_convs(graph, batch))
+                assert_close(got, want, f'{name} split {split} conv {in_shape}->{oc} {k}')
+                np.testing.assert_array_equal(got, rt.graph_inference(graph, batch, x))
+    assert tried >= 5
+
+
+def test_reduced_precision_network_under_parallel_schedules():
+    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    graph.sequential_schedule()
+    greedy = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    greedy.greedy_schedule(8)
+    x = np.random.default_rng(1).standard_normal((2, *graph.enter_node.output_shape)).astype(np.float32)
+    rt.set_option('precision', 'bf16')
+    convs = matrix_path_convs(graph, 2)
+    assert len(convs) == 94
+    want = ios_oracle.run(graph, x, bf16_convs=convs)
+    want_fp32 = ios_oracle.run(graph, x)
+    for executor, g in (('streams', graph), ('fused', greedy), ('fused_graph', greedy)):
+        rt.set_option('executor', executor)
+        with rt.Session(g, 2) as session:
+            session.load_weights()
+            session.set_input(x)
+            for _ in range(2):
+                session.run()
+            got = session.output()
+        # 94 layers deep, a different rounding of one operand (summation order before it) can flip a bfloat16 rounding
+        # downstream: the bfloat16 oracle is matched at the rounding tolerance, a little tighter than the fp32 one
+        assert_close_reduced(got, want, f'bf16 inception {executor}')
+        assert_close_reduced(got, want_fp32, f'bf16 inception {executor} against fp32')
+        assert np.abs(got - want).max() <= np.abs(got - want_fp32).max() * 1.5 + 1e-4
 
 
 def test_merged_convolutions_match_unmerged():

@@ -194,3 +194,15 @@ def test_graph_interpreter_on_small_graph_matches_brute_force():
 def Value_slice(value, begin, end):
     from ios.ir import Value
     return Value(value.node, begin, end)
+
+
+def test_bf16_rounding_is_round_to_nearest_even():
+    """The oracle's bfloat16 view of an operand against the bit-level definition (add 0x7fff + lsb, truncate)."""
+    import torch
+    rng = np.random.default_rng(11)
+    x = np.concatenate([rng.standard_normal(4096).astype(np.float32) * 10.0 ** rng.integers(-6, 6, 4096),
+                        np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.0e38, -2.5e-39], dtype=np.float32)]).astype(np.float32)
+    bits = x.view(np.uint32).astype(np.uint64)
+    want = (((bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000) & 0xFFFFFFFF).astype(np.uint32).view(np.float32)
+    got = ios_oracle.to_bf16(torch.from_numpy(x)).numpy()
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
