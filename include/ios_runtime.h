@@ -65,6 +65,8 @@ const char *ios_last_error(void);
  *       cudnnFind-based selection (src/ios/ios_runtime.cu:150-205); "clear_tuning" = anything forgets them;
  *   "split_k_reduce" = "inline" (the last block of a tile adds the split-K slices inside the convolution kernel)
  *       | "kernel" (a second kernel adds them); same results bit for bit;
+ *   "precision" = "fp32" | "bf16": reduced-precision mode of the matrix-path convolutions (bfloat16 operands, fp32
+ *       accumulation), the counterpart of the reference's USE_FLOAT16 build option (src/ios/ios_runtime.cu:19-43);
  *   "conv_variant" = index or -1 and "conv_split_k" = count or 0 force one convolution kernel configuration (testing). */
 int ios_set_option(const char *key, const char *value);
 
