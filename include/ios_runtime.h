@@ -58,10 +58,10 @@ int graph_inference(const char *graph_json, int batch_size, float *input, int nu
 const char *ios_last_error(void);
 
 /* Options (set them before sessions are created):
- *   "executor" = "streams" (one HIP stream per group, event fork/join) | "graph" (the same, captured into a hipGraph
- *       and replayed) | "fused" (the groups of a stage share one kernel launch per level) | "fused_graph" (fused
- *       launches inside a hipGraph);
- *   "autotune" = "0" | "1": measure convolution kernel configurations on first use, like the reference's
+ *   "executor" = "fused" (default: the groups of a stage share one kernel launch per level) | "fused_graph" (fused
+ *       launches inside a hipGraph) | "streams" (one HIP stream per group, event fork/join) | "graph" (the stream form
+ *       captured into a hipGraph and replayed);
+ *   "autotune" = "1" (default) | "0": measure convolution kernel configurations on first use, like the reference's
  *       cudnnFind-based selection (src/ios/ios_runtime.cu:150-205); "clear_tuning" = anything forgets them;
  *   "split_k_reduce" = "inline" (the last block of a tile adds the split-K slices inside the convolution kernel)
  *       | "kernel" (a second kernel adds them); same results bit for bit;

@@ -76,8 +76,10 @@ private:
     size_t arena_floats_ = 0;
     void *table_ = nullptr;
     size_t table_bytes_ = 0;
-    ExecMode exec_mode_ = ExecMode::Streams;
-    bool autotune_ = false;
+    // defaults: fused stage launches (stream fork / join costs more than the batch-1 kernels it would overlap) and
+    // measured kernel configurations, like the reference's exhaustive algorithm search on first sight of a shape
+    ExecMode exec_mode_ = ExecMode::Fused;
+    bool autotune_ = true;
     int forced_variant_ = -1;
     int forced_split_k_ = 0;
 };

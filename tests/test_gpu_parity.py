@@ -33,10 +33,12 @@ def default_options():
     rt.set_option('conv_variant', -1)
     rt.set_option('conv_split_k', 0)
     rt.set_option('executor', 'streams')
+    rt.set_option('autotune', 0)            # closed-form kernel configurations keep the suite short and repeatable
     rt.set_option('split_k_reduce', 'inline')
     rt.set_option('precision', 'fp32')
     yield
     rt.set_option('precision', 'fp32')
+    rt.set_option('autotune', 0)
     rt.set_option('conv_variant', -1)
     rt.set_option('conv_split_k', 0)
     rt.set_option('executor', 'streams')
