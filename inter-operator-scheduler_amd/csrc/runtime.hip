@@ -142,7 +142,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     IOS_HIP(hipEventCreate(&stop));
     // one winner per footprint budget: the whole device, a half, a quarter, an eighth (threads in flight);
     // a convolution that shares its stage with other groups uses the winner of the matching budget
-    const double capacity = (double)num_cus_ * 2048.0;
+    const double capacity = (double)num_cus_ * (double)share_threads_per_cu_;
     struct Candidate {
         ConvLaunch launch;
         float ms;
@@ -200,6 +200,27 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
             return cand.fusable && (!fit || cand.footprint <= capacity / (1 << c));
         };
         found[c] = false;
+        if (c > 0 && share_cost_rule_) {
+            // soft form: time weighted by the share of the device the kernel holds while 2^c - 1 neighbours want theirs
+            auto score = [&](const Candidate &cand) { return cand.ms * (1.0 + ((1 << c) - 1) * cand.footprint / capacity); };
+            std::vector<size_t> order;
+            for (size_t i = 0; i < candidates.size(); i++)
+                if (candidates[i].fusable) order.push_back(i);
+            std::sort(order.begin(), order.end(), [&](size_t a, size_t b) { return score(candidates[a]) < score(candidates[b]); });
+            double best = 1e300;
+            for (size_t n = 0; n < order.size() && n < 3; n++) {
+                Candidate &cand = candidates[order[n]];
+                if (!refined[order[n]]) {
+                    cand.ms = std::min(cand.ms, measure(cand.launch, 16));
+                    refined[order[n]] = 1;
+                }
+                if (score(cand) < best) {
+                    best = score(cand);
+                    result.best[c] = cand.launch;
+                    found[c] = true;
+                }
+            }
+        }
         for (int pass = 0; pass < 2 && !found[c]; pass++) {
             int taken = 0;
             float best = 1e30f;
@@ -296,6 +317,14 @@ void DeviceContext::set_option(const std::string &key, const std::string &value)
         const int v = atoi(value.c_str());
         if (v < 0 || v > 64) throw std::runtime_error("option conv_split_k: expected 0..64");
         forced_split_k_ = v;
+    } else if (key == "share_rule") {
+        if (value == "cost") share_cost_rule_ = true;
+        else if (value == "budget") share_cost_rule_ = false;
+        else throw std::runtime_error("option share_rule: expected cost or budget");
+    } else if (key == "share_threads_per_cu") {
+        const int v = atoi(value.c_str());
+        if (v < 64 || v > 4096) throw std::runtime_error("option share_threads_per_cu: expected 64..4096");
+        share_threads_per_cu_ = v;
     } else if (key == "precision") {
         if (value == "fp32") bf16_ = false;
         else if (value == "bf16") bf16_ = true;
