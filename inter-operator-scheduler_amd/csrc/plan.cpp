@@ -590,12 +590,18 @@ private:
         plan_.output = view_of(out_node);
         plan_.output_name = nodes_[out_node].name;
         std::vector<int> share(plan_.convs.size(), 1);
-        for (const PlanOp &op : plan_.ops)
-            if (op.conv >= 0 && op.stage >= 0) {
-                int busy = 0;
-                for (const auto &group : plan_.stages[op.stage]) busy += group.empty() ? 0 : 1;
-                share[op.conv] = std::max(1, busy);
-            }
+        // a convolution shares the device with the operators at the same position of the other groups of its stage
+        // (the fused executor runs position after position); in a multi-group stage it counts at least two, because
+        // it must be able to run inside a fused launch even when it is the only operator left at its position
+        for (const auto &stage : plan_.stages)
+            for (const auto &group : stage)
+                for (size_t pos = 0; pos < group.size(); pos++) {
+                    const PlanOp &op = plan_.ops[group[pos]];
+                    if (op.conv < 0) continue;
+                    int busy = 0;
+                    for (const auto &other : stage) busy += other.size() > pos ? 1 : 0;
+                    share[op.conv] = stage.size() > 1 ? std::max(2, busy) : 1;
+                }
         for (size_t i = 0; i < plan_.convs.size(); i++) {
             PlanConv &conv = plan_.convs[i];
             if (!conv.matrix_path) continue;
