@@ -166,10 +166,10 @@ struct ConvTiled {
     static constexpr int LDA = BM + PAD, LDB = BN + PAD;
     static constexpr int TILE_FLOATS = 2 * BK * (LDA + LDB);
     static constexpr int RED_FLOATS = (WK - 1) * BM * BN;
-    // Accumulators + prefetched operands per lane: bodies above the budget would lower the occupancy of every
-    // other operator inside a fused stage launch; they only run as stand-alone kernels.
-    static constexpr int LANE_REGS = BM * BN / (64 * WM * WN) + PD * (4 * ((BK * BM / 4 + T - 1) / T) + BK * BN / T);
-    static constexpr bool FUSABLE = LANE_REGS <= 56;
+    // The LDS-tiled bodies need 85 registers and more per lane; inside a fused stage launch they would lower the
+    // occupancy of every other operator (the wave-split bodies that serve small problems need 32-72), so they
+    // only run as stand-alone kernels.
+    static constexpr bool FUSABLE = false;
     static constexpr int SMEM_FLOATS = TILE_FLOATS > RED_FLOATS ? TILE_FLOATS : RED_FLOATS;
 
     // one block: output tile `tile` of group `g`, K slice `z`; smem holds SMEM_FLOATS floats, 16-byte aligned

@@ -113,7 +113,7 @@ ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only
         return best;
     }
     static const int tiled_mid = variant_by_name("m64n64k16_w2x2x1_t32");
-    if (blocks_of(tiled_mid) >= 4LL * num_cus) {
+    if (!fusable_only && blocks_of(tiled_mid) >= 4LL * num_cus) {
         static const int by_size[] = {variant_by_name("m128n128k16_w2x2x1_t32"), variant_by_name("m128n64k16_w2x2x1_t32"),
                                       variant_by_name("m64n128k16_w2x2x1_t32")};
         best.variant = tiled_mid;

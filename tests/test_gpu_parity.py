@@ -230,7 +230,7 @@ def test_fused_stage_launch_covers_every_operator_kind():
     for split in (0, 3):
         rt.set_option('conv_split_k', split)
         names = rt.device_info()['conv_variants']
-        for variant in (-1, names.index('m64n64k16_w2x2x1_t32'), names.index('wq_m32n16_w8_t16'), names.index('ws_m32n16_w16_t16')):
+        for variant in (-1, names.index('wq_m32n32_w4_t16'), names.index('wq_m32n16_w8_t16'), names.index('ws_m32n16_w16_t16')):
             rt.set_option('conv_variant', variant)
             for batch in (1, 2):
                 x = np.random.default_rng(5).standard_normal((batch, 16, 14, 14)).astype(np.float32)
@@ -327,7 +327,7 @@ def test_network_matches_oracle_under_every_schedule_and_executor(name, make, ba
         return outs
 
     run_all(pinned=False)
-    rt.set_option('conv_variant', rt.device_info()['conv_variants'].index('m32n16k64_w2x1x2_t16'))
+    rt.set_option('conv_variant', rt.device_info()['conv_variants'].index('wq_m32n16_w8_t16'))
     rt.set_option('conv_split_k', 2)
     outs = run_all(pinned=True)
     first = outs[('streams', 'sequential')]
