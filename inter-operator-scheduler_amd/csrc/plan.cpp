@@ -662,7 +662,8 @@ std::string describe_plan(const Plan &plan) {
                << ",\"kw\":" << p.KW << ",\"sh\":" << p.sh << ",\"sw\":" << p.sw << ",\"ph\":" << p.ph << ",\"pw\":" << p.pw
                << ",\"groups\":" << p.groups << ",\"act\":" << p.act << ",\"pre_relu\":" << p.pre_relu << "}";
             if (c.matrix_path) {
-                os << ",\"variant\":\"" << conv_variant(c.launch.variant).name << "\",\"split_k\":" << c.launch.split_k;
+                os << ",\"variant\":\"" << conv_variant(c.launch.variant).name << "\",\"split_k\":" << c.launch.split_k
+                   << ",\"fusable\":" << (conv_variant(c.launch.variant).fusable() ? "true" : "false");
             }
         }
         if (op.kind == OpKind::Nary) os << ",\"inputs\":" << op.srcs.size() << ",\"accumulate\":" << op.accumulate;

@@ -77,3 +77,22 @@ def test_host_planner_rejects_bad_documents():
     assert b'unsupported type softmax' in rt.get_lib().ios_last_error()
     with pytest.raises(RuntimeError):
         rt.plan_describe(graph, 0)
+
+
+def test_convolutions_of_parallel_stages_get_kernels_that_can_share_a_launch():
+    """Host planner, closed-form kernel choice: every matrix-path convolution of a multi-group stage must be able
+    to run inside a fused stage launch, at batch 1 and at a batch large enough for the LDS-tiled kernels."""
+    import collections
+    for batch in (1, 64):
+        graph = ios.models.inception_v3()
+        graph.greedy_schedule(8)
+        ops = rt.plan_describe(graph, batch)
+        groups = collections.defaultdict(set)
+        for op in ops:
+            groups[op['stage']].add(op['group'])
+        shared = [op for op in ops if op['kind'] == 'conv_mfma' and len(groups[op['stage']]) > 1]
+        alone = [op for op in ops if op['kind'] == 'conv_mfma' and len(groups[op['stage']]) == 1]
+        assert len(shared) > 60 and alone
+        assert all(op['fusable'] for op in shared), [op['variant'] for op in shared if not op['fusable']]
+    # alone on the device at batch 64 the large layers take the LDS-tiled kernels, which are not fusable
+    assert any(not op['fusable'] for op in alone)
