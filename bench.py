@@ -159,6 +159,8 @@ def main():
     parser.add_argument('--search', default='measured', choices=['measured', 'analytic'],
                         help="cost model of the schedule search: on-device stage measurements (default) or the "
                              "closed-form model (no device probes; keeps profiler traces small)")
+    parser.add_argument('--search-number', type=int, default=6, help='passes per stage probe of the schedule search')
+    parser.add_argument('--search-repeat', type=int, default=3, help='probes per candidate stage of the schedule search')
     parser.add_argument('--no-sweep', action='store_true', help='skip the batch 16 / 64 sweep')
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     parser.add_argument('--no-configs', action='store_true', help='skip the other four configuration networks')
@@ -193,7 +195,7 @@ def main():
     t0 = time.time()
     cost_model = ios.IOSCostModel() if args.search == 'measured' else ios.AnalyticCostModel()
     optimized = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
-                             warmup=2, number=6, repeat=3)
+                             warmup=2, number=args.search_number, repeat=args.search_repeat)
     search_s = time.time() - t0
     graph.sequential_schedule()
 
