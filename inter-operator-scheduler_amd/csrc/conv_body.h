@@ -563,6 +563,15 @@ struct ConvWsplit {
 #pragma unroll
     for (int j = 0; j < TN; j++) n_kill[j] = n_ok[j] ? 0u : kOutOfRange;
 
+    // the bias of the outputs this lane finishes in the epilogue, requested now so that its latency hides behind the K loop
+    constexpr int EPW = (E + NW - 1) / NW;
+    float bias_pre[EPW];
+#pragma unroll
+    for (int t = 0; t < EPW; t++) {
+        const int e = min(wave + t * NW, E - 1);
+        const int m = m0 + (e / (M::ACC * TN)) * MT + M::row(e % M::ACC, lane);
+        bias_pre[t] = a.bias[g * a.OCg + min(m, a.OCg - 1)];
+    }
     typename M::acc_t acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
@@ -778,7 +787,10 @@ struct ConvWsplit {
         __syncthreads();
         if (*last_flag == 0) return;
     }
-    for (int e = wave; e < E; e += NW) {
+#pragma unroll
+    for (int t = 0; t < EPW; t++) {
+        const int e = wave + t * NW;
+        if (e >= E) break;
         float sum = 0.f;
         if (a.split_k > 1) {
             for (int s2 = 0; s2 < a.split_k; s2++)
@@ -795,7 +807,7 @@ struct ConvWsplit {
         if (m < a.OCg && nn < a.Npix) {
             const int b = (int)fast_div((unsigned)nn, a.div_ohw);
             const int r = nn - b * a.OHW;
-            a.y[(long long)b * a.y_bs + ((long long)g * a.OCg + m) * a.OHW + r] = apply_act(sum + a.bias[g * a.OCg + m], a.act);
+            a.y[(long long)b * a.y_bs + ((long long)g * a.OCg + m) * a.OHW + r] = apply_act(sum + bias_pre[t], a.act);
         }
     }
 }   // run
