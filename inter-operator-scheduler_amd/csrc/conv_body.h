@@ -1,4 +1,10 @@
-// Implicit-GEMM convolution on the CDNA4 fp32 matrix cores.
+// Device-side bodies of the convolution kernels; included by the translation units that instantiate them
+// (the stand-alone kernels and the fused stage kernel).
+//
+// Implicit-GEMM convolution on the CDNA4 fp32 matrix cores, in two forms: ConvTiled stages operand tiles in LDS
+// (large problems), ConvWsplit feeds the matrix cores straight from global memory and divides K among the
+// wavefronts of a block (small and medium problems, and the bfloat16 mode).  This comment describes ConvTiled;
+// ConvWsplit is described at its definition.
 //
 // GEMM view per group:  Y[m][n] = sum_k Wp[k][m] * X_im2col[k][n]
 //   m = output channel inside the group (OCg), n = flattened (image, oh, ow) pixel,
@@ -20,8 +26,6 @@
 // back and invalidate whole L2s); everything else is M x N tiling.
 // The epilogue adds the bias, applies the activation and stores through the output view, i.e. directly
 // into the consumer's channel window when the output lives inside a concat buffer.
-// Device-side bodies of the convolution kernels; included by the translation units that instantiate them
-// (the stand-alone kernels and the fused stage kernel).
 #pragma once
 
 #include "kernels.h"

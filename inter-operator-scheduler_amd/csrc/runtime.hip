@@ -1,10 +1,11 @@
 // Stage executor, timers and device context.
 //
-// A forward pass walks the plan's stages.  Group g of a stage is issued to stream g of a fixed pool;
-// stream 0 is the main stream.  A multi-group stage forks (the extra streams wait on an event recorded on
-// the main stream) and joins (the main stream waits on one event per extra stream), so stage boundaries
-// are device-side dependencies and the host never blocks inside a pass.  In graph mode the same
-// issue sequence is captured once into a hipGraph and replayed.
+// A forward pass walks the plan's stages.  Fused executor (default): a multi-group stage is issued as one
+// fused launch per chain position on the main stream (see build_fused).  Streams executor: group g of a stage
+// is issued to stream g of a fixed pool; stream 0 is the main stream; a multi-group stage forks (the extra
+// streams wait on an event recorded on the main stream) and joins (the main stream waits on one event per
+// extra stream).  Either way stage boundaries are device-side dependencies and the host never blocks inside
+// a pass.  The graph modes capture the same issue sequence once into a hipGraph and replay it.
 //
 // Timing follows the reference runtime (src/ios/ios_runtime.cu:1328-1455): graph / block latency is the
 // mean over `number` individually bracketed passes per repeat, with optional per-stage times from events
