@@ -292,6 +292,20 @@ def main():
             configs[name] = {'sequential_ms': c_seq['wall'], f'{label}_ms': c_par['wall'],
                              'network_roofline_ms': network_roofline_ms(ops_c, parallel=False)}
         result['other_configs_batch1'] = configs
+        # the model variants the reference's own result table uses (its large RandWire / NASNet and SqueezeNet 1.0 with
+        # bypass), sequential and greedy schedules: points of comparison with that table, not part of the metric
+        variants = {}
+        for name, make in (('squeezenet', ios.models.squeezenet), ('randwire_large', ios.models.randwire_large),
+                           ('nasnet_large', ios.models.nasnet_large)):
+            g = make(init_seed=0, init_scheme='he_normal')
+            g.sequential_schedule()
+            scheduled = make(init_seed=0, init_scheme='he_normal')
+            scheduled.greedy_schedule(4)
+            xc = np.random.default_rng(1).standard_normal((1, *g.enter_node.output_shape)).astype(np.float32)
+            v_seq, _ = timed_latency(rt, np, g, 1, xc, 50, 5)
+            v_par, _ = timed_latency(rt, np, scheduled, 1, xc, 50, 5)
+            variants[name] = {'sequential_ms': v_seq['wall'], 'greedy_ms': v_par['wall']}
+        result['reference_table_variants_batch1'] = variants
 
     if not args.no_cpu:
         import torch
