@@ -96,3 +96,12 @@ def test_convolutions_of_parallel_stages_get_kernels_that_can_share_a_launch():
         assert all(op['fusable'] for op in shared), [op['variant'] for op in shared if not op['fusable']]
     # alone on the device at batch 64 the large layers take the LDS-tiled kernels, which are not fusable
     assert any(not op['fusable'] for op in alone)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    done = subprocess.run([sys.executable, os.path.join(root, 'bench.py'), '--gpus', '2'], capture_output=True, text=True, timeout=60)
+    assert done.returncode != 0
+    assert 'single-GPU' in done.stderr
