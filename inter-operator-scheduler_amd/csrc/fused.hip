@@ -6,7 +6,7 @@
 namespace ios {
 
 template <int T>
-__global__ __launch_bounds__(T, 1024 / T) void fused_kernel(const WorkItem *__restrict__ items, int num_items) {
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fused_kernel(const WorkItem *__restrict__ items, int num_items) {
     extern __shared__ floatx4 fused_smem[];
     float *smem = reinterpret_cast<float *>(fused_smem);
     const int bid = blockIdx.x;

@@ -59,6 +59,8 @@ DirectConvArgs make_direct_conv_args(const ConvProblem &p, const TensorView &x, 
     a.x_bs = x.bstride;
     a.y_bs = y.bstride;
     a.p = p;
+    const unsigned long long x_bytes = ((unsigned long long)(p.B - 1) * x.bstride + (unsigned long long)p.IC * p.H * p.W) * 4ull;
+    a.x_bytes = x_bytes < (1ull << 31) ? (unsigned)x_bytes : 0u;
     *blocks = blocks_for((long long)p.B * p.OC * p.OH * p.OW, 256, 8192);
     return a;
 }

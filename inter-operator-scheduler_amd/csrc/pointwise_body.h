@@ -152,7 +152,13 @@ struct DirectConvArgs {
     float *y;
     long long x_bs, y_bs;
     ConvProblem p;
+    unsigned x_bytes;   // extent of the input view in bytes when it is below 2^31 (branch-free depth-wise loads), else 0
 };
+
+// raw buffer loads as in the matrix-path convolution: an offset with the top bit set is out of range and reads zero
+__device__ __forceinline__ float pw_buffer_load(__amdgpu_buffer_rsrc_t r, unsigned byte_offset) {
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_offset, 0, 0));
+}
 
 template <int KH, int KW>
 __device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, int num_blocks) {
@@ -161,6 +167,7 @@ __device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, 
     const unsigned plane = (unsigned)(p.OH * p.OW);
     const unsigned per_image = (unsigned)p.OC * plane;
     const unsigned total = per_image * (unsigned)p.B;
+    const int relu_floor = p.pre_relu ? 0 : (int)0x80000000;   // folded ReLU as an integer max
     for (unsigned i = block * blockDim.x + threadIdx.x; i < total; i += num_blocks * blockDim.x) {
         const unsigned b = i / per_image;
         const unsigned o = i - b * per_image;
@@ -168,21 +175,38 @@ __device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, 
         const unsigned r = o - c * plane;
         const int oh = (int)(r / (unsigned)p.OW);
         const int ow = (int)r - oh * p.OW;
-        const float *xc = a.x + (long long)b * a.x_bs + (long long)c * p.H * p.W;
         const float *wc = a.w + (size_t)c * kh_n * kw_n;
         const int h0 = oh * p.sh - p.ph, w0 = ow * p.sw - p.pw;
         float acc = a.bias[c];
+        if (KH > 0 && a.x_bytes != 0) {
+            // fixed window: every tap is one independent load, taps outside the image get the out-of-range bit, so
+            // the KH * KW loads of an output are in flight together instead of one bounds-checked load after another
+            const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a.x), 0, a.x_bytes, 0x00020000);
+            const unsigned base = (unsigned)(((long long)b * a.x_bs + (long long)c * p.H * p.W + (long long)h0 * p.W + w0) * 4);
+            float v[KH > 0 ? KH * KW : 1];
 #pragma unroll
-        for (int i2 = 0; i2 < kh_n; i2++) {
-            const int h = h0 + i2;
-            if ((unsigned)h >= (unsigned)p.H) continue;
+            for (int i2 = 0; i2 < KH; i2++) {
+                const unsigned row_kill = (unsigned)(h0 + i2) < (unsigned)p.H ? 0u : 0x80000000u;
 #pragma unroll
-            for (int j = 0; j < kw_n; j++) {
-                const int ww = w0 + j;
-                if ((unsigned)ww >= (unsigned)p.W) continue;
-                float v = xc[h * p.W + ww];
-                if (p.pre_relu) v = fmaxf(v, 0.f);
-                acc = fmaf(v, wc[i2 * kw_n + j], acc);
+                for (int j = 0; j < KW; j++) {
+                    const unsigned kill = (unsigned)(w0 + j) < (unsigned)p.W ? row_kill : 0x80000000u;
+                    v[i2 * KW + j] = pw_buffer_load(xr, (base + (unsigned)(i2 * p.W + j) * 4u) | kill);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < KH * KW; t++) acc = fmaf(__int_as_float(max(__float_as_int(v[t]), relu_floor)), wc[t], acc);
+        } else {
+            const float *xc = a.x + (long long)b * a.x_bs + (long long)c * p.H * p.W;
+            for (int i2 = 0; i2 < kh_n; i2++) {
+                const int h = h0 + i2;
+                if ((unsigned)h >= (unsigned)p.H) continue;
+                for (int j = 0; j < kw_n; j++) {
+                    const int ww = w0 + j;
+                    if ((unsigned)ww >= (unsigned)p.W) continue;
+                    float v = xc[h * p.W + ww];
+                    if (p.pre_relu) v = fmaxf(v, 0.f);
+                    acc = fmaf(v, wc[i2 * kw_n + j], acc);
+                }
             }
         }
         a.y[(long long)b * a.y_bs + o] = act_apply(acc, p.act);
