@@ -83,12 +83,16 @@ __device__ __forceinline__ void pool3x3_body(const PoolArgs &a, int block, int n
         float *yc = a.y + (long long)b * a.y_bs + (long long)c * p.OH * p.OW + ow;
         const int w0 = ow * p.sw - p.pw;
         const bool c0 = (unsigned)w0 < (unsigned)p.W, c1 = (unsigned)(w0 + 1) < (unsigned)p.W, c2 = (unsigned)(w0 + 2) < (unsigned)p.W;
+        // clamped addresses and selects instead of conditional loads: the loads of a window are independent and in
+        // flight together
+        const int wa = min(max(w0, 0), p.W - 1), wb = min(max(w0 + 1, 0), p.W - 1), wc2 = min(max(w0 + 2, 0), p.W - 1);
         auto row = [&](int h) -> float {
-            if ((unsigned)h >= (unsigned)p.H) return neutral;
-            const float *xr = xc + h * p.W + w0;
-            const float v0 = c0 ? xr[0] : neutral;
-            const float v1 = c1 ? xr[1] : neutral;
-            const float v2 = c2 ? xr[2] : neutral;
+            const bool in_h = (unsigned)h < (unsigned)p.H;
+            const float *xr = xc + min(max(h, 0), p.H - 1) * p.W;
+            const float l0 = xr[wa], l1 = xr[wb], l2 = xr[wc2];
+            const float v0 = (c0 && in_h) ? l0 : neutral;
+            const float v1 = (c1 && in_h) ? l1 : neutral;
+            const float v2 = (c2 && in_h) ? l2 : neutral;
             return is_max ? fmaxf(fmaxf(v0, v1), v2) : (v0 + v1) + v2;
         };
         auto combine = [&](float r0, float r1, float r2) -> float {
