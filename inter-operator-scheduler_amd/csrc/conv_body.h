@@ -501,17 +501,22 @@ __device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int bloc
 // BF16 (reduced-precision mode): filters are packed as bfloat16 in the quad layout (a lane's four k are one 8-byte
 // load), inputs are rounded to bfloat16 (nearest even) after loading, and one v_mfma_f32_16x16x16_bf16 consumes
 // the four k of a lane group at once - the same k assignment as QUAD; accumulation stays fp32.
-template <int MT, int TM, int TN, int NW, int U, bool QUAD = false, int D = 2, bool BF16 = false>
+//
+// CP: channel padding of the packed filters when it should differ from the default (8, or the batch with QUAD); 4 serves
+// layers with a handful of input channels (the first layer of an image network), whose K would otherwise be mostly padding.
+template <int MT, int TM, int TN, int NW, int U, bool QUAD = false, int D = 2, bool BF16 = false, int CP = 0>
 struct ConvWsplit {
     using M = Mfma<MT>;
     static constexpr int BM = TM * MT, BN = TN * MT;
     static constexpr int E = TM * TN * M::ACC;
     static constexpr int THREADS = 64 * NW;
     static constexpr int SMEM_FLOATS = NW * E * 64;
-    static constexpr int CPAD = QUAD ? U * M::KSTEP : 8;   // channel padding of the packed filters this kernel expects
+    static constexpr int CPAD = CP ? CP : (QUAD ? U * M::KSTEP : 8);   // channel padding of the packed filters this kernel expects
+    static_assert(CP == 0 || (!QUAD && CP % M::KSTEP == 0), "a k-step must lie inside one filter tap");
     static constexpr bool KQUAD = QUAD;                    // packed filters are [k / 4][m][4] instead of [k][m]
     // accumulators + staged operands per lane decide whether the body fits the register budget of a fused launch
-    static constexpr bool FUSABLE = E + D * U * (TM + TN) <= 56;
+    // (the channel-padding-4 forms serve first layers, which are stages of their own: kept out of the fused launches)
+    static constexpr bool FUSABLE = CP == 0 && E + D * U * (TM + TN) <= 56;
     static constexpr bool KBF16 = BF16;                    // packed filters hold bfloat16
     static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
     static_assert(!BF16 || (QUAD && MT == 16 && U == 4), "the bfloat16 path is the 16 x 16 x 16 form of the quad layout");
@@ -875,6 +880,12 @@ struct ConvWsplit {
     X(50, "wb_m64n32_w8", 16, 4, 2, 8, 4, true, 2, true)      \
     X(51, "wb_m64n32_w4_d4", 16, 4, 2, 4, 4, true, 4, true)   \
     X(52, "wb_m64n64_w4", 16, 4, 4, 4, 4, true, 2, true)
-constexpr int kNumConvVariants = 53;
+// X(index, name, MT, TM, TN, NW, U, QUAD, D, BF16): wave-split configurations with channels padded to 4
+#define IOS_WSPLIT_C4_VARIANTS(X)                                \
+    X(53, "ws_m32n32_w1_t16_c4", 16, 2, 2, 1, 4, false, 2, false) \
+    X(54, "ws_m32n64_w1_t16_c4", 16, 2, 4, 1, 4, false, 2, false) \
+    X(55, "ws_m32n32_w2_t16_c4", 16, 2, 2, 2, 4, false, 2, false) \
+    X(56, "ws_m32n16_w4_t16_c4", 16, 2, 1, 4, 4, false, 2, false)
+constexpr int kNumConvVariants = 57;
 
 }  // namespace ios

@@ -34,8 +34,13 @@ struct VariantEntry {
     {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::CPAD, QUAD, \
       ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::FUSABLE, BF16},      \
      conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>>, ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::SMEM_FLOATS},
+#define IOS_WSPLIT_C4_ENTRY(IDX, NAME, MT, TM, TN, NW, U, QUAD, D, BF16)                                                                  \
+    {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::CPAD, QUAD, \
+      ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::FUSABLE, BF16},                                                                 \
+     conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>>, ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::SMEM_FLOATS},
 
-static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)};
+static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)
+                                             IOS_WSPLIT_C4_VARIANTS(IOS_WSPLIT_C4_ENTRY)};
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 static_assert(kNumVariants == kNumConvVariants, "variant lists and count disagree");
 

@@ -34,8 +34,15 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fus
         if constexpr (64 * NW <= T && ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::FUSABLE)              \
             ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::run(a, smem, tile, g, z);                       \
         break;
+#define IOS_CASE_WSPLIT_C4(IDX, NAME, MT, TM, TN, NW, U, QUAD, D, BF16)                                     \
+    case IDX:                                                                                      \
+        if constexpr (64 * NW <= T && ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::FUSABLE)           \
+            ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::run(a, smem, tile, g, z);                    \
+        break;
                 IOS_TILED_VARIANTS(IOS_CASE_TILED)
                 IOS_WSPLIT_VARIANTS(IOS_CASE_WSPLIT)
+                IOS_WSPLIT_C4_VARIANTS(IOS_CASE_WSPLIT_C4)
+#undef IOS_CASE_WSPLIT_C4
 #undef IOS_CASE_TILED
 #undef IOS_CASE_WSPLIT
                 default: break;
