@@ -9,7 +9,9 @@
  * sees the reference behaviour minus the exit().
  *
  * All pointers are owned by the caller and only used during the call.  Host buffers are float32,
- * C-contiguous, NCHW.  The library is not re-entrant: call it from one thread at a time.
+ * C-contiguous, NCHW.  The library keeps process-wide state like the reference (one device
+ * context, one stream pool); calls from several host threads are serialised by an internal lock, and
+ * ios_last_error() reports the most recent failure of any thread.
  * JSON documents are the wire format exported by ios.Graph.export_config() / Block.export_config()
  * (reference python/ios/ir.py:855-865,1038-1046).
  */

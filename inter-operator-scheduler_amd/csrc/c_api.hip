@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <string>
 
 #include "../../include/ios_runtime.h"
@@ -13,6 +14,9 @@
 namespace {
 
 std::string g_last_error;
+// The library keeps process-wide state (device context, stream pool, shared arena, configuration cache); calls from
+// several host threads are serialised here rather than left to race.
+std::recursive_mutex g_api_mutex;
 
 ios::LaunchChooser device_chooser() {
     ios::DeviceContext &ctx = ios::DeviceContext::get();
@@ -21,6 +25,7 @@ ios::LaunchChooser device_chooser() {
 
 template <typename F>
 int guarded(F &&body) {
+    std::lock_guard<std::recursive_mutex> lock(g_api_mutex);
     try {
         body();
         return 0;
@@ -91,6 +96,8 @@ int graph_inference(const char *graph_json, int batch_size, float *input, int nu
         ios::Plan plan = ios::build_plan(ios::PlanMode::Graph, doc, nullptr, batch_size, device_chooser());
         ios::Session session(std::move(plan), /*shared=*/true);
         session.set_input(input);
+        if (num_convs > 0 && (conv_names == nullptr || filter_data == nullptr || bias_data == nullptr))
+            throw std::runtime_error("conv_names, filter_data or bias_data is null");
         for (int i = 0; i < num_convs; i++) session.set_conv_weights(conv_names[i], filter_data[i], bias_data[i]);
         session.run();
         session.get_output(output);
@@ -152,6 +159,8 @@ void ios_session_destroy(ios_session *s) {
 int ios_session_set_conv_weights(ios_session *s, int num_convs, char **conv_names, float **filter_data, float **bias_data) {
     return guarded([&]() {
         ios::Session &session = unbox(s);
+        if (num_convs > 0 && (conv_names == nullptr || filter_data == nullptr || bias_data == nullptr))
+            throw std::runtime_error("conv_names, filter_data or bias_data is null");
         for (int i = 0; i < num_convs; i++) session.set_conv_weights(conv_names[i], filter_data[i], bias_data[i]);
     });
 }

@@ -91,6 +91,7 @@ public:
     // `shared` sessions live in the context's shared arena (one at a time), others own their memory
     Session(Plan plan, bool shared);
     ~Session();
+    void release() noexcept;   // frees device memory, events and the captured graph; safe to call twice
     Session(const Session &) = delete;
     Session &operator=(const Session &) = delete;
 

@@ -68,24 +68,27 @@ static std::string conv_signature(const ConvProblem &p) {
 void DeviceContext::load_tune_cache() {
     FILE *f = fopen(tune_cache_path_.c_str(), "r");
     if (f == nullptr) return;
-    int v[12];
-    // line: 12 problem integers, then kShareClasses pairs (variant name, split_k)
-    while (true) {
+    // line: 12 problem integers, then kShareClasses pairs (configuration name, split_k).  A line that does not parse
+    // (truncated write, a configuration name this build no longer has) is skipped: its shape is measured again.
+    char line[1024];
+    while (fgets(line, sizeof(line), f) != nullptr) {
+        std::istringstream in(line);
+        int v[12];
         bool ok = true;
-        for (int i = 0; i < 12 && ok; i++) ok = fscanf(f, "%d", &v[i]) == 1;
+        for (int i = 0; i < 12 && ok; i++) ok = static_cast<bool>(in >> v[i]);
         TunedConv entry;
         for (int c = 0; c < kShareClasses && ok; c++) {
-            char name[128];
+            std::string name;
             int split = 0;
-            ok = fscanf(f, "%127s %d", name, &split) == 2 && split >= 1;
+            ok = static_cast<bool>(in >> name >> split) && split >= 1 && split <= 64;
             int variant = -1;
             for (int i = 0; ok && i < conv_num_variants(); i++)
-                if (strcmp(conv_variant(i).name, name) == 0) variant = i;
+                if (name == conv_variant(i).name) variant = i;
             ok = ok && variant >= 0;
             entry.best[c].variant = variant;
             entry.best[c].split_k = split;
         }
-        if (!ok) break;
+        if (!ok) continue;
         std::ostringstream os;
         for (int i = 0; i < 12; i++) os << (i ? " " : "") << v[i];
         if (conv_variant(entry.best[0].variant).bf16) os << " bf16";   // reduced-precision entries have their own keys
@@ -138,9 +141,16 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     float *packed = tuning_buffer(2, conv_packed_floats_max(p) + p.OC);
     float *bias = packed + conv_packed_floats_max(p);
     hipStream_t stream = streams_[0];
-    hipEvent_t start, stop;
-    IOS_HIP(hipEventCreate(&start));
-    IOS_HIP(hipEventCreate(&stop));
+    struct EventPair {   // destroyed on every way out, a failing launch included
+        hipEvent_t start = nullptr, stop = nullptr;
+        ~EventPair() {
+            if (start != nullptr) (void)hipEventDestroy(start);
+            if (stop != nullptr) (void)hipEventDestroy(stop);
+        }
+    } events;
+    IOS_HIP(hipEventCreate(&events.start));
+    IOS_HIP(hipEventCreate(&events.stop));
+    const hipEvent_t start = events.start, stop = events.stop;
     // one winner per footprint budget: the whole device, a half, a quarter, an eighth (threads in flight);
     // a convolution that shares its stage with other groups uses the winner of the matching budget
     const double capacity = (double)num_cus_ * (double)share_threads_per_cu_;
@@ -241,8 +251,6 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
         }
         if (!found[c]) result.best[c] = conv_pick_launch(p, std::max(1, num_cus_ >> c), c > 0, bf16_);
     }
-    IOS_HIP(hipEventDestroy(start));
-    IOS_HIP(hipEventDestroy(stop));
     if (!tune_cache_path_.empty()) {
         FILE *f = fopen(tune_cache_path_.c_str(), "a");
         if (f != nullptr) {
@@ -365,12 +373,14 @@ Session::Session(Plan plan, bool shared) : plan_(std::move(plan)), ctx_(DeviceCo
     try {
         setup();
     } catch (...) {
-        if (owns_memory_ && base_ != nullptr) (void)hipFree(base_);
+        release();   // the destructor does not run for a constructor that throws
         throw;
     }
 }
 
-Session::~Session() {
+Session::~Session() { release(); }
+
+void Session::release() noexcept {
     (void)hipDeviceSynchronize();
     if (graph_exec_ != nullptr) (void)hipGraphExecDestroy(graph_exec_);
     if (graph_ != nullptr) (void)hipGraphDestroy(graph_);
@@ -383,6 +393,14 @@ Session::~Session() {
     if (stop_ != nullptr) (void)hipEventDestroy(stop_);
     if (owns_memory_ && fused_items_ != nullptr) (void)hipFree(fused_items_);
     if (owns_memory_ && base_ != nullptr) (void)hipFree(base_);
+    graph_exec_ = nullptr;
+    graph_ = nullptr;
+    fork_events_.clear();
+    join_events_.clear();
+    stage_events_.clear();
+    start_ = stop_ = nullptr;
+    fused_items_ = nullptr;
+    base_ = nullptr;
 }
 
 TensorView Session::tv(const ViewRef &v) const {
