@@ -886,6 +886,22 @@ struct ConvWsplit {
     X(54, "ws_m32n64_w1_t16_c4", 16, 2, 4, 1, 4, false, 2, false) \
     X(55, "ws_m32n32_w2_t16_c4", 16, 2, 2, 2, 4, false, 2, false) \
     X(56, "ws_m32n16_w4_t16_c4", 16, 2, 1, 4, 4, false, 2, false)
-constexpr int kNumConvVariants = 57;
+// X(index, name, MT, TM, TN, NW, U, QUAD, D, BF16): quad-load wave-split configurations on the 32 x 32 x 2 MFMA.  A
+// wavefront's input load covers two channels x 32 consecutive pixels (two full 128-byte lines) instead of four
+// channels x 16 pixels, and the instruction's ceiling is higher than that of the 16 x 16 x 4 form.
+#define IOS_WSPLIT_T32_VARIANTS(X)                                   \
+    X(57, "wq_m32n32_w8_t32", 32, 1, 1, 8, 8, true, 2, false)        \
+    X(58, "wq_m32n32_w16_t32", 32, 1, 1, 16, 8, true, 2, false)      \
+    X(59, "wq_m32n32_w4_t32", 32, 1, 1, 4, 8, true, 2, false)        \
+    X(60, "wq_m64n32_w8_t32", 32, 2, 1, 8, 8, true, 2, false)        \
+    X(61, "wq_m64n32_w4_t32", 32, 2, 1, 4, 8, true, 2, false)        \
+    X(62, "wq_m32n64_w8_t32", 32, 1, 2, 8, 8, true, 2, false)        \
+    X(63, "wq_m32n64_w4_t32", 32, 1, 2, 4, 8, true, 2, false)        \
+    X(64, "wq_m64n64_w8_t32", 32, 2, 2, 8, 8, true, 2, false)        \
+    X(65, "wq_m32n32_w8_t32_u4", 32, 1, 1, 8, 4, true, 2, false)     \
+    X(66, "wq_m64n32_w8_t32_u4", 32, 2, 1, 8, 4, true, 2, false)     \
+    X(67, "wq_m64n64_w4_t32_u4", 32, 2, 2, 4, 4, true, 2, false)     \
+    X(68, "wq_m64n32_w4_t32_u4_d4", 32, 2, 1, 4, 4, true, 4, false)
+constexpr int kNumConvVariants = 69;
 
 }  // namespace ios

@@ -40,7 +40,8 @@ struct VariantEntry {
      conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>>, ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::SMEM_FLOATS},
 
 static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)
-                                             IOS_WSPLIT_C4_VARIANTS(IOS_WSPLIT_C4_ENTRY)};
+                                             IOS_WSPLIT_C4_VARIANTS(IOS_WSPLIT_C4_ENTRY)
+                                             IOS_WSPLIT_T32_VARIANTS(IOS_WSPLIT_ENTRY)};
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 static_assert(kNumVariants == kNumConvVariants, "variant lists and count disagree");
 

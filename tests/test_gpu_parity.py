@@ -93,7 +93,7 @@ def test_conv_matches_oracle(case):
     assert_close(got, want, f'conv {case}')
 
 
-@pytest.mark.parametrize('variant', range(64))
+@pytest.mark.parametrize('variant', range(80))
 @pytest.mark.parametrize('split_k', [1, 3])
 def test_every_conv_kernel_variant(variant, split_k):
     names = rt.device_info()['conv_variants']
