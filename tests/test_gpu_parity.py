@@ -113,6 +113,19 @@ def test_every_conv_kernel_variant(variant, split_k):
         np.testing.assert_array_equal(got, got2)      # split-K reduction order is fixed
 
 
+@pytest.mark.parametrize('variant_name', ['ws_m32n32_w1_t16_c4', 'ws_m32n64_w1_t16_c4', 'ws_m32n32_w2_t16_c4', 'ws_m32n16_w4_t16_c4'])
+def test_first_layer_configurations_on_three_and_five_channel_inputs(variant_name):
+    """Channel padding 4: K = taps x 4 (3 channels) or taps x 8 (5 channels), strided, with and without padding."""
+    names = rt.device_info()['conv_variants']
+    rt.set_option('conv_variant', names.index(variant_name))
+    rt.set_option('conv_split_k', 1)
+    for in_shape, oc, k, s, p, batch in [((3, 41, 41), 32, (3, 3), (2, 2), (0, 0), 2), ((3, 23, 29), 39, (3, 3), (2, 2), (1, 1), 1),
+                                          ((5, 17, 17), 20, (5, 5), (1, 1), (2, 2), 3), ((1, 19, 19), 8, (7, 7), (2, 2), (3, 3), 1)]:
+        graph = single_op_graph(in_shape, lambda b, v: ios.conv2d(b, [[v]], oc, k, s, p, 1, 'relu', is_exit=True))
+        got, want = run_both(graph, batch)
+        assert_close(got, want, f'{variant_name} conv {in_shape}->{oc} {k}')
+
+
 @pytest.mark.parametrize('variant_name', ['m64n64k32_w2x2x1_t32', 'm32n32k64_w1x1x4_t32', 'm64n16k64_w4x1x1_t16',
                                           'm32n16k64_w2x1x2_t16', 'm128n64k16_w2x2x1_t32', 'ws_m32n16_w8_t16',
                                           'wq_m16n16_w16_t16', 'wq_m32n32_w16_t16', 'ws_m32n32_w16_t32'])
