@@ -246,10 +246,21 @@ def main():
             steps = max(10, args.steps // (b * 2))
             s_seq, out_seq = timed_latency(rt, np, graph, b, xb, steps, 3)
             s_opt, out_opt = timed_latency(rt, np, optimized, b, xb, steps, 3)
+            # the schedule searched at this batch size (the reference's batch-size specialisation, experiments/specialization)
+            rt.set_option('executor', args.search_executor)
+            t0 = time.time()
+            optimized_b = ios.optimize(graph, batch_size=b, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
+                                       warmup=2, number=args.search_number, repeat=args.search_repeat)
+            search_b = time.time() - t0
+            graph.sequential_schedule()
+            rt.set_option('executor', args.executor)
+            s_own, out_own = timed_latency(rt, np, optimized_b, b, xb, steps, 3)
             _, _, roof_b, _ = conv_roofline(rt, graph, b, xb)
             ops_b = rt.plan_describe(graph, b)
-            best = min(s_seq['wall'], s_opt['wall'])
+            best = min(s_seq['wall'], s_opt['wall'], s_own['wall'])
             sweep[str(b)] = {'sequential_ms': s_seq['wall'], 'dp_parallel_batch1_schedule_ms': s_opt['wall'],
+                             'dp_parallel_ms': s_own['wall'], 'search_seconds': search_b,
+                             'max_abs_diff_between_schedules': float(np.abs(out_seq - out_own).max()),
                              'images_per_s': b / (best * 1e-3),
                              'network_roofline_ms': network_roofline_ms(ops_b, parallel=False),
                              'fraction_of_network_roofline': network_roofline_ms(ops_b, parallel=False) / best,
