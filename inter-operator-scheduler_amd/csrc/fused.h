@@ -28,12 +28,21 @@ struct WorkItem {
     };
 };
 
+// Passed by value with the launch: a block finds its item from the kernel-argument segment alone (one scalar load,
+// no walk through the item table), then reads the item's fields from the table.
+constexpr int kMaxFusedItems = 16;    // = groups per stage
+constexpr int kFusedHeaderItems = 8;  // the schedule search builds stages of up to 8 groups; wider stages walk the table
+struct FusedHeader {
+    int num_items;
+    int first_block[kFusedHeaderItems];   // ascending; entries beyond num_items are unused
+};
+
 // Thread-block sizes the fused kernel is instantiated for.  A launch uses the size of its widest convolution body;
 // bodies that need fewer wavefronts let the surplus wavefronts of their blocks end at once (barriers only count
 // wavefronts that have not ended), the memory-bound bodies adapt to any block size.
 constexpr int kFusedThreadClasses[] = {256, 512, 1024};
 
 // Launch `num_items` items (device pointer) as one grid of `total_blocks` blocks of `threads` threads.
-void launch_fused(int threads, const WorkItem *device_items, int num_items, int total_blocks, int smem_bytes, hipStream_t stream);
+void launch_fused(int threads, const WorkItem *device_items, const FusedHeader &header, int total_blocks, int smem_bytes, hipStream_t stream);
 
 }  // namespace ios

@@ -6,12 +6,17 @@
 namespace ios {
 
 template <int T>
-__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fused_kernel(const WorkItem *__restrict__ items, int num_items) {
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fused_kernel(const WorkItem *__restrict__ items, FusedHeader header) {
     extern __shared__ floatx4 fused_smem[];
     float *smem = reinterpret_cast<float *>(fused_smem);
     const int bid = blockIdx.x;
-    int index = 0;
-    while (index + 1 < num_items && bid >= items[index + 1].first_block) index++;
+    int index = 0;   // number of further items that start at or before this block
+    if (header.num_items <= kFusedHeaderItems) {
+#pragma unroll
+        for (int i = 1; i < kFusedHeaderItems; i++) index += (i < header.num_items && bid >= header.first_block[i]) ? 1 : 0;
+    } else {
+        while (index + 1 < header.num_items && bid >= items[index + 1].first_block) index++;
+    }
     const WorkItem &item = items[index];
     const int local = bid - item.first_block;
     const int num_blocks = item.num_blocks;
@@ -83,13 +88,13 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fus
     }
 }
 
-void launch_fused(int threads, const WorkItem *device_items, int num_items, int total_blocks, int smem_bytes, hipStream_t stream) {
-    if (num_items < 1 || total_blocks < 1) throw std::runtime_error("fused launch: nothing to do");
+void launch_fused(int threads, const WorkItem *device_items, const FusedHeader &header, int total_blocks, int smem_bytes, hipStream_t stream) {
+    if (header.num_items < 1 || header.num_items > kMaxFusedItems || total_blocks < 1) throw std::runtime_error("fused launch: bad item count");
     const dim3 grid((unsigned)total_blocks);
     switch (threads) {
-        case 256: hipLaunchKernelGGL(fused_kernel<256>, grid, dim3(256), smem_bytes, stream, device_items, num_items); break;
-        case 512: hipLaunchKernelGGL(fused_kernel<512>, grid, dim3(512), smem_bytes, stream, device_items, num_items); break;
-        case 1024: hipLaunchKernelGGL(fused_kernel<1024>, grid, dim3(1024), smem_bytes, stream, device_items, num_items); break;
+        case 256: hipLaunchKernelGGL(fused_kernel<256>, grid, dim3(256), smem_bytes, stream, device_items, header); break;
+        case 512: hipLaunchKernelGGL(fused_kernel<512>, grid, dim3(512), smem_bytes, stream, device_items, header); break;
+        case 1024: hipLaunchKernelGGL(fused_kernel<1024>, grid, dim3(1024), smem_bytes, stream, device_items, header); break;
         default: throw std::runtime_error("fused launch: unsupported block size");
     }
 }

@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "plan.h"
+#include "fused.h"
 
 namespace ios {
 
@@ -135,6 +136,7 @@ private:
     hipEvent_t start_ = nullptr, stop_ = nullptr;
     struct FusedLaunch {
         int threads, first_item, num_items, total_blocks, smem_bytes;
+        FusedHeader header;
     };
     std::vector<std::vector<FusedLaunch>> fused_stages_;   // per stage; empty for single-group stages
     void *fused_items_ = nullptr;                          // device copy of all work items

@@ -657,17 +657,20 @@ void Session::build_fused() {
                 }
             widest = std::max(widest, 256);   // narrowest instantiation of the fused kernel
             // one launch per level, as wide as its widest convolution body
-            FusedLaunch launch{widest, (int)items.size(), 0, 0, 0};
+            if (here.size() > (size_t)kMaxFusedItems) throw std::runtime_error("fused launch: too many groups in a stage");
+            FusedLaunch launch{widest, (int)items.size(), 0, 0, 0, {}};
             for (Pending *pend : here) {
                 WorkItem item = pend->item;
                 item.threads = pend->threads == 0 ? widest : pend->threads;
                 if (pend->threads == 0) item.num_blocks = std::max(1, (item.num_blocks * 256 + widest - 1) / widest);
                 item.first_block = launch.total_blocks;
+                if (launch.num_items < kFusedHeaderItems) launch.header.first_block[launch.num_items] = item.first_block;
                 launch.total_blocks += item.num_blocks;
                 launch.smem_bytes = std::max(launch.smem_bytes, pend->smem_bytes);
                 launch.num_items++;
                 items.push_back(item);
             }
+            launch.header.num_items = launch.num_items;
             fused_stages_[s].push_back(launch);
         }
     }
@@ -691,7 +694,7 @@ void Session::enqueue_fused(bool stage_events) {
                 for (int op : group) launch_op(plan_.ops[op], main);
         } else {
             for (const FusedLaunch &l : fused_stages_[s])
-                launch_fused(l.threads, items + l.first_item, l.num_items, l.total_blocks, l.smem_bytes, main);
+                launch_fused(l.threads, items + l.first_item, l.header, l.total_blocks, l.smem_bytes, main);
         }
         if (stage_events) IOS_HIP(hipEventRecord(stage_events_[s], main));
     }
