@@ -74,6 +74,7 @@ struct ConvKernelArgs {
     int Npix;
     int act, pre_relu;
     int split_k, k_chunk;
+    int steps_total, steps_chunk, steps_per_wave;   // wave-split kernels: MFMA k-steps in K, in a grid slice, in a wavefront's share of a full slice
     int tiles_m, tiles_n;
     int weights_major;   // 1: consecutive tiles share filter rows (filters larger than the input), 0: share pixels
     FastDiv div_tile;    // by tiles_n (weights_major) or tiles_m
@@ -516,7 +517,7 @@ struct ConvWsplit {
     static constexpr bool KQUAD = QUAD;                    // packed filters are [k / 4][m][4] instead of [k][m]
     // accumulators + staged operands per lane decide whether the body fits the register budget of a fused launch
     // (the channel-padding-4 forms serve first layers, which are stages of their own: kept out of the fused launches)
-    static constexpr bool FUSABLE = CP == 0 && E + D * U * (TM + TN) <= 56;
+    static constexpr bool FUSABLE = CP == 0 && E + D * U * (TM + TN) <= (QUAD ? 56 : 48);   // per-step addressing of the plain layout needs more registers
     static constexpr bool KBF16 = BF16;                    // packed filters hold bfloat16
     static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
     static_assert(!BF16 || (QUAD && MT == 16 && U == 4), "the bfloat16 path is the 16 x 16 x 16 form of the quad layout");
@@ -533,13 +534,12 @@ struct ConvWsplit {
     const int m0 = tm * BM;
     const int n0 = tn * BN;
 
-    // K slice z of the grid (k_chunk is a multiple of the batch U * KSTEP), divided among the wavefronts
-    const int s_lo = z * (a.k_chunk / M::KSTEP);
-    const int s_hi = min(a.Kq / M::KSTEP, s_lo + a.k_chunk / M::KSTEP);   // Kq is a multiple of 8 (of U * KSTEP with QUAD)
-    const int steps_slice = s_hi - s_lo;
-    const int steps_per_wave = QUAD ? ((steps_slice + U - 1) / U + NW - 1) / NW * U : (steps_slice + NW - 1) / NW;
-    const int s_begin = s_lo + wave * steps_per_wave;
-    const int s_end = min(s_hi, s_begin + steps_per_wave);
+    // K slice z of the grid (k_chunk is a multiple of the batch U * KSTEP), divided among the wavefronts; the host did the
+    // divisions (every wavefront of a block repeats this prologue on the SIMD's one scalar issue slot, so it is kept short)
+    const int s_lo = z * a.steps_chunk;
+    const int s_hi = min(a.steps_total, s_lo + a.steps_chunk);
+    const int s_begin = s_lo + wave * a.steps_per_wave;
+    const int s_end = min(s_hi, s_begin + a.steps_per_wave);
 
     int ih0[TN], iw0[TN];
     unsigned x_lane[TN];   // byte offset of (image, group channel lk, ih0, iw0); wraps like x_thread above
@@ -549,14 +549,17 @@ struct ConvWsplit {
         const int n = n0 + j * MT + lc;
         n_ok[j] = n < a.Npix;
         const int nn = n_ok[j] ? n : 0;
+        // image sizes are below 2^15 per side and OH * OW below 2^24 (checked on the host): 24-bit multiplies, which
+        // run at full rate, are exact here; byte offsets are wanted modulo 2^32, so 32-bit arithmetic gives them
         const int b = (int)fast_div((unsigned)nn, a.div_ohw);
-        const int r = nn - b * a.OHW;
+        const int r = nn - __mul24(b, a.OHW);
         const int oh = (int)fast_div((unsigned)r, a.div_ow);
-        const int ow = r - oh * a.OW;
-        ih0[j] = oh * a.sh - a.ph;
-        iw0[j] = ow * a.sw - a.pw;
+        const int ow = r - __mul24(oh, a.OW);
+        ih0[j] = __mul24(oh, a.sh) - a.ph;
+        iw0[j] = __mul24(ow, a.sw) - a.pw;
         const int lane_channel = QUAD ? U * lk : lk;   // first channel of this lane inside a step / batch
-        x_lane[j] = (unsigned)(((long long)b * a.x_bs + ((long long)g * a.ICg + lane_channel) * a.HW + (long long)ih0[j] * a.W + iw0[j]) * 4);
+        x_lane[j] = ((unsigned)b * (unsigned)a.x_bs + (unsigned)(g * a.ICg + lane_channel) * (unsigned)a.HW +
+                     (unsigned)(__mul24(ih0[j], a.W) + iw0[j])) * 4u;
     }
     const __amdgpu_buffer_rsrc_t xr = buffer_of(a.x, a.x_bytes);
     const __amdgpu_buffer_rsrc_t wr = buffer_of(a.wp, a.w_bytes);
@@ -564,10 +567,11 @@ struct ConvWsplit {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         w_kill[i] = m0 + i * MT + lc < a.OCgP ? 0u : kOutOfRange;
+        // byte offsets below 2^31 (checked on the host)
         if (QUAD)   // [g][k / 4][m][4]: this lane's first quad of a batch is row (U / 4) * lk
-            w_lane[i] = (unsigned)((((size_t)g * (a.Kq / 4) + (size_t)(U / 4) * lk) * a.OCgP + m0 + i * MT + lc) * (BF16 ? 8 : 16));
+            w_lane[i] = (((unsigned)g * ((unsigned)a.Kq >> 2) + (unsigned)((U / 4) * lk)) * (unsigned)a.OCgP + (unsigned)(m0 + i * MT + lc)) * (BF16 ? 8u : 16u);
         else
-            w_lane[i] = (unsigned)(((size_t)g * a.Kq * a.OCgP + (size_t)lk * a.OCgP + m0 + i * MT + lc) * 4);
+            w_lane[i] = (((unsigned)g * (unsigned)a.Kq + (unsigned)lk) * (unsigned)a.OCgP + (unsigned)(m0 + i * MT + lc)) * 4u;
     }
 #pragma unroll
     for (int j = 0; j < TN; j++) n_kill[j] = n_ok[j] ? 0u : kOutOfRange;

@@ -153,7 +153,9 @@ bool conv_matrix_path_supported(const ConvProblem &p) {
     // packed filter rows are indexed with 16 bits, input and filter byte offsets with 31 bits
     const unsigned long long x_bytes = (unsigned long long)p.B * p.IC * p.H * p.W * 4ull;
     const unsigned long long w_bytes = (unsigned long long)p.groups * p.Kq(128) * p.OCgP() * 4ull;
-    return p.Kq(128) < 65536 && p.Npix() < (1LL << 31) && x_bytes < (1ull << 30) && w_bytes < (1ull << 31);
+    // image sides below 2^15 and output planes below 2^24 elements keep the kernels' 24-bit index multiplies exact
+    return p.Kq(128) < 65536 && p.Npix() < (1LL << 31) && x_bytes < (1ull << 30) && w_bytes < (1ull << 31) && p.H < 32768 && p.W < 32768 &&
+           (long long)p.OH * p.OW < (1LL << 24);
 }
 
 ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
@@ -189,6 +191,14 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     a.act = p.act; a.pre_relu = p.pre_relu;
     a.k_chunk = k_chunk_of(p, l);
     a.split_k = effective_split(p, l);
+    {
+        // the wave-split kernels' division of a grid slice among the wavefronts of a block (BK = U k-steps, WK wavefronts)
+        const int kstep = e.v.MT == 32 ? 2 : 4;
+        const int u = std::max(1, e.v.BK / kstep);
+        a.steps_total = a.Kq / kstep;
+        a.steps_chunk = a.k_chunk / kstep;
+        a.steps_per_wave = e.v.kquad ? ceil_div(ceil_div(a.steps_chunk, u), e.v.WK) * u : ceil_div(a.steps_chunk, e.v.WK);
+    }
     a.tiles_m = ceil_div(p.OCg(), e.v.BM);
     a.tiles_n = ceil_div(p.Npix(), e.v.BN);
     a.weights_major = (double)p.OC * p.K() > (double)p.B * p.IC * p.H * p.W ? 1 : 0;
