@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per convolution launch of a batch-1 Inception-v3 pass, from FETCH_SIZE / WRITE_SIZE counter runs scaled by a
 # copy kernel of known size (profiles/conv_kernel_hbm_traffic_inception_v3.md); counters cannot be read from inside this
 # script, so the figure is the offline measurement of the same kernels.
-MEASURED_CONV_TRAFFIC_BYTES_PER_LAUNCH = {1: 4.50e6, 64: 81.1e6}
+MEASURED_CONV_TRAFFIC_BYTES_PER_LAUNCH = {1: 4.49e6, 64: 76.5e6}
 
 
 def op_bound_ms(op):
