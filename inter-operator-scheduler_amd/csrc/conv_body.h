@@ -77,7 +77,9 @@ struct ConvKernelArgs {
     int steps_total, steps_chunk, steps_per_wave;   // wave-split kernels: MFMA k-steps in K, in a grid slice, in a wavefront's share of a full slice
     int tiles_m, tiles_n;
     int weights_major;   // 1: consecutive tiles share filter rows (filters larger than the input), 0: share pixels
-    FastDiv div_tile;    // by tiles_n (weights_major) or tiles_m
+    int xcd_q, xcd_r;    // tiles_m * tiles_n = 8 * xcd_q + xcd_r
+    int tile_div;        // tiles_n (weights_major) or tiles_m
+    FastDiv div_tile;    // by tile_div
     FastDiv div_ohw, div_ow;
 };
 
@@ -85,18 +87,13 @@ struct ConvKernelArgs {
 // receives a contiguous range of them, and the range runs along the operand that is cheaper to duplicate: the
 // more expensive operand (filters at batch 1, activations at large batch) is then fetched into one L2 only.
 __device__ __forceinline__ void xcd_tile(const ConvKernelArgs &a, int block, int &tm, int &tn) {
-    const int total = a.tiles_m * a.tiles_n;
+    // XCD x owns tiles [x * q + min(x, r), ...): q + 1 tiles for the first r XCDs, q for the others
     const int xcd = block & 7, slot = block >> 3;
-    const int q = total >> 3, r = total & 7;
-    const int t = xcd < r ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
+    const int t = slot + xcd * a.xcd_q + min(xcd, a.xcd_r);
     const int q2 = (int)fast_div((unsigned)t, a.div_tile);
-    if (a.weights_major) {
-        tm = q2;
-        tn = t - tm * a.tiles_n;
-    } else {
-        tn = q2;
-        tm = t - tn * a.tiles_m;
-    }
+    const int rest = t - q2 * a.tile_div;
+    tm = a.weights_major ? q2 : rest;
+    tn = a.weights_major ? rest : q2;
 }
 
 __device__ __forceinline__ float apply_act(float v, int act) {

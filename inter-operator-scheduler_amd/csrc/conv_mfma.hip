@@ -202,7 +202,10 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     a.tiles_m = ceil_div(p.OCg(), e.v.BM);
     a.tiles_n = ceil_div(p.Npix(), e.v.BN);
     a.weights_major = (double)p.OC * p.K() > (double)p.B * p.IC * p.H * p.W ? 1 : 0;
-    a.div_tile = make_fast_div((unsigned)(a.weights_major ? a.tiles_n : a.tiles_m));
+    a.tile_div = a.weights_major ? a.tiles_n : a.tiles_m;
+    a.xcd_q = (a.tiles_m * a.tiles_n) >> 3;
+    a.xcd_r = (a.tiles_m * a.tiles_n) & 7;
+    a.div_tile = make_fast_div((unsigned)a.tile_div);
     a.div_ohw = make_fast_div((unsigned)a.OHW);
     a.div_ow = make_fast_div((unsigned)a.OW);
     if (a.split_k > 1 && workspace == nullptr) throw std::runtime_error("conv: split-K launch without workspace");
