@@ -546,7 +546,7 @@ struct ConvWsplit {
         const int n = n0 + j * MT + lc;
         n_ok[j] = n < a.Npix;
         const int nn = n_ok[j] ? n : 0;
-        // image sizes are below 2^15 per side and OH * OW below 2^24 (checked on the host): 24-bit multiplies, which
+        // image sizes are below 2^15 per side and OH * OW below 2^23 (checked on the host): signed 24-bit multiplies, which
         // run at full rate, are exact here; byte offsets are wanted modulo 2^32, so 32-bit arithmetic gives them
         const int b = (int)fast_div((unsigned)nn, a.div_ohw);
         const int r = nn - __mul24(b, a.OHW);

@@ -153,9 +153,9 @@ bool conv_matrix_path_supported(const ConvProblem &p) {
     // packed filter rows are indexed with 16 bits, input and filter byte offsets with 31 bits
     const unsigned long long x_bytes = (unsigned long long)p.B * p.IC * p.H * p.W * 4ull;
     const unsigned long long w_bytes = (unsigned long long)p.groups * p.Kq(128) * p.OCgP() * 4ull;
-    // image sides below 2^15 and output planes below 2^24 elements keep the kernels' 24-bit index multiplies exact
+    // image sides below 2^15 and output planes below 2^23 elements keep the kernels' signed 24-bit index multiplies exact
     return p.Kq(128) < 65536 && p.Npix() < (1LL << 31) && x_bytes < (1ull << 30) && w_bytes < (1ull << 31) && p.H < 32768 && p.W < 32768 &&
-           (long long)p.OH * p.OW < (1LL << 24);
+           (long long)p.OH * p.OW < (1LL << 23) && p.B < (1 << 23);
 }
 
 ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
