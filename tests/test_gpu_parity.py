@@ -371,6 +371,35 @@ def test_large_batch_parallel_stages_with_measured_kernel_configurations():
         rt.set_option('autotune', 0)
 
 
+def test_batch_64_images_are_independent_and_match_the_oracle():
+    """
+    The largest configuration of the batch sweep with the measured kernel configurations the benchmark runs: an
+    image's output depends on that image alone, so a sample of the 64 outputs is checked against the oracle run
+    on those images only, and two identical images inside the batch must give identical outputs.
+    """
+    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    graph.sequential_schedule()
+    batch = 64
+    x = np.random.default_rng(9).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
+    x[41] = x[5]
+    sample = [0, 5, 17, 63]
+    want = ios_oracle.run(graph, x[sample])
+    rt.set_option('autotune', 1)
+    rt.set_option('executor', 'fused_graph')
+    try:
+        with rt.Session(graph, batch) as session:
+            session.load_weights()
+            session.set_input(x)
+            session.run()
+            got = session.output()
+    finally:
+        rt.set_option('autotune', 0)
+        rt.set_option('executor', 'streams')
+    assert got.shape[0] == batch and np.isfinite(got).all()
+    assert_close(got[sample], want, 'inception batch 64, sampled images')
+    np.testing.assert_array_equal(got[41], got[5])
+
+
 def matrix_path_convs(graph, batch):
     return frozenset(op['node'] for op in rt.plan_describe(graph, batch) if op['kind'] == 'conv_mfma')
 
