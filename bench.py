@@ -239,6 +239,20 @@ def main():
         'device': {k: device[k] for k in ('name', 'arch', 'compute_units')},
     }
 
+    # the reference's best schedule family (parallel groups + merged convolutions, "IOS-Both"); the headline metric
+    # is the dp_parallel schedule, this one is reported beside it
+    rt.set_option('executor', args.search_executor)
+    t0 = time.time()
+    merged = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel_merge', compute_weight=True,
+                          warmup=2, number=args.search_number, repeat=args.search_repeat)
+    merge_search_s = time.time() - t0
+    graph.sequential_schedule()
+    rt.set_option('executor', args.executor)
+    both, both_out = timed_latency(rt, np, merged, batch, x, args.steps, args.warmup)
+    result['dp_parallel_merge'] = {'latency_ms': both, 'images_per_s': batch / (both['wall'] * 1e-3), 'search_seconds': merge_search_s,
+                                   'num_stages': sum(len(b.stages) for b in merged.blocks),
+                                   'max_abs_diff_to_sequential': float(np.abs(seq_out - both_out).max())}
+
     if not args.no_sweep:
         sweep = {}
         for b in (16, 64):
