@@ -118,6 +118,8 @@ private:
         n.C = shape[0].as_int();
         n.H = shape[1].as_int();
         n.W = shape[2].as_int();
+        if (n.C < 1 || n.H < 1 || n.W < 1 || n.C > kMaxChannels || n.H > kMaxExtent || n.W > kMaxExtent)
+            throw std::runtime_error("placeholder '" + name + "': bad shape");
         n.own = true;
         by_name_[name] = static_cast<int>(nodes_.size());
         nodes_.push_back(n);
@@ -220,7 +222,9 @@ private:
             n.C = cfg["out_channels"].as_int();
             if (groups < 1 || C % groups != 0 || n.C % groups != 0)
                 throw std::runtime_error("conv '" + name + "': channels not divisible by groups");
-            if (sh < 1 || sw < 1 || kh < 1 || kw < 1) throw std::runtime_error("conv '" + name + "': bad geometry");
+            if (sh < 1 || sw < 1 || kh < 1 || kw < 1 || ph < 0 || pw < 0 || std::max({kh, kw, sh, sw, ph, pw}) > kMaxExtent)
+                throw std::runtime_error("conv '" + name + "': bad geometry");
+            if (n.C < 1 || n.C > kMaxChannels) throw std::runtime_error("conv '" + name + "': bad channel count");
             n.H = 1 + (H - kh + 2 * ph) / sh;
             n.W = 1 + (W - kw + 2 * pw) / sw;
             act_code(cfg["act"].as_string());
@@ -228,6 +232,8 @@ private:
             n.type = NodeType::Pool;
             n.C = C;
             const std::string pool_type = cfg["pool_type"].as_string();
+            if (pool_type != "max" && pool_type != "avg" && pool_type != "global_max" && pool_type != "global_avg")
+                throw std::runtime_error("pool '" + name + "': unknown pool_type '" + pool_type + "'");
             if (pool_type.find("global") != std::string::npos) {
                 n.H = 1;
                 n.W = 1;
@@ -235,7 +241,8 @@ private:
                 const int kh = cfg["kernel"][0].as_int(), kw = cfg["kernel"][1].as_int();
                 const int sh = cfg["stride"][0].as_int(), sw = cfg["stride"][1].as_int();
                 const int ph = cfg["padding"][0].as_int(), pw = cfg["padding"][1].as_int();
-                if (sh < 1 || sw < 1 || kh < 1 || kw < 1) throw std::runtime_error("pool '" + name + "': bad geometry");
+                if (sh < 1 || sw < 1 || kh < 1 || kw < 1 || ph < 0 || pw < 0 || std::max({kh, kw, sh, sw, ph, pw}) > kMaxExtent)
+                    throw std::runtime_error("pool '" + name + "': bad geometry");
                 n.H = 1 + (H - kh + 2 * ph) / sh;
                 n.W = 1 + (W - kw + 2 * pw) / sw;
             }

@@ -22,6 +22,8 @@
 namespace ios {
 
 constexpr int kMaxGroups = 16;   // concurrent groups (streams) per stage
+constexpr int kMaxExtent = 1 << 16;     // image sides, filter sides, strides and padding a document may ask for
+constexpr int kMaxChannels = 1 << 20;   // channels of a tensor
 
 struct ViewRef {
     size_t offset = 0;   // in floats from the arena base

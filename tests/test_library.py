@@ -79,6 +79,39 @@ def test_host_planner_rejects_bad_documents():
         rt.plan_describe(graph, 0)
 
 
+def test_host_planner_rejects_bad_operator_fields():
+    """Geometry, channel counts and type names are checked before anything is sized or launched."""
+    import copy
+    import json
+    graph = ios.models.squeezenet_1_1()
+    graph.sequential_schedule()
+    base = graph.export_config()
+
+    def first_node_with(doc, field):
+        for block in doc['blocks']:
+            for node in block['inner_nodes'] + [block['exit_node']]:
+                if field in node:
+                    return node
+        raise AssertionError(field)
+
+    cases = [('stride', [0, 1], 'bad geometry'), ('kernel', [3, -3], 'bad geometry'), ('padding', [-1, 0], 'bad geometry'),
+             ('padding', [1 << 20, 0], 'bad geometry'), ('groups', 0, 'not divisible by groups'), ('groups', 7, 'not divisible by groups'),
+             ('out_channels', 0, 'channel'), ('out_channels', 10 ** 9, 'bad channel count'), ('pool_type', 'median', 'unknown pool_type'),
+             ('act', 'gelu', 'unsupported activation')]
+    for field, value, message in cases:
+        doc = copy.deepcopy(base)
+        first_node_with(doc, field)[field] = value
+        assert rt.get_lib().ios_plan_describe(rt.c_string(json.dumps(doc)), 1, None, 0) == -1, (field, value)
+        assert message.encode() in rt.get_lib().ios_last_error(), (field, value, rt.get_lib().ios_last_error())
+    for shape in ([0, 224, 224], [3, -1, 224], [3, 224, 1 << 20]):
+        doc = copy.deepcopy(base)
+        doc['input']['output_shape'] = shape
+        assert rt.get_lib().ios_plan_describe(rt.c_string(json.dumps(doc)), 1, None, 0) == -1, shape
+        assert b'bad shape' in rt.get_lib().ios_last_error()
+    for text in ('', '{', '{"name": 1}', 'null', '[]'):
+        assert rt.get_lib().ios_plan_describe(rt.c_string(text), 1, None, 0) == -1, text
+
+
 def test_convolutions_of_parallel_stages_get_kernels_that_can_share_a_launch():
     """Host planner, closed-form kernel choice: every matrix-path convolution of a multi-group stage must be able
     to run inside a fused stage launch, at batch 1 and at a batch large enough for the LDS-tiled kernels."""
