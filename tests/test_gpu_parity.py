@@ -93,6 +93,26 @@ def test_conv_matches_oracle(case):
     assert_close(got, want, f'conv {case}')
 
 
+def test_committed_operator_vectors():
+    """The fixed inputs, weights and brute-force outputs of tests/golden/operator_vectors.npz through the C ABI."""
+    import os
+    import sys
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden')
+    sys.path.insert(0, golden)
+    import make_operator_vectors as spec
+    data = np.load(os.path.join(golden, 'operator_vectors.npz'))
+    for name, shape, oc, kernel, stride, padding, groups, act in spec.CONVS:
+        graph = single_op_graph(shape[1:], lambda b, v: ios.conv2d(b, [[v]], oc, kernel, stride, padding, groups, act, is_exit=True))
+        conv = list(graph.conv_nodes())[0]
+        conv.weight, conv.bias = data[f'{name}.w'], data[f'{name}.b']
+        got = rt.graph_inference(graph, shape[0], data[f'{name}.x'])
+        assert_close(got, data[f'{name}.y'], name)
+    for name, shape, pool_type, kernel, stride, padding in spec.POOLS:
+        graph = single_op_graph(shape[1:], lambda b, v: ios.pool2d(b, [[v]], pool_type, kernel, stride, padding, is_exit=True))
+        got = rt.graph_inference(graph, shape[0], data[f'{name}.x'])
+        assert_close(got, data[f'{name}.y'], name)
+
+
 @pytest.mark.parametrize('variant', range(80))
 @pytest.mark.parametrize('split_k', [1, 3])
 def test_every_conv_kernel_variant(variant, split_k):

@@ -206,3 +206,27 @@ def test_bf16_rounding_is_round_to_nearest_even():
     want = (((bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000) & 0xFFFFFFFF).astype(np.uint32).view(np.float32)
     got = ios_oracle.to_bf16(torch.from_numpy(x)).numpy()
     np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def _golden_vectors():
+    import os
+    import sys
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden')
+    sys.path.insert(0, golden)
+    import make_operator_vectors as spec
+    return spec, np.load(os.path.join(golden, 'operator_vectors.npz'))
+
+
+def test_committed_operator_vectors_pin_the_oracle_and_the_c_restatement():
+    """tests/golden/operator_vectors.npz holds inputs and brute-force outputs; both oracles must reproduce them."""
+    spec, data = _golden_vectors()
+    for name, shape, oc, kernel, stride, padding, groups, act in spec.CONVS:
+        x, w, b, want = (data[f'{name}.{k}'] for k in 'xwby')
+        assert x.shape == tuple(shape) and want.dtype == np.float32
+        np.testing.assert_allclose(_oracle_conv(x, w, b, stride, padding, groups, act), want, rtol=RTOL, atol=ATOL, err_msg=name)
+        np.testing.assert_allclose(c_oracle.conv2d(x, w, b, stride, padding, groups, act), want, rtol=RTOL, atol=ATOL, err_msg=name)
+    for name, shape, pool_type, kernel, stride, padding in spec.POOLS:
+        x, want = data[f'{name}.x'], data[f'{name}.y']
+        got = ios_oracle.pool2d(torch.from_numpy(x), pool_type, kernel, stride, padding).numpy()
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL, err_msg=name)
+        np.testing.assert_allclose(c_oracle.pool2d(x, pool_type, kernel, stride, padding), want, rtol=RTOL, atol=ATOL, err_msg=name)
