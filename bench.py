@@ -161,6 +161,8 @@ def main():
                              "closed-form model (no device probes; keeps profiler traces small)")
     parser.add_argument('--search-number', type=int, default=6, help='passes per stage probe of the schedule search')
     parser.add_argument('--search-repeat', type=int, default=3, help='probes per candidate stage of the schedule search')
+    parser.add_argument('--search-restarts', type=int, default=2,
+                        help='schedule searches to run (stage measurements are noisy: the schedule that measures faster as a whole is kept)')
     parser.add_argument('--no-sweep', action='store_true', help='skip the batch 16 / 64 sweep')
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     parser.add_argument('--no-configs', action='store_true', help='skip the other four configuration networks')
@@ -194,8 +196,15 @@ def main():
     rt.set_option('executor', args.search_executor)
     t0 = time.time()
     cost_model = ios.IOSCostModel() if args.search == 'measured' else ios.AnalyticCostModel()
-    optimized = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
-                             warmup=2, number=args.search_number, repeat=args.search_repeat)
+    optimized, optimized_ms = None, None
+    for _ in range(max(1, args.search_restarts if args.search == 'measured' else 1)):
+        candidate = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
+                                 warmup=2, number=args.search_number, repeat=args.search_repeat)
+        rt.set_option('executor', args.executor)
+        candidate_ms = float(np.mean(rt.graph_latency(candidate, batch, warmup=2, number=6, repeat=6)))
+        rt.set_option('executor', args.search_executor)
+        if optimized is None or candidate_ms < optimized_ms:
+            optimized, optimized_ms = candidate, candidate_ms
     search_s = time.time() - t0
     graph.sequential_schedule()
 
