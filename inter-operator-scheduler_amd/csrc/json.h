@@ -60,6 +60,8 @@ public:
 
     int as_int() const {
         if (kind_ != Number) throw std::runtime_error("json: expected a number");
+        // NaN fails both comparisons; a value outside int cannot be converted without undefined behaviour
+        if (!(number_ >= -2147483648.0 && number_ <= 2147483647.0)) throw std::runtime_error("json: number out of integer range");
         return static_cast<int>(number_);
     }
     double as_double() const {

@@ -108,6 +108,10 @@ def test_host_planner_rejects_bad_operator_fields():
         doc['input']['output_shape'] = shape
         assert rt.get_lib().ios_plan_describe(rt.c_string(json.dumps(doc)), 1, None, 0) == -1, shape
         assert b'bad shape' in rt.get_lib().ios_last_error()
+    doc = copy.deepcopy(base)
+    doc['input']['output_shape'] = [3, 1e30, 224]      # a number no int can hold
+    assert rt.get_lib().ios_plan_describe(rt.c_string(json.dumps(doc)), 1, None, 0) == -1
+    assert b'out of integer range' in rt.get_lib().ios_last_error()
     for text in ('', '{', '{"name": 1}', 'null', '[]'):
         assert rt.get_lib().ios_plan_describe(rt.c_string(text), 1, None, 0) == -1, text
 
