@@ -540,6 +540,34 @@ def test_optimize_with_measured_cost_model_on_sample_net():
     assert_close(got, ios_oracle.run(graph, x.astype(np.float32)), 'optimized sample net')
 
 
+def test_calls_from_two_host_threads_are_serialised():
+    """The library keeps process-wide state; its entry points take a lock, so concurrent callers get correct results."""
+    import threading
+    graph = ios.models.squeezenet_1_1(init_seed=0, init_scheme='he_normal')
+    graph.greedy_schedule(8)
+    x = np.random.default_rng(3).standard_normal((1, *graph.enter_node.output_shape)).astype(np.float32)
+    want = ios_oracle.run(graph, x)
+    results, errors = {}, []
+
+    def worker(index):
+        try:
+            for _ in range(3):
+                results[index] = rt.graph_inference(graph, 1, x)
+                latency = rt.graph_latency(graph, 1, warmup=1, number=2, repeat=2)
+                assert len(latency) == 2 and all(v > 0 for v in latency)
+        except Exception as error:   # noqa: BLE001 - reported by the main thread
+            errors.append(error)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for index in range(2):
+        assert_close(results[index], want, f'thread {index}')
+
+
 def test_errors_are_reported_not_fatal():
     graph = ios.models.sample_network(init_seed=0)
     with pytest.raises(RuntimeError, match='no schedule'):
