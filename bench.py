@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per convolution launch of a batch-1 Inception-v3 pass, from FETCH_SIZE / WRITE_SIZE counter runs scaled by a
 # copy kernel of known size (profiles/conv_kernel_hbm_traffic_inception_v3.md); counters cannot be read from inside this
 # script, so the figure is the offline measurement of the same kernels.
-MEASURED_CONV_TRAFFIC_BYTES_PER_LAUNCH = {1: 4.49e6, 64: 76.5e6}
+MEASURED_CONV_TRAFFIC_BYTES_PER_LAUNCH = {1: 4.43e6, 64: 82.9e6}
 
 
 def op_bound_ms(op):
@@ -161,13 +161,19 @@ def main():
                              "closed-form model (no device probes; keeps profiler traces small)")
     parser.add_argument('--search-number', type=int, default=6, help='passes per stage probe of the schedule search')
     parser.add_argument('--search-repeat', type=int, default=3, help='probes per candidate stage of the schedule search')
+    parser.add_argument('--max-group-size', type=int, default=1,
+                        help='pruning knob r of the schedule search (operators per group).  The fused executor runs the groups of a '
+                             'stage level by level, so groups of one operator (r = 1) let the search place every level freely; the '
+                             'reference default r = 3 is measured beside it')
+    parser.add_argument('--max-num-groups', type=int, default=8, help='pruning knob s of the schedule search (groups per stage)')
     parser.add_argument('--search-restarts', type=int, default=2,
                         help='schedule searches to run (stage measurements are noisy: the schedule that measures faster as a whole is kept)')
     parser.add_argument('--no-sweep', action='store_true', help='skip the batch 16 / 64 sweep')
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     parser.add_argument('--no-configs', action='store_true', help='skip the other four configuration networks')
-    parser.add_argument('--search-all', action='store_true',
-                        help='run the measured schedule search on RandWire and NASNet too (minutes each) instead of the greedy schedule')
+    parser.add_argument('--greedy-big', action='store_true',
+                        help='use the greedy schedule for RandWire and NASNet instead of the measured search (half a minute each at r = 1, '
+                             'minutes at r = 3)')
     parser.add_argument('--option', action='append', default=[], metavar='KEY=VALUE', help='extra runtime option (repeatable)')
     parser.add_argument('--probe', choices=['copy', 'pass'], help='run a profiler probe instead of the benchmark')
     args = parser.parse_args()
@@ -199,7 +205,8 @@ def main():
     optimized, optimized_ms = None, None
     for _ in range(max(1, args.search_restarts if args.search == 'measured' else 1)):
         candidate = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
-                                 warmup=2, number=args.search_number, repeat=args.search_repeat)
+                                 warmup=2, number=args.search_number, repeat=args.search_repeat,
+                                 max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
         rt.set_option('executor', args.executor)
         candidate_ms = float(np.mean(rt.graph_latency(candidate, batch, warmup=2, number=6, repeat=6)))
         rt.set_option('executor', args.search_executor)
@@ -232,7 +239,7 @@ def main():
         'vs_baseline': None,
         'dtype': 'f32',
         'data': 'synthetic (N(0,1) input, seeded He-normal weights, zero bias)',
-        'config': {'workload': f'inception_v3 3x299x299 batch {batch}, dp_parallel schedule (r=3, s=8), {args.executor} executor',
+        'config': {'workload': f'inception_v3 3x299x299 batch {batch}, dp_parallel schedule (r={args.max_group_size}, s={args.max_num_groups}), {args.executor} executor',
                    'global_batch': batch},
         'latency_ms': {'dp_parallel': opt, 'sequential': seq},
         'speedup_vs_own_sequential': seq['wall'] / opt['wall'],
@@ -247,6 +254,19 @@ def main():
         'stage_overlap': stage_overlap(ops, op_ms, stage_ms),
         'device': {k: device[k] for k in ('name', 'arch', 'compute_units')},
     }
+
+    # the same search with the reference's default pruning (r = 3, s = 8), for comparison with the headline's r and s
+    if (args.max_group_size, args.max_num_groups) != (3, 8):
+        rt.set_option('executor', args.search_executor)
+        t0 = time.time()
+        default_knobs = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
+                                     warmup=2, number=args.search_number, repeat=args.search_repeat)
+        default_search_s = time.time() - t0
+        graph.sequential_schedule()
+        rt.set_option('executor', args.executor)
+        r3, _ = timed_latency(rt, np, default_knobs, batch, x, args.steps, args.warmup)
+        result['dp_parallel_r3_s8'] = {'latency_ms': r3, 'images_per_s': batch / (r3['wall'] * 1e-3), 'search_seconds': default_search_s,
+                                       'num_stages': sum(len(b.stages) for b in default_knobs.blocks)}
 
     # the reference's best schedule family (parallel groups + merged convolutions, "IOS-Both"); the headline metric
     # is the dp_parallel schedule, this one is reported beside it
@@ -273,7 +293,8 @@ def main():
             rt.set_option('executor', args.search_executor)
             t0 = time.time()
             optimized_b = ios.optimize(graph, batch_size=b, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
-                                       warmup=2, number=args.search_number, repeat=args.search_repeat)
+                                       warmup=2, number=args.search_number, repeat=args.search_repeat,
+                                       max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
             search_b = time.time() - t0
             graph.sequential_schedule()
             rt.set_option('executor', args.executor)
@@ -310,20 +331,24 @@ def main():
                                    ('nasnet_mobile', ios.models.nasnet_mobile, False)):
             g = make(init_seed=0, init_scheme='he_normal')
             xc = np.random.default_rng(1).standard_normal((1, *g.enter_node.output_shape)).astype(np.float32)
-            if search or args.search_all:
+            if search or not args.greedy_big:
                 rt.set_option('executor', args.search_executor)
-                scheduled = ios.optimize(g, batch_size=1, opt_type='dp_parallel', compute_weight=True, warmup=2, number=6, repeat=3)
+                t0 = time.time()
+                scheduled = ios.optimize(g, batch_size=1, opt_type='dp_parallel', compute_weight=True, warmup=2, number=6, repeat=3,
+                                         max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
+                search_c = time.time() - t0
                 label = 'dp_parallel'
                 rt.set_option('executor', args.executor)
-            else:   # the measured search takes minutes on these graphs (--search-all): use the greedy schedule
+            else:   # --greedy-big
                 scheduled = make(init_seed=0, init_scheme='he_normal')
                 scheduled.greedy_schedule(4)
                 label = 'greedy'
+                search_c = 0.0
             g.sequential_schedule()
             c_seq, _ = timed_latency(rt, np, g, 1, xc, 100, 10)
             c_par, _ = timed_latency(rt, np, scheduled, 1, xc, 100, 10)
             ops_c = rt.plan_describe(g, 1)
-            configs[name] = {'sequential_ms': c_seq['wall'], f'{label}_ms': c_par['wall'],
+            configs[name] = {'sequential_ms': c_seq['wall'], f'{label}_ms': c_par['wall'], 'search_seconds': search_c,
                              'network_roofline_ms': network_roofline_ms(ops_c, parallel=False)}
         result['other_configs_batch1'] = configs
         # the model variants the reference's own result table uses (its large RandWire / NASNet and SqueezeNet 1.0 with
