@@ -174,6 +174,8 @@ def main():
     parser.add_argument('--greedy-big', action='store_true',
                         help='use the greedy schedule for RandWire and NASNet instead of the measured search (half a minute each at r = 1, '
                              'minutes at r = 3)')
+    parser.add_argument('--search-variants', action='store_true',
+                        help="measured schedule search also for the reference table's large model variants (about two more minutes)")
     parser.add_argument('--option', action='append', default=[], metavar='KEY=VALUE', help='extra runtime option (repeatable)')
     parser.add_argument('--probe', choices=['copy', 'pass'], help='run a profiler probe instead of the benchmark')
     args = parser.parse_args()
@@ -364,6 +366,15 @@ def main():
             v_seq, _ = timed_latency(rt, np, g, 1, xc, 50, 5)
             v_par, _ = timed_latency(rt, np, scheduled, 1, xc, 50, 5)
             variants[name] = {'sequential_ms': v_seq['wall'], 'greedy_ms': v_par['wall']}
+            if args.search_variants:
+                rt.set_option('executor', args.search_executor)
+                t0 = time.time()
+                searched = ios.optimize(make(init_seed=0, init_scheme='he_normal'), batch_size=1, opt_type='dp_parallel', compute_weight=True,
+                                        warmup=2, number=6, repeat=3, max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
+                variants[name]['search_seconds'] = time.time() - t0
+                rt.set_option('executor', args.executor)
+                v_dp, _ = timed_latency(rt, np, searched, 1, xc, 50, 5)
+                variants[name]['dp_parallel_ms'] = v_dp['wall']
         result['reference_table_variants_batch1'] = variants
 
     if not args.no_cpu:
