@@ -69,6 +69,7 @@ private:
     bool share_cost_rule_ = true;   // share classes weigh time by the held share of the device (false: hard footprint budgets)
     int share_threads_per_cu_ = 1024;   // resident threads per compute unit the share-class budgets assume (four wavefronts per SIMD)
     void load_tune_cache();
+    std::string settings_token() const;
     float *tune_buf_[4] = {nullptr, nullptr, nullptr, nullptr};
     size_t tune_floats_[4] = {0, 0, 0, 0};
     std::string tune_cache_path_;

@@ -65,17 +65,26 @@ static std::string conv_signature(const ConvProblem &p) {
     return os.str();
 }
 
+// the measured winners of the share classes depend on these settings: they are part of every cache key
+std::string DeviceContext::settings_token() const {
+    std::ostringstream os;
+    os << (share_cost_rule_ ? "cost" : "budget") << '/' << share_threads_per_cu_ << '/' << (inline_reduce_ ? "inline" : "kernel");
+    return os.str();
+}
+
 void DeviceContext::load_tune_cache() {
     FILE *f = fopen(tune_cache_path_.c_str(), "r");
     if (f == nullptr) return;
-    // line: 12 problem integers, then kShareClasses pairs (configuration name, split_k).  A line that does not parse
-    // (truncated write, a configuration name this build no longer has) is skipped: its shape is measured again.
+    // line: 12 problem integers, the settings token, then kShareClasses pairs (configuration name, split_k).  A line that
+    // does not parse (truncated write, a configuration name this build no longer has) is skipped: its shape is measured again.
     char line[1024];
     while (fgets(line, sizeof(line), f) != nullptr) {
         std::istringstream in(line);
         int v[12];
         bool ok = true;
         for (int i = 0; i < 12 && ok; i++) ok = static_cast<bool>(in >> v[i]);
+        std::string token;
+        ok = ok && static_cast<bool>(in >> token) && token.find('/') != std::string::npos;
         TunedConv entry;
         for (int c = 0; c < kShareClasses && ok; c++) {
             std::string name;
@@ -91,6 +100,7 @@ void DeviceContext::load_tune_cache() {
         if (!ok) continue;
         std::ostringstream os;
         for (int i = 0; i < 12; i++) os << (i ? " " : "") << v[i];
+        os << ' ' << token;
         if (conv_variant(entry.best[0].variant).bf16) os << " bf16";   // reduced-precision entries have their own keys
         tuned[os.str()] = entry;
     }
@@ -254,7 +264,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     if (!tune_cache_path_.empty()) {
         FILE *f = fopen(tune_cache_path_.c_str(), "a");
         if (f != nullptr) {
-            fprintf(f, "%s", conv_signature(p).c_str());
+            fprintf(f, "%s %s", conv_signature(p).c_str(), settings_token().c_str());
             for (int c = 0; c < kShareClasses; c++) fprintf(f, " %s %d", conv_variant(result.best[c].variant).name, result.best[c].split_k);
             fprintf(f, "\n");
             fclose(f);
@@ -268,7 +278,7 @@ ConvLaunch DeviceContext::choose_launch(const ConvProblem &p, int share) {
     while (cls + 1 < kShareClasses && (1 << (cls + 1)) <= share) cls++;   // floor(log2(share)), capped
     ConvLaunch launch;
     if (autotune_) {
-        const std::string key = conv_signature(p) + (bf16_ ? " bf16" : "");
+        const std::string key = conv_signature(p) + " " + settings_token() + (bf16_ ? " bf16" : "");
         auto it = tuned.find(key);
         if (it == tuned.end()) it = tuned.emplace(key, tune_conv(p)).first;
         launch = it->second.best[cls];
