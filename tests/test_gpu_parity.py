@@ -540,6 +540,30 @@ def test_optimize_with_measured_cost_model_on_sample_net():
     assert_close(got, ios_oracle.run(graph, x.astype(np.float32)), 'optimized sample net')
 
 
+def test_measured_search_with_groups_of_one_operator_under_the_fused_executor():
+    """The pruning the benchmark uses (r = 1, s = 8): stages are sets of independent operators, one fused launch each."""
+    rt.set_option('executor', 'fused')
+    rt.set_option('autotune', 1)
+    try:
+        for make in (ios.models.squeezenet_1_1, ios.models.inception_v3):
+            graph = make(init_seed=0, init_scheme='he_normal')
+            optimized = ios.optimize(graph, batch_size=1, opt_type='dp_parallel', compute_weight=True, warmup=1, number=2, repeat=1,
+                                     max_group_size=1, max_num_groups=8)
+            stages = [stage for block in optimized.blocks for stage in block.stages]
+            assert all(len(group) == 1 for stage in stages for group in stage) and all(len(stage) <= 8 for stage in stages)
+            assert any(len(stage) > 1 for stage in stages)
+            assert sorted(n for stage in stages for group in stage for n in group) == sorted(n.name for n in graph.nodes() if n is not graph.enter_node)
+            x = np.random.default_rng(2).standard_normal((1, *graph.enter_node.output_shape)).astype(np.float32)
+            graph.sequential_schedule()
+            want = ios_oracle.run(graph, x)
+            for executor in ('fused', 'fused_graph'):
+                rt.set_option('executor', executor)
+                assert_close(rt.graph_inference(optimized, 1, x), want, f'{graph.name} r=1 {executor}')
+            rt.set_option('executor', 'fused')
+    finally:
+        rt.set_option('autotune', 0)
+
+
 def test_calls_from_two_host_threads_are_serialised():
     """The library keeps process-wide state; its entry points take a lock, so concurrent callers get correct results."""
     import threading
