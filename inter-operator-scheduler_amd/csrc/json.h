@@ -21,7 +21,7 @@ public:
 
     static Json parse(const char *text) {
         if (text == nullptr) throw std::runtime_error("json: null document");
-        Reader r{text, text};
+        Reader r{text, text, 0};
         Json v = r.value();
         r.skip_ws();
         if (*r.p != '\0') r.fail("trailing characters");
@@ -82,6 +82,17 @@ private:
     struct Reader {
         const char *begin;
         const char *p;
+        int depth;   // open arrays / objects around the value being read
+        // graph documents nest a handful of levels (graph > blocks > nodes > inputs > term > value); a bound keeps a
+        // hostile document from exhausting the stack, which no exception handler could report
+        static constexpr int kMaxDepth = 64;
+        struct Nest {
+            Reader &r;
+            explicit Nest(Reader &reader) : r(reader) {
+                if (++r.depth > kMaxDepth) r.fail("nesting deeper than 64 levels");
+            }
+            ~Nest() { --r.depth; }
+        };
 
         [[noreturn]] void fail(const std::string &what) const {
             throw std::runtime_error("json: " + what + " at byte " + std::to_string(p - begin));
@@ -103,6 +114,7 @@ private:
             Json v;
             switch (*p) {
                 case '{': {
+                    Nest nest(*this);
                     ++p;
                     v.kind_ = Object;
                     if (consume('}')) return v;
@@ -117,6 +129,7 @@ private:
                     return v;
                 }
                 case '[': {
+                    Nest nest(*this);
                     ++p;
                     v.kind_ = Array;
                     if (consume(']')) return v;
@@ -195,6 +208,7 @@ private:
                             }
                             break;
                         }
+                        case '\0': fail("unterminated string");   // a backslash was the last byte of the document
                         default: out += *p;  // \" \\ \/
                     }
                     ++p;

@@ -225,6 +225,8 @@ private:
             if (sh < 1 || sw < 1 || kh < 1 || kw < 1 || ph < 0 || pw < 0 || std::max({kh, kw, sh, sw, ph, pw}) > kMaxExtent)
                 throw std::runtime_error("conv '" + name + "': bad geometry");
             if (n.C < 1 || n.C > kMaxChannels) throw std::runtime_error("conv '" + name + "': bad channel count");
+            // C++ division truncates towards zero: a window larger than the padded input would come out as one output row
+            if (H + 2 * ph < kh || W + 2 * pw < kw) throw std::runtime_error("conv '" + name + "': kernel larger than the padded input");
             n.H = 1 + (H - kh + 2 * ph) / sh;
             n.W = 1 + (W - kw + 2 * pw) / sw;
             act_code(cfg["act"].as_string());
@@ -243,6 +245,7 @@ private:
                 const int ph = cfg["padding"][0].as_int(), pw = cfg["padding"][1].as_int();
                 if (sh < 1 || sw < 1 || kh < 1 || kw < 1 || ph < 0 || pw < 0 || std::max({kh, kw, sh, sw, ph, pw}) > kMaxExtent)
                     throw std::runtime_error("pool '" + name + "': bad geometry");
+                if (H + 2 * ph < kh || W + 2 * pw < kw) throw std::runtime_error("pool '" + name + "': window larger than the padded input");
                 n.H = 1 + (H - kh + 2 * ph) / sh;
                 n.W = 1 + (W - kw + 2 * pw) / sw;
             }

@@ -67,6 +67,8 @@ def _terms_to_config(terms):
 
 def _window_out(size, kernel, pad, stride):
     # floor formula shared by convolution and pooling (reference ir.py:388-393,538-542)
+    if size + 2 * pad < kernel:
+        raise ValueError(f'window of {kernel} does not fit an input of {size} with padding {pad}')
     return 1 + (size - kernel + 2 * pad) // stride
 
 

@@ -116,6 +116,50 @@ def test_host_planner_rejects_bad_operator_fields():
         assert rt.get_lib().ios_plan_describe(rt.c_string(text), 1, None, 0) == -1, text
 
 
+def test_json_reader_survives_hostile_documents():
+    """A backslash as the last byte, a truncated \\u escape and absurd nesting are errors, not crashes."""
+    lib = rt.get_lib()
+    for text, message in (('{"name": "abc\\', b'unterminated string'), ('["\\', b'unterminated string'),
+                          ('{"a\\u12', b'bad \\u escape'), ('["\\u', b'bad \\u escape'), ('["\\u00g0"]', b'bad \\u escape'),
+                          ('[' * 100000, b'nesting deeper'), ('{"a":' * 70 + '1' + '}' * 70, b'nesting deeper'),
+                          ('[' * 2000000, b'nesting deeper')):
+        assert lib.ios_plan_describe(rt.c_string(text), 1, None, 0) == -1, text[:20]
+        assert message in lib.ios_last_error(), (text[:20], lib.ios_last_error())
+    # 60 levels are fine for the reader (the planner then rejects the document for its content)
+    assert lib.ios_plan_describe(rt.c_string('[' * 60 + ']' * 60), 1, None, 0) == -1
+    assert b'nesting' not in lib.ios_last_error()
+
+
+def test_windows_larger_than_the_padded_input_are_rejected():
+    """Truncating division would turn a window that does not fit into one output row: both sides refuse instead."""
+    import copy
+    import json
+    ios.reset_name()
+    v = ios.placeholder((4, 6, 6))
+    block = ios.Block(v.node)
+    ios.conv2d(block, [[v]], 4, (3, 3), (2, 2), (0, 0), is_exit=True)
+    graph = ios.Graph('t', v.node, [block])
+    graph.sequential_schedule()
+    base = graph.export_config()
+    assert len(rt.plan_describe(graph, 1)) == 1
+    for shape in ([4, 2, 6], [4, 6, 2]):
+        doc = copy.deepcopy(base)
+        doc['input']['output_shape'] = shape
+        assert rt.get_lib().ios_plan_describe(rt.c_string(json.dumps(doc)), 1, None, 0) == -1
+        assert b'larger than the padded input' in rt.get_lib().ios_last_error()
+    doc = copy.deepcopy(base)
+    doc['input']['output_shape'] = [4, 2, 2]
+    doc['blocks'][0]['exit_node'].update({'type': 'pool', 'pool_type': 'max'})
+    assert rt.get_lib().ios_plan_describe(rt.c_string(json.dumps(doc)), 1, None, 0) == -1
+    assert b'larger than the padded input' in rt.get_lib().ios_last_error()
+    for build in (lambda b, x: ios.conv2d(b, [[x]], 4, (3, 3), (2, 2), (0, 0), is_exit=True),
+                  lambda b, x: ios.pool2d(b, [[x]], 'max', (3, 3), (2, 2), (0, 0), is_exit=True)):
+        ios.reset_name()
+        small = ios.placeholder((4, 2, 2))
+        with pytest.raises(ValueError, match='does not fit'):
+            build(ios.Block(small.node), small)
+
+
 def test_convolutions_of_parallel_stages_get_kernels_that_can_share_a_launch():
     """Host planner, closed-form kernel choice: every matrix-path convolution of a multi-group stage must be able
     to run inside a fused stage launch, at batch 1 and at a batch large enough for the LDS-tiled kernels."""
