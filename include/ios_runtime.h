@@ -75,6 +75,10 @@ int ios_set_option(const char *key, const char *value);
 /* JSON description of device 0 ({"name", "arch", "compute_units", ...}) into buf. */
 int ios_device_info(char *buf, int cap);
 
+/* JSON list of the convolution kernel configuration names this build holds, in index order, into buf; returns the
+ * length (call again with a larger buffer when the return value >= cap).  Touches no device. */
+int ios_conv_variant_names(char *buf, int cap);
+
 /* Host-only planning: writes the JSON list of device operations for a graph into buf and returns its length
  * (call again with a larger buffer when the return value >= cap); -1 on error.  Touches no device. */
 int ios_plan_describe(const char *graph_json, int batch_size, char *buf, int cap);

@@ -121,6 +121,14 @@ int ios_device_info(char *buf, int cap) {
     });
 }
 
+int ios_conv_variant_names(char *buf, int cap) {
+    std::string text = "[";
+    for (int i = 0; i < ios::conv_num_variants(); i++) text += std::string(i ? "," : "") + '"' + ios::conv_variant(i).name + '"';
+    text += "]";
+    if (buf != nullptr && cap > (int)text.size()) memcpy(buf, text.c_str(), text.size() + 1);
+    return (int)text.size();
+}
+
 int ios_plan_describe(const char *graph_json, int batch_size, char *buf, int cap) {
     int needed = -1;
     guarded([&]() {

@@ -54,6 +54,8 @@ def _declare(handle):
     handle.ios_set_option.restype = i
     handle.ios_device_info.argtypes = [ctypes.c_char_p, i]
     handle.ios_device_info.restype = i
+    handle.ios_conv_variant_names.argtypes = [ctypes.c_char_p, i]
+    handle.ios_conv_variant_names.restype = i
     handle.ios_plan_describe.argtypes = [s, i, ctypes.c_char_p, i]
     handle.ios_plan_describe.restype = i
     handle.ios_session_create.argtypes = [s, i]
@@ -110,6 +112,18 @@ def device_info() -> dict:
     buf = ctypes.create_string_buffer(4096)
     _check(get_lib().ios_device_info(buf, len(buf)), 'ios_device_info')
     return json.loads(buf.value.decode())
+
+
+def conv_variant_names() -> List[str]:
+    """Names of the convolution kernel configurations of this build, in index order (needs no GPU)."""
+    handle = get_lib()
+    cap = 1 << 14
+    while True:
+        buf = ctypes.create_string_buffer(cap)
+        need = handle.ios_conv_variant_names(buf, c_int(cap))
+        if need < cap:
+            return json.loads(buf.value.decode())
+        cap = need + 1
 
 
 def plan_describe(graph: Graph, batch_size=1) -> List[dict]:

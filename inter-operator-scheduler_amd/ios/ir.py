@@ -250,24 +250,36 @@ class Conv(Node):
     def fan_in(self):
         return self.kernel[0] * self.kernel[1] * self.input_shape[0] // self.groups
 
-    def init_weights(self, rng=None, scheme='uniform'):
+    def init_weights(self, rng=None, scheme='uniform', gain=1.0):
         """
         Fill ``weight``/``bias``.
 
         scheme 'uniform' draws both from U(-1/sqrt(fan_in), 1/sqrt(fan_in)) like the reference
-        (ir.py:360-363); scheme 'he_normal' draws weight ~ N(0, 2/fan_in) and sets bias to zero.
+        (ir.py:360-363); 'he_normal' draws weight ~ N(0, 2/fan_in) and sets bias to zero; 'he_normal_bias' adds a
+        bias ~ N(0, 0.1^2); 'bn_folded' is a convolution with a batch normalisation folded into it
+        (w' = w * gamma / sigma, b' = beta - mu * gamma / sigma): weight ~ N(0, gain/fan_in) times a per-channel
+        factor from U(0.75, 1.25), bias ~ N(0, 0.1^2), where the caller passes the ``gain`` that stands for
+        1 / sigma^2 of the convolution's unit-variance inputs (see Graph.init_weights).
         ``rng`` is a ``numpy.random.Generator``; ``None`` uses the global numpy state.
         """
+        normal = np.random.standard_normal if rng is None else rng.standard_normal
+        uniform = np.random.uniform if rng is None else rng.uniform
         if scheme == 'uniform':
             bound = 1.0 / np.sqrt(self.fan_in)
-            draw = np.random.uniform if rng is None else rng.uniform
-            self.weight = draw(low=-bound, high=bound, size=self.weight_shape).astype(np.float32)
-            self.bias = draw(low=-bound, high=bound, size=self.bias_shape).astype(np.float32)
-        elif scheme == 'he_normal':
+            self.weight = uniform(low=-bound, high=bound, size=self.weight_shape).astype(np.float32)
+            self.bias = uniform(low=-bound, high=bound, size=self.bias_shape).astype(np.float32)
+        elif scheme in ('he_normal', 'he_normal_bias'):
             std = np.sqrt(2.0 / self.fan_in)
-            draw = np.random.standard_normal if rng is None else rng.standard_normal
-            self.weight = (draw(size=self.weight_shape) * std).astype(np.float32)
-            self.bias = np.zeros(self.bias_shape, dtype=np.float32)
+            self.weight = (normal(size=self.weight_shape) * std).astype(np.float32)
+            if scheme == 'he_normal':
+                self.bias = np.zeros(self.bias_shape, dtype=np.float32)
+            else:
+                self.bias = (normal(size=self.bias_shape) * 0.1).astype(np.float32)
+        elif scheme == 'bn_folded':
+            std = np.sqrt(gain / self.fan_in)
+            per_channel = uniform(low=0.75, high=1.25, size=(self.out_channels, 1, 1, 1))
+            self.weight = (normal(size=self.weight_shape) * std * per_channel).astype(np.float32)
+            self.bias = (normal(size=self.bias_shape) * 0.1).astype(np.float32)
         else:
             raise ValueError(f'unknown init scheme {scheme}')
 
@@ -635,11 +647,45 @@ class Graph:
         Initialise every convolution.  Without arguments this is the reference behaviour
         (ir.py:1057-1070: unseeded uniform weights and biases).  With ``seed`` the draws come from
         ``numpy.random.default_rng(seed)`` in graph order; ``scheme='he_normal'`` gives N(0, 2/fan_in)
-        weights and zero bias.
+        weights and zero bias, ``'he_normal_bias'`` the same with a small seeded bias.
+
+        ``scheme='bn_folded'`` stands for networks whose convolutions carry a folded batch normalisation
+        (RandWire): every convolution is scaled so that unit-variance inputs give unit-variance outputs, i.e. its
+        weight variance is gain / fan_in with gain = 1 / (second moment of its input: sums add, a ReLU halves),
+        which is what dividing by the batch statistics' sigma would do.  Activations then stay O(1) at any depth
+        and fan-in.
         """
         rng = None if seed is None else np.random.default_rng(seed)
+        if scheme != 'bn_folded':
+            for conv in self.conv_nodes():
+                conv.init_weights(rng, scheme)
+            return
+
+        # second moment of every operator's output under this initialisation, for unit-variance network input:
+        # a convolution normalises to 1, a sum adds, a ReLU of a zero-mean value halves, concatenation takes the
+        # largest term, pooling keeps it
+        moment: Dict[str, float] = {}
+
+        def of_terms(terms) -> float:
+            return max(sum(moment_of(v.node) for v in term) for term in terms)
+
+        def moment_of(node: Node) -> float:
+            if node.name not in moment:
+                if isinstance(node, (Placeholder, Conv)):
+                    value = 1.0
+                elif isinstance(node, Sequential):
+                    value = moment_of(node.nodes[-1])
+                elif isinstance(node, Relu) or (isinstance(node, Activation) and node.act_type == 'relu'):
+                    value = of_terms(node.inputs) / 2.0
+                elif isinstance(node, Activation):
+                    value = 1.0      # tanh and sigmoid are bounded
+                else:                # identity (sums and concatenations), element, pool
+                    value = of_terms(node.inputs)
+                moment[node.name] = value
+            return moment[node.name]
+
         for conv in self.conv_nodes():
-            conv.init_weights(rng, scheme)
+            conv.init_weights(rng, scheme, gain=1.0 / of_terms(conv.inputs))
 
     def sequential_schedule(self):
         for block in self.blocks:

@@ -1,9 +1,11 @@
 """
 GPU parity: the HIP runtime, called through its C ABI, against the CPU oracle on the same seeded inputs.
-Tolerance for fp32: |got - want| <= atol + 1e-3 * |want| with atol = 1e-4 * max(1, max|want|): rel 1e-3 / abs 1e-4,
-the absolute part taken relative to the tensor's scale because the seeded He-normal networks without batch norm
-(RandWire, NASNet) reach activations of 1e4 and more, where single fp32 roundings already exceed 1e-4.
-With the kernel configuration pinned, schedule and executor changes must not change results at all.
+Tolerance for fp32: |got - want| <= 1e-4 + 1e-3 * |want| (rel 1e-3 / abs 1e-4), element by element, everywhere
+except NASNet under the He-normal initialisation its configuration names: without normalisation its activations
+reach 1e5, where one fp32 rounding is 8e-3, so that case is held to the same formula with the absolute part scaled
+by the tensor's largest magnitude and reports how many elements miss the unscaled formula and by how many ulps.
+Whole networks run with seeded non-zero biases.  With the kernel configuration pinned, schedule and executor
+changes must not change results at all.
 """
 import numpy as np
 import pytest
@@ -18,9 +20,9 @@ pytestmark = pytest.mark.gpu
 RTOL, ATOL = 1e-3, 1e-4
 
 
-def assert_close(got, want, what=''):
+def assert_close(got, want, what='', scaled=False):
     err = np.abs(got.astype(np.float64) - want.astype(np.float64))
-    scale = max(1.0, float(np.abs(want).max())) if want.size else 1.0
+    scale = max(1.0, float(np.abs(want).max())) if (scaled and want.size) else 1.0
     bound = ATOL * scale + RTOL * np.abs(want.astype(np.float64))
     bad = err > bound
     assert not bad.any(), (f'{what}: {bad.sum()} of {bad.size} elements out of tolerance, max abs err '
@@ -113,14 +115,14 @@ def test_committed_operator_vectors():
         assert_close(got, data[f'{name}.y'], name)
 
 
-@pytest.mark.parametrize('variant', range(80))
+# every fp32 kernel configuration the library was built with (host-only query; the bfloat16 ones have their own test)
+FP32_VARIANTS = [name for name in rt.conv_variant_names() if not name.startswith('wb_')]
+
+
+@pytest.mark.parametrize('variant_name', FP32_VARIANTS)
 @pytest.mark.parametrize('split_k', [1, 3])
-def test_every_conv_kernel_variant(variant, split_k):
-    names = rt.device_info()['conv_variants']
-    if variant >= len(names):
-        pytest.skip('no such kernel variant')
-    if names[variant].startswith('wb_'):
-        pytest.skip('reduced-precision configuration: see test_every_reduced_precision_kernel_configuration')
+def test_every_conv_kernel_variant(variant_name, split_k):
+    variant = rt.device_info()['conv_variants'].index(variant_name)
     rt.set_option('conv_variant', variant)
     rt.set_option('conv_split_k', split_k)
     for in_shape, oc, k, s, p, batch in [((72, 19, 19), 88, (3, 3), (1, 1), (1, 1), 2),
@@ -299,24 +301,37 @@ def test_sequential_units_and_folded_relu():
 
 
 def model_cases():
+    # (id, constructor, batch, strict tolerance).  Seeded non-zero biases everywhere; RandWire in the folded-batch-norm
+    # form its configuration describes; NASNet both under the He-normal initialisation its configuration names (scaled
+    # tolerance, see the module docstring) and in the folded form (strict).
     return [
-        ('sample', lambda: ios.models.sample_network(init_seed=0, init_scheme='he_normal'), 1),
-        ('squeezenet_1_1', lambda: ios.models.squeezenet_1_1(init_seed=0, init_scheme='he_normal'), 1),
-        ('inception_v3', lambda: ios.models.inception_v3(init_seed=0, init_scheme='he_normal'), 1),
-        ('randwire_small', lambda: ios.models.randwire_small(init_seed=0, init_scheme='he_normal'), 1),
-        ('nasnet_mobile', lambda: ios.models.nasnet_mobile(init_seed=0, init_scheme='he_normal'), 1),
-        ('inception_v3_b4', lambda: ios.models.inception_v3(init_seed=0, init_scheme='he_normal'), 4),
+        ('sample', lambda: ios.models.sample_network(init_seed=0, init_scheme='he_normal_bias'), 1, True),
+        ('squeezenet_1_1', lambda: ios.models.squeezenet_1_1(init_seed=0, init_scheme='he_normal_bias'), 1, True),
+        ('inception_v3', lambda: ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias'), 1, True),
+        ('randwire_small', lambda: ios.models.randwire_small(init_seed=0, init_scheme='bn_folded'), 1, True),
+        ('nasnet_mobile', lambda: ios.models.nasnet_mobile(init_seed=0, init_scheme='he_normal_bias'), 1, False),
+        ('nasnet_mobile_folded', lambda: ios.models.nasnet_mobile(init_seed=0, init_scheme='bn_folded'), 1, True),
+        ('inception_v3_b4', lambda: ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias'), 4, True),
     ]
 
 
-@pytest.mark.parametrize('name,make,batch', model_cases(), ids=[c[0] for c in model_cases()])
-def test_network_matches_oracle_under_every_schedule_and_executor(name, make, batch):
+def strict_misses(got, want):
+    """Elements outside |d| <= 1e-4 + 1e-3 |want|, and the largest error in units of the last place of the tensor's largest value."""
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    misses = int((err > ATOL + RTOL * np.abs(want.astype(np.float64))).sum())
+    ulp = float(np.spacing(np.float32(np.abs(want).max()))) if want.size else 1.0
+    return misses, float(err.max()) / ulp
+
+
+@pytest.mark.parametrize('name,make,batch,strict', model_cases(), ids=[c[0] for c in model_cases()])
+def test_network_matches_oracle_under_every_schedule_and_executor(name, make, batch, strict):
     """
     Outputs match the CPU oracle within tolerance for the sequential, greedy and dp_parallel schedules under
     every executor.  With the kernel configuration pinned (it otherwise depends on how many groups share a
     stage, which changes the summation order) all schedules and executors agree bit for bit.
     """
     graph = make()
+    assert any(np.abs(conv.bias).max() > 0 for conv in graph.conv_nodes())
     graph.sequential_schedule()
     x = np.random.default_rng(1).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
     want_all = ios_oracle.run(graph, x, keep_all=True)
@@ -326,11 +341,21 @@ def test_network_matches_oracle_under_every_schedule_and_executor(name, make, ba
         session.set_input(x)
         session.run()
         got = session.output()
-        if not np.allclose(got, want, rtol=RTOL, atol=ATOL):
-            # name the first operator that went wrong
-            for node in list(graph.nodes())[1:]:
-                assert_close(session.tensor(node), want_all[node.name], f'{name}: node {node.name} ({node.type})')
-    assert_close(got, want, name)
+        # every operator's output, node by node: names the first operator that goes wrong
+        report = []
+        for node in list(graph.nodes())[1:]:
+            tensor = session.tensor(node)
+            assert_close(tensor, want_all[node.name], f'{name}: node {node.name} ({node.type})', scaled=not strict)
+            if not strict:
+                misses, ulps = strict_misses(tensor, want_all[node.name])
+                if misses:
+                    report.append((node.name, misses, tensor.size, ulps))
+        if not strict:
+            # He-normal without normalisation: the misses of the unscaled formula are roundings at the tensor's scale
+            print(f'{name}: {len(report)} operators with elements outside |d| <= 1e-4 + 1e-3|want| '
+                  f'(worst: {max(report, key=lambda r: r[3]) if report else None}; node, elements, of, max error in ulps of the largest value)')
+            assert all(ulps <= 64.0 for _, _, _, ulps in report), report
+    assert_close(got, want, name, scaled=not strict)
     assert np.isfinite(got).all() and np.abs(got).max() > 0
 
     big = name.startswith(('randwire', 'nasnet'))
@@ -356,7 +381,7 @@ def test_network_matches_oracle_under_every_schedule_and_executor(name, make, ba
                     for _ in range(2):      # the second pass replays the captured graph
                         session.run()
                     outs[(executor, label)] = session.output()
-                assert_close(outs[(executor, label)], want, f'{name} {executor} {label} pinned={pinned}')
+                assert_close(outs[(executor, label)], want, f'{name} {executor} {label} pinned={pinned}', scaled=not strict)
         return outs
 
     run_all(pinned=False)
@@ -368,12 +393,74 @@ def test_network_matches_oracle_under_every_schedule_and_executor(name, make, ba
         np.testing.assert_array_equal(value, first, err_msg=str(key))
 
 
+def test_inception_batch_16_under_the_schedule_searched_at_that_batch():
+    """
+    The middle point of the batch sweep, the way the benchmark runs it: dp_parallel schedule searched with on-device stage
+    measurements at batch 16 (r = 1, s = 8), measured kernel configurations, fused launches replayed from a hipGraph;
+    sampled images against the oracle, which sees those images only.
+    """
+    batch = 16
+    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias')
+    rt.set_option('autotune', 1)
+    rt.set_option('executor', 'fused')
+    try:
+        optimized = ios.optimize(graph, batch_size=batch, opt_type='dp_parallel', compute_weight=True, warmup=1, number=2, repeat=1,
+                                 max_group_size=1, max_num_groups=8)
+        assert any(len(stage) > 1 for block in optimized.blocks for stage in block.stages)
+        x = np.random.default_rng(6).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
+        x[11] = x[3]
+        sample = [0, 3, 9, 15]
+        graph.sequential_schedule()
+        want = ios_oracle.run(graph, x[sample])
+        outs = {}
+        for executor, g in (('fused_graph', optimized), ('fused', optimized), ('fused_graph', graph)):
+            rt.set_option('executor', executor)
+            with rt.Session(g, batch) as session:
+                session.load_weights()
+                session.set_input(x)
+                for _ in range(2):
+                    session.run()
+                got = session.output()
+            assert got.shape[0] == batch and np.isfinite(got).all()
+            assert_close(got[sample], want, f'inception batch 16 {executor} {"dp_parallel" if g is optimized else "sequential"}')
+            np.testing.assert_array_equal(got[11], got[3])
+    finally:
+        rt.set_option('autotune', 0)
+        rt.set_option('executor', 'streams')
+
+
+@pytest.mark.parametrize('name', ['1', '16', '32', '64', '128', 'k80', 'v100'])
+def test_reference_schedule_files_run_and_match_the_plain_model(name):
+    """
+    The reference's own optimised schedules (experiments/specialization/schedules/*.json: merged convolutions read through
+    channel slices, up to five groups per stage), loaded unchanged and run at the batch size each was tuned for
+    (experiments/specialization/main.py:43-48).  With the plain model's weights stacked into the merged convolutions the
+    result must equal the plain model's on the oracle.
+    """
+    import reference_schedules
+    batch = reference_schedules.TUNED_BATCH[name]
+    plain = ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias')
+    plain.sequential_schedule()
+    graph = reference_schedules.load(name)
+    reference_schedules.adopt_weights(graph, plain)
+    x = np.random.default_rng(8).standard_normal((batch, 3, 299, 299)).astype(np.float32)
+    sample = sorted({0, batch // 2, batch - 1})
+    want = ios_oracle.run(plain, x[sample])
+    for executor in ('fused', 'streams'):
+        rt.set_option('executor', executor)
+        got = rt.graph_inference(graph, batch, x)
+        assert got.shape == (batch, 2048, 1, 1)
+        assert_close(got[sample], want, f'reference schedule {name}.json at batch {batch}, {executor}')
+    latency = rt.graph_latency(graph, batch, warmup=1, number=2, repeat=2)
+    assert len(latency) == 2 and all(v > 0 for v in latency)
+
+
 def test_large_batch_parallel_stages_with_measured_kernel_configurations():
     """
     At batch 32 no kernel configuration fits the share of the device a group of a parallel stage is budgeted,
     so the tuner falls back; whatever it picks must be able to run inside the fused stage launch.
     """
-    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias')
     graph.greedy_schedule(8)
     batch = 32
     x = np.random.default_rng(4).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
@@ -397,7 +484,7 @@ def test_batch_64_images_are_independent_and_match_the_oracle():
     image's output depends on that image alone, so a sample of the 64 outputs is checked against the oracle run
     on those images only, and two identical images inside the batch must give identical outputs.
     """
-    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias')
     graph.sequential_schedule()
     batch = 64
     x = np.random.default_rng(9).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
@@ -472,9 +559,9 @@ def test_every_reduced_precision_kernel_configuration():
 
 
 def test_reduced_precision_network_under_parallel_schedules():
-    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias')
     graph.sequential_schedule()
-    greedy = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    greedy = ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias')
     greedy.greedy_schedule(8)
     x = np.random.default_rng(1).standard_normal((2, *graph.enter_node.output_shape)).astype(np.float32)
     rt.set_option('precision', 'bf16')
@@ -498,7 +585,7 @@ def test_reduced_precision_network_under_parallel_schedules():
 
 
 def test_merged_convolutions_match_unmerged():
-    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias')
     merged = ios.optimize(graph, 1, ios.AnalyticCostModel(launch=1.0, rate=2e7, sync=1.5), 'dp_parallel_merge',
                           compute_weight=True)
     assert any(' ' in node.hint_name for node in merged.nodes())
@@ -530,7 +617,7 @@ def test_latency_entry_points():
 
 
 def test_optimize_with_measured_cost_model_on_sample_net():
-    graph = ios.models.sample_network(init_seed=0, init_scheme='he_normal')
+    graph = ios.models.sample_network(init_seed=0, init_scheme='he_normal_bias')
     optimized = ios.optimize(graph, batch_size=1, opt_type='dp_parallel', compute_weight=True, warmup=1, number=2, repeat=2)
     names = sorted(n for stage in optimized.blocks[0].stages for group in stage for n in group)
     assert names == ['1', '2', '3', '4', '5']
@@ -546,7 +633,7 @@ def test_measured_search_with_groups_of_one_operator_under_the_fused_executor():
     rt.set_option('autotune', 1)
     try:
         for make in (ios.models.squeezenet_1_1, ios.models.inception_v3):
-            graph = make(init_seed=0, init_scheme='he_normal')
+            graph = make(init_seed=0, init_scheme='he_normal_bias')
             optimized = ios.optimize(graph, batch_size=1, opt_type='dp_parallel', compute_weight=True, warmup=1, number=2, repeat=1,
                                      max_group_size=1, max_num_groups=8)
             stages = [stage for block in optimized.blocks for stage in block.stages]
@@ -567,7 +654,7 @@ def test_measured_search_with_groups_of_one_operator_under_the_fused_executor():
 def test_calls_from_two_host_threads_are_serialised():
     """The library keeps process-wide state; its entry points take a lock, so concurrent callers get correct results."""
     import threading
-    graph = ios.models.squeezenet_1_1(init_seed=0, init_scheme='he_normal')
+    graph = ios.models.squeezenet_1_1(init_seed=0, init_scheme='he_normal_bias')
     graph.greedy_schedule(8)
     x = np.random.default_rng(3).standard_normal((1, *graph.enter_node.output_shape)).astype(np.float32)
     want = ios_oracle.run(graph, x)

@@ -63,6 +63,61 @@ def test_inception_schedule_fixture_round_trip():
     assert seen == {str(i) for i in range(120)}
 
 
+@pytest.mark.parametrize('name', ['1', '16', '32', '64', '128', 'k80', 'v100'])
+def test_reference_schedule_files_load_round_trip_and_plan(name):
+    """
+    The reference's own schedule files (experiments/specialization/schedules/*.json, committed as fixtures): they load,
+    export back to the identical document, name the plain model's operators, and the host planner accepts them.
+    """
+    import reference_schedules
+    from ios.contrib import ios_runtime as rt
+    config = reference_schedules.load_config(name)
+    graph = Graph.from_config(config)
+    assert json.loads(json.dumps(graph.export_config())) == config
+    assert tuple(graph.enter_node.output_shape) == (3, 299, 299) and tuple(graph.exit_node.output_shape) == (2048, 1, 1)
+    plain = {n.name: n for n in ios.models.inception_v3().nodes()}
+    tokens = []
+    for node in graph.nodes():
+        tokens += node.hint_name.split()
+        if ' ' in node.hint_name:
+            assert node.type == 'conv' and node.out_channels == sum(plain[t].out_channels for t in node.hint_name.split())
+            continue
+        ref = plain[node.name]
+        assert node.type == ref.type and tuple(node.output_shape) == tuple(ref.output_shape) and node.hint_name == ref.hint_name
+        if node.type == 'conv':
+            assert (node.out_channels, tuple(node.kernel), tuple(node.stride), tuple(node.padding), node.groups, node.act) == \
+                   (ref.out_channels, tuple(ref.kernel), tuple(ref.stride), tuple(ref.padding), ref.groups, ref.act)
+        if node.type == 'pool':
+            assert (node.pool_type, tuple(node.kernel), tuple(node.stride), tuple(node.padding)) == \
+                   (ref.pool_type, tuple(ref.kernel), tuple(ref.stride), tuple(ref.padding))
+    # every operator of the plain model (placeholder 0, operators 1..119) appears exactly once, merged or not
+    assert sorted(tokens, key=int) == [str(i) for i in range(120)]
+    scheduled = sorted(n for block in graph.blocks for stage in block.stages for group in stage for n in group)
+    assert scheduled == sorted(n.name for n in graph.nodes() if n is not graph.enter_node)
+    ops = rt.plan_describe(graph, reference_schedules.TUNED_BATCH[name])
+    # slices of merged convolutions are read in place by convolutions and pools; only a slice that is itself a term of a
+    # block's concatenation is copied there (at most one per merged convolution)
+    assert {op['kind'] for op in ops} <= {'conv_mfma', 'pool', 'global_pool', 'unary'}
+    merged = sum(' ' in n.hint_name for n in graph.nodes())
+    assert sum(op['kind'] == 'unary' for op in ops) <= merged
+    assert sum(op['kind'] == 'conv_mfma' for op in ops) == sum(n.type == 'conv' for n in graph.nodes())
+
+
+def test_reference_schedule_weights_from_the_plain_model_reproduce_its_output_on_the_oracle():
+    """Stacked weights of the merged convolutions (reference optimizer.py:662-711): same network function."""
+    import reference_schedules
+    from oracle import ios_oracle
+    plain = ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias')
+    plain.sequential_schedule()
+    x = np.random.default_rng(2).standard_normal((1, 3, 299, 299)).astype(np.float32)
+    want = ios_oracle.run(plain, x)
+    for name in ('1', '64'):
+        graph = reference_schedules.load(name)
+        reference_schedules.adopt_weights(graph, plain)
+        got = ios_oracle.run(graph, x)
+        assert np.abs(got - want).max() <= 1e-5 * max(1.0, np.abs(want).max())
+
+
 def test_config_round_trip_all_models():
     for make in (ios.models.sample_network, ios.models.squeezenet_1_1, ios.models.squeezenet,
                  ios.models.randwire_small, ios.models.nasnet_mobile):
