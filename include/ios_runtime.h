@@ -56,6 +56,22 @@ int graph_inference(const char *graph_json, int batch_size, float *input, int nu
 
 /* ---- extensions without a counterpart in the reference ------------------------------------------------ */
 
+/*
+ * graph_inference for callers that cannot allocate device memory (harnesses that forbid hipMalloc, tight serving
+ * loops).  No counterpart in the reference.  Same arguments and results as graph_inference, but the call makes no
+ * hipMalloc / hipFree and creates no events or streams: every device buffer of the pass (operator outputs, filters,
+ * packed filters, split-K partial tiles and their ticket counters) is laid out in a static device array of
+ * IOS_NO_ALLOC_SCRATCH_BYTES that device 0 holds from library load to process end.  A graph whose plan needs more
+ * at the given batch size is refused with an error that names both figures.  Kernel configurations come from the
+ * tuning cache where a shape was measured before and from the closed-form model otherwise (nothing is measured here);
+ * operators run on one stream in schedule order.  All calls share the one array, which keeps the previous call's
+ * contents (what must start at zero is cleared by a fill kernel); the library's lock serialises calls inside a
+ * process, calls from several processes do not share the array.
+ */
+#define IOS_NO_ALLOC_SCRATCH_BYTES (256u << 20)
+int graph_inference_no_alloc(const char *graph_json, int batch_size, float *input, int num_convs, char **conv_names,
+                             float **filter_data, float **bias_data, float *output);
+
 /* Message of the most recent failure (valid until the next failing call). */
 const char *ios_last_error(void);
 
@@ -82,6 +98,10 @@ int ios_conv_variant_names(char *buf, int cap);
 /* Host-only planning: writes the JSON list of device operations for a graph into buf and returns its length
  * (call again with a larger buffer when the return value >= cap); -1 on error.  Touches no device. */
 int ios_plan_describe(const char *graph_json, int batch_size, char *buf, int cap);
+
+/* Host-only planning: bytes of device memory the plan of a graph lays out at a batch size (closed-form kernel
+ * configurations); -1 on error.  Touches no device. */
+long long ios_plan_arena_bytes(const char *graph_json, int batch_size);
 
 /* Persistent session: plan once, keep weights and activations on the device, run many times. */
 typedef struct ios_session ios_session;

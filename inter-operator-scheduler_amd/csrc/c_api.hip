@@ -104,6 +104,24 @@ int graph_inference(const char *graph_json, int batch_size, float *input, int nu
     });
 }
 
+int graph_inference_no_alloc(const char *graph_json, int batch_size, float *input, int num_convs, char **conv_names, float **filter_data,
+                             float **bias_data, float *output) {
+    return guarded([&]() {
+        const ios::Json doc = ios::Json::parse(graph_json);
+        ios::DeviceContext &ctx = ios::DeviceContext::get();
+        // cached kernel configurations are used, missing ones are not measured (measuring allocates scratch tensors)
+        ios::Plan plan = ios::build_plan(ios::PlanMode::Graph, doc, nullptr, batch_size,
+                                         [&ctx](const ios::ConvProblem &p, int share) { return ctx.choose_launch(p, share, /*allow_tuning=*/false); });
+        ios::Session session(std::move(plan), ios::Session::Storage::Static);
+        session.set_input(input);
+        if (num_convs > 0 && (conv_names == nullptr || filter_data == nullptr || bias_data == nullptr))
+            throw std::runtime_error("conv_names, filter_data or bias_data is null");
+        for (int i = 0; i < num_convs; i++) session.set_conv_weights(conv_names[i], filter_data[i], bias_data[i]);
+        session.run();
+        session.get_output(output);
+    });
+}
+
 const char *ios_last_error(void) { return g_last_error.c_str(); }
 
 int ios_set_option(const char *key, const char *value) {
@@ -141,6 +159,17 @@ int ios_plan_describe(const char *graph_json, int batch_size, char *buf, int cap
         if (buf != nullptr && cap > needed) memcpy(buf, text.c_str(), text.size() + 1);
     });
     return needed;
+}
+
+long long ios_plan_arena_bytes(const char *graph_json, int batch_size) {
+    long long bytes = -1;
+    guarded([&]() {
+        const ios::Json doc = ios::Json::parse(graph_json);
+        ios::Plan plan = ios::build_plan(ios::PlanMode::Graph, doc, nullptr, batch_size,
+                                         [](const ios::ConvProblem &p, int share) { return ios::conv_pick_launch(p, 256 / (share > 0 ? share : 1), share > 1); });
+        bytes = (long long)(plan.arena_floats * sizeof(float));
+    });
+    return bytes;
 }
 
 ios_session *ios_session_create(const char *graph_json, int batch_size) {

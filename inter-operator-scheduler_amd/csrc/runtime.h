@@ -50,7 +50,14 @@ public:
     // per problem signature for the life of the process, and in the file named by IOS_TUNE_CACHE when set),
     // else the closed-form model; the testing overrides win over both.
     // `share` = number of groups running concurrently with this convolution (1 = alone on the device).
-    ConvLaunch choose_launch(const ConvProblem &p, int share);
+    // allow_tuning = false never measures (measuring allocates scratch tensors): a shape that has no cached winner
+    // gets the closed-form choice.
+    ConvLaunch choose_launch(const ConvProblem &p, int share, bool allow_tuning = true);
+
+    // Static device scratch of the entry point that allocates nothing: address on device 0 (resolved once, when the
+    // context is created) and size in bytes.
+    float *static_scratch() const { return static_scratch_; }
+    static size_t static_scratch_bytes();
     static constexpr int kShareClasses = 4;   // footprint budgets 1, 1/2, 1/4, 1/8 of the device
     struct TunedConv {
         ConvLaunch best[kShareClasses];
@@ -62,6 +69,7 @@ private:
     TunedConv tune_conv(const ConvProblem &p);
     float *tuning_buffer(int which, size_t floats);
     unsigned *tuning_counters(size_t count);
+    float *static_scratch_ = nullptr;
     unsigned *tune_counters_ = nullptr;
     size_t tune_counter_count_ = 0;
     bool inline_reduce_ = true;
@@ -90,8 +98,12 @@ private:
 
 class Session {
 public:
-    // `shared` sessions live in the context's shared arena (one at a time), others own their memory
-    Session(Plan plan, bool shared);
+    // Where a session's device memory comes from: its own allocation, the context's shared arena (one such session at
+    // a time), or the static scratch array (one at a time; such a session allocates nothing, creates no events, and
+    // issues every operator on the main stream in schedule order whatever the executor option says).
+    enum class Storage { Own, Shared, Static };
+    Session(Plan plan, Storage storage);
+    Session(Plan plan, bool shared) : Session(std::move(plan), shared ? Storage::Shared : Storage::Own) {}
     ~Session();
     void release() noexcept;   // frees device memory, events and the captured graph; safe to call twice
     Session(const Session &) = delete;
@@ -121,6 +133,7 @@ private:
     void enqueue(bool stage_events);   // issue one forward pass according to the execution mode
     void enqueue_streams(bool stage_events);
     void enqueue_fused(bool stage_events);
+    void enqueue_serial();
     void build_fused();
     void forward();                    // enqueue or graph launch according to the execution mode
     void build_graph();
@@ -131,6 +144,7 @@ private:
     DeviceContext &ctx_;
     float *base_ = nullptr;
     bool owns_memory_ = false;
+    bool static_ = false;
     std::vector<hipEvent_t> fork_events_;                 // per stage (multi-group stages only)
     std::vector<std::vector<hipEvent_t>> join_events_;    // per stage, per extra group
     std::vector<hipEvent_t> stage_events_;                // per stage, profile mode

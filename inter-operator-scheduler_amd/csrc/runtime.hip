@@ -30,6 +30,16 @@ void hip_check(hipError_t status, const char *what, const char *file, int line) 
     throw std::runtime_error(os.str());
 }
 
+// ---- static scratch ----------------------------------------------------------------------------------------------
+// Device memory of graph_inference_no_alloc: a session created with Storage::Static lays its whole arena (operator
+// outputs, filters, packed filters, split-K partial tiles and ticket counters) out in this array instead of
+// allocating.  The device holds it from the moment the library is loaded until the process ends.  In host code
+// the array's name is only a handle for hipGetSymbolAddress; kernels and copies get the address resolved below.
+constexpr size_t kStaticScratchBytes = size_t(256) << 20;
+static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
+
+size_t DeviceContext::static_scratch_bytes() { return kStaticScratchBytes; }
+
 // ---- device context --------------------------------------------------------------------------------------------
 DeviceContext &DeviceContext::get() {
     static DeviceContext instance;
@@ -46,6 +56,8 @@ DeviceContext::DeviceContext() {
     name_ = prop.name;
     arch_ = prop.gcnArchName;
     for (int i = 0; i < kMaxGroups; i++) IOS_HIP(hipStreamCreateWithFlags(&streams_[i], hipStreamNonBlocking));
+    // the library runs on device 0 only, which is current here: its copy of the array is the one ever used
+    IOS_HIP(hipGetSymbolAddress(reinterpret_cast<void **>(&static_scratch_), HIP_SYMBOL(scratch)));
     const char *mode = getenv("IOS_EXECUTOR");
     if (mode != nullptr) set_option("executor", mode);
     const char *tune = getenv("IOS_AUTOTUNE");
@@ -273,16 +285,21 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     return result;
 }
 
-ConvLaunch DeviceContext::choose_launch(const ConvProblem &p, int share) {
+ConvLaunch DeviceContext::choose_launch(const ConvProblem &p, int share, bool allow_tuning) {
     int cls = 0;
     while (cls + 1 < kShareClasses && (1 << (cls + 1)) <= share) cls++;   // floor(log2(share)), capped
     ConvLaunch launch;
+    bool chosen = false;
     if (autotune_) {
         const std::string key = conv_signature(p) + " " + settings_token() + (bf16_ ? " bf16" : "");
         auto it = tuned.find(key);
-        if (it == tuned.end()) it = tuned.emplace(key, tune_conv(p)).first;
-        launch = it->second.best[cls];
-    } else {
+        if (it == tuned.end() && allow_tuning) it = tuned.emplace(key, tune_conv(p)).first;
+        if (it != tuned.end()) {
+            launch = it->second.best[cls];
+            chosen = true;
+        }
+    }
+    if (!chosen) {
         launch = conv_pick_launch(p, std::max(1, num_cus_ >> cls), cls > 0, bf16_);
     }
     if (forced_variant_ >= 0) launch.variant = forced_variant_;
@@ -372,8 +389,16 @@ std::string DeviceContext::info_json() const {
 }
 
 // ---- session ---------------------------------------------------------------------------------------------------------
-Session::Session(Plan plan, bool shared) : plan_(std::move(plan)), ctx_(DeviceContext::get()) {
-    if (shared) {
+Session::Session(Plan plan, Storage storage) : plan_(std::move(plan)), ctx_(DeviceContext::get()) {
+    if (storage == Storage::Static) {
+        const size_t need = plan_.arena_floats * sizeof(float);
+        if (need > DeviceContext::static_scratch_bytes())
+            throw std::runtime_error("graph needs " + std::to_string(need) + " bytes of device memory at this batch size; the static scratch of "
+                                     "graph_inference_no_alloc holds " + std::to_string(DeviceContext::static_scratch_bytes()));
+        base_ = ctx_.static_scratch();
+        owns_memory_ = false;
+        static_ = true;
+    } else if (storage == Storage::Shared) {
         base_ = ctx_.shared_arena(plan_.arena_floats);
         owns_memory_ = false;
     } else {
@@ -435,6 +460,10 @@ void Session::setup() {
         if (conv.ctr_count > 0) launch_fill_u32(reinterpret_cast<unsigned *>(base_ + conv.ctr_off), conv.ctr_count, 0u, main);
     }
     const size_t num_stages = plan_.stages.size();
+    if (static_) {   // no events: everything is issued on the main stream and the host waits for the stream
+        IOS_HIP(hipStreamSynchronize(main));
+        return;
+    }
     fork_events_.assign(num_stages, nullptr);
     join_events_.assign(num_stages, {});
     for (size_t s = 0; s < num_stages; s++) {
@@ -559,7 +588,19 @@ void Session::enqueue_streams(bool stage_events) {
     }
 }
 
+void Session::enqueue_serial() {
+    hipStream_t main = ctx_.stream(0);
+    for (const auto &groups : plan_.stages)
+        for (const auto &group : groups)
+            for (int op : group) launch_op(plan_.ops[op], main);
+}
+
 void Session::enqueue(bool stage_events) {
+    if (static_) {
+        if (stage_events) throw std::runtime_error("a session in the static scratch cannot profile stages");
+        enqueue_serial();
+        return;
+    }
     const ExecMode mode = ctx_.exec_mode();
     if (mode == ExecMode::Fused || mode == ExecMode::FusedGraph) enqueue_fused(stage_events);
     else enqueue_streams(stage_events);
@@ -726,6 +767,10 @@ void Session::build_graph() {
 }
 
 void Session::forward() {
+    if (static_) {
+        enqueue_serial();
+        return;
+    }
     const ExecMode mode = ctx_.exec_mode();
     if (mode == ExecMode::Graph || mode == ExecMode::FusedGraph) {
         if (graph_exec_ != nullptr && graph_mode_ != mode) {   // the option changed since the capture
@@ -751,6 +796,7 @@ void Session::run() {
 }
 
 void Session::measure(int warmup, int number, int repeat, bool profile_stage, float *results, float *stage_results) {
+    if (static_) throw std::runtime_error("a session in the static scratch has no timers");
     if (number < 1 || repeat < 1 || warmup < 0) throw std::runtime_error("measure: warmup >= 0, number >= 1, repeat >= 1 required");
     hipStream_t main = ctx_.stream(0);
     const size_t num_stages = plan_.stages.size();
@@ -792,6 +838,7 @@ void Session::measure(int warmup, int number, int repeat, bool profile_stage, fl
 }
 
 void Session::measure_back_to_back(int warmup, int number, int repeat, float *results) {
+    if (static_) throw std::runtime_error("a session in the static scratch has no timers");
     if (number < 1 || repeat < 1 || warmup < 0) throw std::runtime_error("measure: warmup >= 0, number >= 1, repeat >= 1 required");
     hipStream_t main = ctx_.stream(0);
     for (int i = 0; i < warmup; i++) forward();
@@ -809,6 +856,7 @@ void Session::measure_back_to_back(int warmup, int number, int repeat, float *re
 }
 
 void Session::profile_ops(int warmup, int repeat, float *ms_out) {
+    if (static_) throw std::runtime_error("a session in the static scratch has no timers");
     if (repeat < 1 || warmup < 0) throw std::runtime_error("profile_ops: warmup >= 0 and repeat >= 1 required");
     hipStream_t main = ctx_.stream(0);
     run();   // every operator sees the inputs it has in a real pass

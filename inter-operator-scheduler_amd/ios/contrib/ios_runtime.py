@@ -46,7 +46,8 @@ def _declare(handle):
     handle.stage_latency.argtypes = [s, s, i, i, i, i, i, f32p, f32p]
     handle.graph_inference.argtypes = [s, i, vp, i, ctypes.POINTER(s), ctypes.POINTER(vp),
                                        ctypes.POINTER(vp), vp]
-    for name in ('graph_latency', 'block_latency', 'stage_latency', 'graph_inference'):
+    handle.graph_inference_no_alloc.argtypes = handle.graph_inference.argtypes
+    for name in ('graph_latency', 'block_latency', 'stage_latency', 'graph_inference', 'graph_inference_no_alloc'):
         getattr(handle, name).restype = i
     handle.ios_last_error.restype = s
     handle.ios_last_error.argtypes = []
@@ -58,6 +59,8 @@ def _declare(handle):
     handle.ios_conv_variant_names.restype = i
     handle.ios_plan_describe.argtypes = [s, i, ctypes.c_char_p, i]
     handle.ios_plan_describe.restype = i
+    handle.ios_plan_arena_bytes.argtypes = [s, i]
+    handle.ios_plan_arena_bytes.restype = ctypes.c_longlong
     handle.ios_session_create.argtypes = [s, i]
     handle.ios_session_create.restype = vp
     handle.ios_session_destroy.argtypes = [vp]
@@ -141,6 +144,14 @@ def plan_describe(graph: Graph, batch_size=1) -> List[dict]:
         cap = need + 1
 
 
+def plan_arena_bytes(graph: Graph, batch_size=1) -> int:
+    """Device memory the library lays out for ``graph`` at ``batch_size`` (host-only planning, needs no GPU)."""
+    need = get_lib().ios_plan_arena_bytes(c_string(json.dumps(graph.export_config())), c_int(batch_size))
+    if need < 0:
+        _check(1, 'ios_plan_arena_bytes')
+    return int(need)
+
+
 def _latency_call(fn_name, documents, batch_size, warmup, number, repeat, num_stages, profile_stage):
     handle = get_lib()
     results = c_float_array(repeat)
@@ -202,8 +213,11 @@ def _weight_lists(graph: Graph):
     return names, weights, biases
 
 
-def graph_inference(graph: Graph, batch_size, input: np.ndarray):
-    """Run ``graph`` on ``input`` (batch, C, H, W) with the weights stored in its Conv operators."""
+def graph_inference(graph: Graph, batch_size, input: np.ndarray, no_alloc=False):
+    """
+    Run ``graph`` on ``input`` (batch, C, H, W) with the weights stored in its Conv operators.  ``no_alloc`` calls the
+    library's variant that lays all device buffers out in its static scratch array and allocates nothing.
+    """
     handle = get_lib()
     x = as_f32(input)
     expected = (batch_size, *graph.enter_node.output_shape)
@@ -212,13 +226,14 @@ def graph_inference(graph: Graph, batch_size, input: np.ndarray):
     output = np.empty(shape=(batch_size, *graph.blocks[-1].exit_node.output_shape), dtype=np.float32)
     names, weights, biases = _weight_lists(graph)
     name_array = c_string_list(names)
-    status = handle.graph_inference(c_string(json.dumps(graph.export_config())), c_int(batch_size),
+    entry = handle.graph_inference_no_alloc if no_alloc else handle.graph_inference
+    status = entry(c_string(json.dumps(graph.export_config())), c_int(batch_size),
                                     x.ctypes.data_as(ctypes.c_void_p), c_int(len(names)),
                                     ctypes.cast(name_array, ctypes.POINTER(ctypes.c_char_p)),
                                     ctypes.cast(c_ndarray_list(weights), ctypes.POINTER(ctypes.c_void_p)),
                                     ctypes.cast(c_ndarray_list(biases), ctypes.POINTER(ctypes.c_void_p)),
                                     output.ctypes.data_as(ctypes.c_void_p))
-    _check(status, 'graph_inference')
+    _check(status, 'graph_inference_no_alloc' if no_alloc else 'graph_inference')
     return output
 
 
