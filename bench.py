@@ -3,16 +3,22 @@ Benchmark of the north-star path: Inception-v3 at batch 1 under the dp_parallel 
 dynamic-programming search with on-device stage measurements, on one MI355X.
 
 A step is one forward pass over one synthetic batch (weights and input already resident in HBM).  Prints one
-JSON line.  `roofline`: the convolution kernels of one pass, achieved = algorithmic FLOPs / HIP-event time of
-their launches on the launch stream, against the fp32 matrix peak.  `cpu_baseline`: the CPU oracle on the same
-graph, weights and input, timed on the host cores for about ten seconds.
+JSON line.
 
-Probe modes for the profiler (`--probe copy`, `--probe pass`) run a fixed small workload and print what the
-counters should be compared with; they are used by the commands recorded under profiles/.
+`roofline` describes the kernel that takes the largest share of the timed pass: every launch of that pass (under the
+executor that is timed) is issued back to back on the launch stream between two HIP events, launches are grouped by
+kernel, and the dominant kernel's algorithmic FLOPs (or bytes) are divided by its time.  `kernels` lists the same
+figures for every kernel of the pass.  `cpu_baseline`: the CPU oracle on the same graph, weights and input, timed on
+the host cores for about ten seconds.  Every configuration network and every batch of the sweep is also compared with
+the oracle under the strict tolerance |d| <= 1e-4 + 1e-3 |want|.
+
+Probe modes for the profiler (`--probe copy | search | pass`) run a fixed small workload and print what the counters
+should be compared with; they are used by the commands recorded under profiles/.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -23,10 +29,17 @@ for path in (ROOT, os.path.join(ROOT, 'inter-operator-scheduler_amd')):
 
 PEAK_FP32_MATRIX_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per convolution launch of a batch-1 Inception-v3 pass, from FETCH_SIZE / WRITE_SIZE counter runs scaled by a
-# copy kernel of known size (profiles/conv_kernel_hbm_traffic_inception_v3.md); counters cannot be read from inside this
-# script, so the figure is the offline measurement of the same kernels.
-MEASURED_CONV_TRAFFIC_BYTES_PER_LAUNCH = {1: 4.43e6, 64: 82.9e6}
+# configuration networks: constructor name, initialisation (RandWire: batch norm folded into the convolutions, as its
+# configuration says; the others seeded He-normal with zero bias)
+CONFIG_MODELS = {'sample_net': ('sample_network', 'he_normal'), 'squeezenet_1_1': ('squeezenet_1_1', 'he_normal'),
+                 'inception_v3': ('inception_v3', 'he_normal'), 'randwire_small': ('randwire_small', 'bn_folded'),
+                 'nasnet_mobile': ('nasnet_mobile', 'he_normal')}
+TRAFFIC_PROFILE = os.path.join(ROOT, 'profiles', 'hbm_traffic_by_kernel_inception_v3_batch1_dp_parallel.md')
+
+
+def make_graph(ios, name):
+    constructor, scheme = CONFIG_MODELS[name]
+    return getattr(ios.models, constructor)(init_seed=0, init_scheme=scheme)
 
 
 def op_bound_ms(op):
@@ -60,50 +73,119 @@ def timed_latency(rt, np, graph, batch, x, steps, warmup):
                 'events_std': float(np.std(events))}, session.output()
 
 
-def conv_roofline(rt, graph, batch, x, stages=False):
-    """Per-kernel HIP-event timing of one pass; returns (ops, ms per op, conv summary, memory-bound GB/s[, stage ms])."""
+def oracle_check(np, got, want):
+    """Strict tolerance of the path (rel 1e-3 / abs 1e-4, element by element) and how far the misses are."""
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    misses = int((err > 1e-4 + 1e-3 * np.abs(want.astype(np.float64))).sum())
+    scale = float(np.abs(want).max())
+    return {'matches_cpu_oracle': misses == 0, 'elements': int(want.size), 'elements_out_of_tolerance': misses,
+            'max_abs_err': float(err.max()), 'output_scale': scale,
+            'max_err_in_ulps_of_largest_output': float(err.max() / np.spacing(np.float32(scale)))}
+
+
+def launch_profile(rt, graph, batch, x, stages=False):
+    """
+    Every launch of one pass under the executor in force, timed back to back with HIP events on the launch stream.
+    Returns (ops, launches with 'ms', per-kernel totals[, per-stage ms of whole passes]).
+    """
     with rt.Session(graph, batch) as session:
         session.load_weights()
         session.set_input(x)
+        for _ in range(3):
+            session.run()
         ops = session.describe()
-        op_ms = session.profile_ops(warmup=3, repeat=20)
+        launches = session.launches()
+        for launch, ms in zip(launches, session.profile_launches(warmup=3, repeat=20)):
+            launch['ms'] = ms
         stage_ms = None
         if stages:
             repeat = 6
             _, per_stage = session.measure(warmup=2, number=6, repeat=repeat, profile_stage=True)
             count = len(per_stage) // repeat
             stage_ms = [sum(per_stage[r * count + i] for r in range(repeat)) / repeat for i in range(count)]
-    conv = [(op, ms) for op, ms in zip(ops, op_ms) if op['kind'] == 'conv_mfma']
-    flops = sum(op['flops'] for op, _ in conv)
-    ms = sum(t for _, t in conv)
-    mem = [(op, t) for op, t in zip(ops, op_ms) if op['kind'] in ('pool', 'global_pool', 'nary', 'unary', 'conv_depthwise')]
-    mem_gbs = (sum(op['bytes'] for op, _ in mem) / (sum(t for _, t in mem) * 1e-3) / 1e9) if mem else None
-    achieved = flops / (ms * 1e-3) / 1e12
-    summary = {'bound': 'mfma', 'kernel': f'conv_kernel<...> ({len(conv)} convolution launches of one pass)',
-               'achieved': achieved, 'peak': PEAK_FP32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
-               'frac': achieved / PEAK_FP32_MATRIX_TFLOPS, 'traffic': MEASURED_CONV_TRAFFIC_BYTES_PER_LAUNCH.get(batch),
-               'traffic_unit': 'bytes per launch (offline counter runs)',
-               'algorithmic_bytes_per_launch': sum(op['bytes'] for op, _ in conv) / len(conv),
-               'algorithmic_flops_per_launch': flops / len(conv), 'avg_launch_us': ms / len(conv) * 1e3,
-               'flops_per_pass': flops, 'kernel_ms_per_pass': ms, 'launches': len(conv)}
+    kernels = {}
+    for launch in launches:
+        k = kernels.setdefault(launch['kernel'], {'launches': 0, 'ms': 0.0, 'flops': 0.0, 'matrix_flops': 0.0, 'bytes': 0.0})
+        k['launches'] += 1
+        for key in ('ms', 'flops', 'matrix_flops', 'bytes'):
+            k[key] += launch[key]
+    for k in kernels.values():
+        k['tflops'] = k['matrix_flops'] / (k['ms'] * 1e-3) / 1e12
+        k['gbs'] = k['bytes'] / (k['ms'] * 1e-3) / 1e9
+        k['avg_launch_us'] = k['ms'] / k['launches'] * 1e3
+        k['mfma_bound'] = k['matrix_flops'] / (PEAK_FP32_MATRIX_TFLOPS * 1e12) > k['bytes'] / (PEAK_HBM_GBS * 1e9)
     if stages:
-        return ops, op_ms, summary, mem_gbs, stage_ms
-    return ops, op_ms, summary, mem_gbs
+        return ops, launches, kernels, stage_ms
+    return ops, launches, kernels
 
 
-def stage_overlap(ops, op_ms, stage_ms):
-    """Multi-group stages: time of their operators launched one by one against the measured time of the stage."""
-    groups, alone = {}, {}
+def committed_traffic(kernel):
+    """HBM bytes per launch of `kernel` from the committed counter summary (None when the summary has no such row)."""
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                match = re.match(r'\|\s*`([^`]+)`\s*\|(.*)\|\s*$', line)
+                if match and match.group(1) == kernel:
+                    cells = [c.strip() for c in match.group(2).split('|')]
+                    return float(cells[-1]) * 1e6    # last column: traffic per launch, MB
+    except (OSError, ValueError):
+        pass
+    return None
+
+
+def roofline_block(kernels, ms_per_step, headline=False):
+    """The roofline object of the kernel with the largest share of the pass (counter traffic exists for the headline pass only)."""
+    name, k = max(kernels.items(), key=lambda item: item[1]['ms'])
+    if k['mfma_bound']:
+        bound, achieved, peak, unit = 'mfma', k['tflops'], PEAK_FP32_MATRIX_TFLOPS, 'TFLOP/s'
+    else:
+        bound, achieved, peak, unit = 'hbm', k['gbs'], PEAK_HBM_GBS, 'GB/s'
+    block = {'bound': bound, 'kernel': name, 'achieved': achieved, 'peak': peak, 'unit': unit, 'frac': achieved / peak,
+             'traffic': committed_traffic(name) if headline else None,
+             'launches_per_pass': k['launches'], 'avg_launch_us': k['avg_launch_us'],
+             'algorithmic_flops_per_launch': k['matrix_flops'] / k['launches'],
+             'algorithmic_bytes_per_launch': k['bytes'] / k['launches'],
+             'kernel_ms_per_pass': k['ms'], 'share_of_launch_time': k['ms'] / sum(v['ms'] for v in kernels.values()),
+             'all_launches_ms_per_pass': sum(v['ms'] for v in kernels.values())}
+    if headline:
+        block['traffic_source'] = ('bytes per launch, FETCH_SIZE + WRITE_SIZE counter runs of the same pass, read from '
+                                   + os.path.relpath(TRAFFIC_PROFILE, ROOT))
+    assert block['kernel_ms_per_pass'] <= ms_per_step, (block['kernel_ms_per_pass'], ms_per_step)
+    return block
+
+
+def memory_bound_ops(rt, graph, batch, x):
+    """Achieved GB/s of the memory-bound operators of a pass, by kind (each launched back to back on one stream)."""
+    rt.set_option('executor', 'streams')      # one launch per operator
+    with rt.Session(graph, batch) as session:
+        session.load_weights()
+        session.set_input(x)
+        ops = session.describe()
+        op_ms = session.profile_ops(warmup=3, repeat=20)
+    kinds = {}
     for op, ms in zip(ops, op_ms):
-        if op['stage'] < 0:
-            continue
-        groups.setdefault(op['stage'], set()).add(op['group'])
-        alone[op['stage']] = alone.get(op['stage'], 0.0) + ms
+        if op['kind'] in ('pool', 'global_pool', 'nary', 'unary', 'conv_depthwise'):
+            k = kinds.setdefault(op['kind'], {'launches': 0, 'ms': 0.0, 'bytes': 0.0})
+            k['launches'] += 1
+            k['ms'] += ms
+            k['bytes'] += op['bytes']
+    for k in kinds.values():
+        k['gbs'] = k['bytes'] / (k['ms'] * 1e-3) / 1e9
+        k['frac_of_hbm_peak'] = k['gbs'] / PEAK_HBM_GBS
+    return kinds
+
+
+def stage_overlap(ops, launches, stage_ms):
+    """Multi-group stages: time of their operators' bounds and launches against the measured time of the stage."""
+    groups = {}
+    for op in ops:
+        if op['stage'] >= 0:
+            groups.setdefault(op['stage'], set()).add(op['group'])
     multi = [s for s, g in groups.items() if len(g) > 1 and s < len(stage_ms)]
     if not multi:
         return None
-    return {'multi_group_stages': len(multi), 'operators_one_by_one_ms': sum(alone[s] for s in multi),
-            'stages_measured_ms': sum(stage_ms[s] for s in multi),
+    return {'multi_group_stages': len(multi), 'stages_measured_ms': sum(stage_ms[s] for s in multi),
+            'their_launches_back_to_back_ms': sum(l['ms'] for l in launches if l['stage'] in multi),
             'single_group_stages_ms': sum(ms for s, ms in enumerate(stage_ms) if s not in multi)}
 
 
@@ -129,21 +211,52 @@ def probe(args, np, ios, rt):
                           'write_bytes_per_launch': nbytes, 'ms_per_launch': ms,
                           'gbs': 2 * nbytes / (ms * 1e-3) / 1e9}))
         return
-    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
-    graph.sequential_schedule()
-    x = np.random.default_rng(1).standard_normal((args.batch, 3, 299, 299)).astype(np.float32)
-    rt.set_option('executor', 'streams')
-    with rt.Session(graph, args.batch) as session:
+    graph = make_graph(ios, args.model)
+    batch = args.batch
+    if args.probe == 'search':
+        # measured schedule search (fills the kernel-configuration cache named by IOS_TUNE_CACHE), schedule written to a file
+        rt.set_option('executor', args.search_executor)
+        t0 = time.time()
+        optimized = ios.optimize(graph, batch_size=batch, opt_type='dp_parallel', compute_weight=True, warmup=2,
+                                 number=args.search_number, repeat=args.search_repeat,
+                                 max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
+        with open(args.schedule_file, 'w') as f:
+            json.dump(optimized.export_config(), f)
+        print(json.dumps({'probe': 'search', 'model': args.model, 'batch': batch, 'search_seconds': time.time() - t0,
+                          'stages': sum(len(b.stages) for b in optimized.blocks), 'schedule_file': args.schedule_file}))
+        return
+    # --probe pass: N passes of one plan and nothing else that launches kernels of the same names
+    if args.schedule_file:
+        with open(args.schedule_file) as f:
+            scheduled = ios.Graph.from_config(json.load(f))
+        scheduled.init_weights(0, CONFIG_MODELS[args.model][1])
+        schedule = 'dp_parallel (from ' + os.path.basename(args.schedule_file) + ')'
+    else:
+        scheduled = graph
+        scheduled.sequential_schedule()
+        schedule = 'sequential'
+    x = np.random.default_rng(1).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
+    rt.set_option('executor', args.executor)
+    with rt.Session(scheduled, batch) as session:
         session.load_weights()
         session.set_input(x)
-        for _ in range(3):
+        for _ in range(args.passes):
             session.run()
         ops = session.describe()
-    conv = [op for op in ops if op['kind'] == 'conv_mfma']
-    print(json.dumps({'probe': 'pass', 'batch': args.batch, 'passes': 3, 'schedule': 'sequential',
-                      'conv_launches_per_pass': len(conv),
-                      'conv_algorithmic_bytes_per_pass': sum(op['bytes'] for op in conv),
-                      'conv_flops_per_pass': sum(op['flops'] for op in conv)}))
+        launches = session.launches()
+    kernels = {}
+    for launch in launches:
+        k = kernels.setdefault(launch['kernel'], {'launches_per_pass': 0, 'flops_per_pass': 0.0, 'bytes_per_pass': 0.0})
+        k['launches_per_pass'] += 1
+        k['flops_per_pass'] += launch['flops']
+        k['bytes_per_pass'] += launch['bytes']
+    print(json.dumps({'probe': 'pass', 'model': args.model, 'batch': batch, 'passes': args.passes, 'schedule': schedule,
+                      'executor': args.executor, 'kernels': kernels,
+                      'launches': [{'stage': l['stage'], 'kernel': l['kernel'], 'blocks': l['blocks'], 'flops': l['flops'],
+                                    'bytes': l['bytes'],
+                                    'ops': [{'node': ops[i]['node'], 'kind': ops[i]['kind'], 'conv': ops[i].get('conv'),
+                                             'out': ops[i]['out'], 'variant': ops[i].get('variant'), 'flops': ops[i]['flops'],
+                                             'bytes': ops[i]['bytes']} for i in l['ops']]} for l in launches]}))
 
 
 def main():
@@ -169,15 +282,20 @@ def main():
     parser.add_argument('--search-restarts', type=int, default=2,
                         help='schedule searches to run (stage measurements are noisy: the schedule that measures faster as a whole is kept)')
     parser.add_argument('--no-sweep', action='store_true', help='skip the batch 16 / 64 sweep')
-    parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg and the oracle comparisons')
     parser.add_argument('--no-configs', action='store_true', help='skip the other four configuration networks')
+    parser.add_argument('--no-extras', action='store_true',
+                        help='skip the r = 3 and merged-convolution searches, the reduced-precision mode and the reference table variants')
     parser.add_argument('--greedy-big', action='store_true',
                         help='use the greedy schedule for RandWire and NASNet instead of the measured search (half a minute each at r = 1, '
                              'minutes at r = 3)')
     parser.add_argument('--search-variants', action='store_true',
                         help="measured schedule search also for the reference table's large model variants (about two more minutes)")
     parser.add_argument('--option', action='append', default=[], metavar='KEY=VALUE', help='extra runtime option (repeatable)')
-    parser.add_argument('--probe', choices=['copy', 'pass'], help='run a profiler probe instead of the benchmark')
+    parser.add_argument('--probe', choices=['copy', 'search', 'pass'], help='run a profiler probe instead of the benchmark')
+    parser.add_argument('--model', default='inception_v3', choices=sorted(CONFIG_MODELS), help='network of the search / pass probes')
+    parser.add_argument('--schedule-file', help='probe search: where to write the schedule; probe pass: schedule to run (default: sequential)')
+    parser.add_argument('--passes', type=int, default=3, help='forward passes of the pass probe')
     args = parser.parse_args()
     if args.gpus != 1:
         print('bench.py: this runtime is a single-GPU path; run with --gpus 1', file=sys.stderr)
@@ -191,9 +309,12 @@ def main():
         probe(args, np, ios, rt)
         return
 
+    if not args.no_cpu:
+        from oracle import ios_oracle
+
     device = rt.device_info()
     batch = args.batch
-    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal')
+    graph = make_graph(ios, 'inception_v3')
     x = np.random.default_rng(1).standard_normal((batch, 3, 299, 299)).astype(np.float32)
 
     # schedule search with measured stage latencies (not part of the timed steps)
@@ -221,12 +342,13 @@ def main():
     seq, seq_out = timed_latency(rt, np, graph, batch, x, args.steps, args.warmup)
     opt, opt_out = timed_latency(rt, np, optimized, batch, x, args.steps, args.warmup)
 
-    # kernel roofline: every convolution in the configuration it runs with when it has the device to itself (the
-    # sequential plan); inside the fused stage launches of the dp_parallel plan kernels cannot be timed one by one
-    _, _, roofline, mem_gbs = conv_roofline(rt, graph, batch, x)
-    ops, op_ms, _, _, stage_ms = conv_roofline(rt, optimized, batch, x, stages=True)
+    # the launches of the timed pass, under the executor that was timed
+    ops, launches, kernels, stage_ms = launch_profile(rt, optimized, batch, x, stages=True)
+    _, _, seq_kernels = launch_profile(rt, graph, batch, x)
     roof_seq = network_roofline_ms(ops, parallel=False)
     roof_par = network_roofline_ms(ops, parallel=True)
+    conv_flops = sum(op['flops'] for op in ops if op['kind'] == 'conv_mfma')
+    total_bytes = sum(op['bytes'] for op in ops)
 
     result = {
         'metric': 'batch-1 latency (ms) + images/s, Inception-v3 IOS dp_parallel schedule',
@@ -248,41 +370,49 @@ def main():
         'max_abs_diff_between_schedules': float(np.abs(seq_out - opt_out).max()),
         'search_seconds': search_s,
         'num_stages': sum(len(b.stages) for b in optimized.blocks),
+        'launches_per_pass': len(launches),
         'network_roofline_ms': {'sequential': roof_seq, 'critical_path': roof_par,
                                 'fraction_of_critical_path_roofline': roof_par / opt['wall'],
                                 'fraction_of_sequential_roofline': roof_seq / opt['wall']},
-        'roofline': roofline,
-        'memory_bound_ops_gbs': mem_gbs,
-        'stage_overlap': stage_overlap(ops, op_ms, stage_ms),
+        'whole_pass': {'matrix_tflops': conv_flops / (opt['wall'] * 1e-3) / 1e12,
+                       'frac_of_fp32_matrix_peak': conv_flops / (opt['wall'] * 1e-3) / 1e12 / PEAK_FP32_MATRIX_TFLOPS,
+                       'algorithmic_gbs': total_bytes / (opt['wall'] * 1e-3) / 1e9},
+        'roofline': roofline_block(kernels, opt['wall'], headline=True),
+        'kernels': kernels,
+        'kernels_sequential_pass': seq_kernels,
+        'stage_overlap': stage_overlap(ops, launches, stage_ms),
         'device': {k: device[k] for k in ('name', 'arch', 'compute_units')},
     }
+    result['memory_bound_ops_gbs'] = memory_bound_ops(rt, graph, batch, x)
+    rt.set_option('executor', args.executor)
 
-    # the same search with the reference's default pruning (r = 3, s = 8), for comparison with the headline's r and s
-    if (args.max_group_size, args.max_num_groups) != (3, 8):
+    if not args.no_extras:
+        # the same search with the reference's default pruning (r = 3, s = 8), for comparison with the headline's r and s
+        if (args.max_group_size, args.max_num_groups) != (3, 8):
+            rt.set_option('executor', args.search_executor)
+            t0 = time.time()
+            default_knobs = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
+                                         warmup=2, number=args.search_number, repeat=args.search_repeat)
+            default_search_s = time.time() - t0
+            graph.sequential_schedule()
+            rt.set_option('executor', args.executor)
+            r3, _ = timed_latency(rt, np, default_knobs, batch, x, args.steps, args.warmup)
+            result['dp_parallel_r3_s8'] = {'latency_ms': r3, 'images_per_s': batch / (r3['wall'] * 1e-3), 'search_seconds': default_search_s,
+                                           'num_stages': sum(len(b.stages) for b in default_knobs.blocks)}
+
+        # the reference's best schedule family (parallel groups + merged convolutions, "IOS-Both"); the headline metric
+        # is the dp_parallel schedule, this one is reported beside it
         rt.set_option('executor', args.search_executor)
         t0 = time.time()
-        default_knobs = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
-                                     warmup=2, number=args.search_number, repeat=args.search_repeat)
-        default_search_s = time.time() - t0
+        merged = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel_merge', compute_weight=True,
+                              warmup=2, number=args.search_number, repeat=args.search_repeat)
+        merge_search_s = time.time() - t0
         graph.sequential_schedule()
         rt.set_option('executor', args.executor)
-        r3, _ = timed_latency(rt, np, default_knobs, batch, x, args.steps, args.warmup)
-        result['dp_parallel_r3_s8'] = {'latency_ms': r3, 'images_per_s': batch / (r3['wall'] * 1e-3), 'search_seconds': default_search_s,
-                                       'num_stages': sum(len(b.stages) for b in default_knobs.blocks)}
-
-    # the reference's best schedule family (parallel groups + merged convolutions, "IOS-Both"); the headline metric
-    # is the dp_parallel schedule, this one is reported beside it
-    rt.set_option('executor', args.search_executor)
-    t0 = time.time()
-    merged = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel_merge', compute_weight=True,
-                          warmup=2, number=args.search_number, repeat=args.search_repeat)
-    merge_search_s = time.time() - t0
-    graph.sequential_schedule()
-    rt.set_option('executor', args.executor)
-    both, both_out = timed_latency(rt, np, merged, batch, x, args.steps, args.warmup)
-    result['dp_parallel_merge'] = {'latency_ms': both, 'images_per_s': batch / (both['wall'] * 1e-3), 'search_seconds': merge_search_s,
-                                   'num_stages': sum(len(b.stages) for b in merged.blocks),
-                                   'max_abs_diff_to_sequential': float(np.abs(seq_out - both_out).max())}
+        both, both_out = timed_latency(rt, np, merged, batch, x, args.steps, args.warmup)
+        result['dp_parallel_merge'] = {'latency_ms': both, 'images_per_s': batch / (both['wall'] * 1e-3), 'search_seconds': merge_search_s,
+                                       'num_stages': sum(len(b.stages) for b in merged.blocks),
+                                       'max_abs_diff_to_sequential': float(np.abs(seq_out - both_out).max())}
 
     if not args.no_sweep:
         sweep = {}
@@ -301,37 +431,44 @@ def main():
             graph.sequential_schedule()
             rt.set_option('executor', args.executor)
             s_own, out_own = timed_latency(rt, np, optimized_b, b, xb, steps, 3)
-            _, _, roof_b, _ = conv_roofline(rt, graph, b, xb)
+            _, _, kernels_b = launch_profile(rt, graph if s_seq['wall'] < s_own['wall'] else optimized_b, b, xb)
             ops_b = rt.plan_describe(graph, b)
             best = min(s_seq['wall'], s_opt['wall'], s_own['wall'])
+            matrix_ms = sum(k['ms'] for k in kernels_b.values() if k['matrix_flops'] > 0)
+            matrix_flops = sum(k['matrix_flops'] for k in kernels_b.values())
             sweep[str(b)] = {'sequential_ms': s_seq['wall'], 'dp_parallel_batch1_schedule_ms': s_opt['wall'],
                              'dp_parallel_ms': s_own['wall'], 'search_seconds': search_b,
                              'max_abs_diff_between_schedules': float(np.abs(out_seq - out_own).max()),
                              'images_per_s': b / (best * 1e-3),
                              'network_roofline_ms': network_roofline_ms(ops_b, parallel=False),
                              'fraction_of_network_roofline': network_roofline_ms(ops_b, parallel=False) / best,
-                             'conv_tflops': roof_b['achieved'], 'conv_frac_of_fp32_matrix_peak': roof_b['frac']}
+                             'conv_tflops': matrix_flops / (matrix_ms * 1e-3) / 1e12,
+                             'conv_frac_of_fp32_matrix_peak': matrix_flops / (matrix_ms * 1e-3) / 1e12 / PEAK_FP32_MATRIX_TFLOPS,
+                             'roofline': roofline_block(kernels_b, best),
+                             'memory_bound_ops_gbs': memory_bound_ops(rt, graph, b, xb)}
+            rt.set_option('executor', args.executor)
+            if not args.no_cpu:
+                sample = sorted({0, b // 3, b - 1})      # an image's output depends on that image alone
+                sweep[str(b)]['oracle'] = dict(oracle_check(np, out_own[sample], ios_oracle.run(graph, xb[sample])), images_checked=sample)
         result['batch_sweep'] = sweep
-        # reduced-precision mode (bfloat16 operands, fp32 accumulation): not the headline metric, reported beside it
-        rt.set_option('precision', 'bf16')
-        reduced = {}
-        for b in (1, 64):
-            xb = np.random.default_rng(1).standard_normal((b, 3, 299, 299)).astype(np.float32)
-            r_seq, out_b = timed_latency(rt, np, graph, b, xb, max(10, args.steps // (b * 2)), 3)
-            reduced[str(b)] = {'sequential_ms': r_seq['wall'], 'images_per_s': b / (r_seq['wall'] * 1e-3)}
-            if b == 1:
-                reduced[str(b)]['max_abs_diff_to_fp32'] = float(np.abs(out_b - seq_out).max())
-                reduced[str(b)]['fp32_output_scale'] = float(np.abs(seq_out).max())
-        rt.set_option('precision', 'fp32')
-        result['reduced_precision_bf16'] = reduced
+        if not args.no_extras:
+            # reduced-precision mode (bfloat16 operands, fp32 accumulation): not the headline metric, reported beside it
+            rt.set_option('precision', 'bf16')
+            reduced = {}
+            for b in (1, 64):
+                xb = np.random.default_rng(1).standard_normal((b, 3, 299, 299)).astype(np.float32)
+                r_seq, out_b = timed_latency(rt, np, graph, b, xb, max(10, args.steps // (b * 2)), 3)
+                reduced[str(b)] = {'sequential_ms': r_seq['wall'], 'images_per_s': b / (r_seq['wall'] * 1e-3)}
+                if b == 1:
+                    reduced[str(b)]['max_abs_diff_to_fp32'] = float(np.abs(out_b - seq_out).max())
+                    reduced[str(b)]['fp32_output_scale'] = float(np.abs(seq_out).max())
+            rt.set_option('precision', 'fp32')
+            result['reduced_precision_bf16'] = reduced
 
     if not args.no_configs:
         configs = {}
-        for name, make, search in (('sample_net', ios.models.sample_network, True),
-                                   ('squeezenet_1_1', ios.models.squeezenet_1_1, True),
-                                   ('randwire_small', ios.models.randwire_small, False),
-                                   ('nasnet_mobile', ios.models.nasnet_mobile, False)):
-            g = make(init_seed=0, init_scheme='he_normal')
+        for name, search in (('sample_net', True), ('squeezenet_1_1', True), ('randwire_small', False), ('nasnet_mobile', False)):
+            g = make_graph(ios, name)
             xc = np.random.default_rng(1).standard_normal((1, *g.enter_node.output_shape)).astype(np.float32)
             if search or not args.greedy_big:
                 rt.set_option('executor', args.search_executor)
@@ -342,44 +479,52 @@ def main():
                 label = 'dp_parallel'
                 rt.set_option('executor', args.executor)
             else:   # --greedy-big
-                scheduled = make(init_seed=0, init_scheme='he_normal')
+                scheduled = make_graph(ios, name)
                 scheduled.greedy_schedule(4)
                 label = 'greedy'
                 search_c = 0.0
             g.sequential_schedule()
             c_seq, _ = timed_latency(rt, np, g, 1, xc, 100, 10)
-            c_par, _ = timed_latency(rt, np, scheduled, 1, xc, 100, 10)
+            c_par, c_out = timed_latency(rt, np, scheduled, 1, xc, 100, 10)
             ops_c = rt.plan_describe(g, 1)
+            _, launches_c, kernels_c = launch_profile(rt, scheduled, 1, xc)
             configs[name] = {'sequential_ms': c_seq['wall'], f'{label}_ms': c_par['wall'], 'search_seconds': search_c,
-                             'network_roofline_ms': network_roofline_ms(ops_c, parallel=False)}
+                             'initialisation': CONFIG_MODELS[name][1], 'device_operations': len(ops_c), 'launches_per_pass': len(launches_c),
+                             'network_roofline_ms': network_roofline_ms(ops_c, parallel=False),
+                             'fraction_of_network_roofline': network_roofline_ms(ops_c, parallel=False) / c_par['wall'],
+                             'roofline': roofline_block(kernels_c, c_par['wall']),
+                             'memory_bound_ops_gbs': memory_bound_ops(rt, g, 1, xc)}
+            rt.set_option('executor', args.executor)
+            if not args.no_cpu:
+                configs[name]['oracle'] = oracle_check(np, c_out, ios_oracle.run(g, xc))
         result['other_configs_batch1'] = configs
-        # the model variants the reference's own result table uses (its large RandWire / NASNet and SqueezeNet 1.0 with
-        # bypass), sequential and greedy schedules: points of comparison with that table, not part of the metric
-        variants = {}
-        for name, make in (('squeezenet', ios.models.squeezenet), ('randwire_large', ios.models.randwire_large),
-                           ('nasnet_large', ios.models.nasnet_large)):
-            g = make(init_seed=0, init_scheme='he_normal')
-            g.sequential_schedule()
-            scheduled = make(init_seed=0, init_scheme='he_normal')
-            scheduled.greedy_schedule(4)
-            xc = np.random.default_rng(1).standard_normal((1, *g.enter_node.output_shape)).astype(np.float32)
-            v_seq, _ = timed_latency(rt, np, g, 1, xc, 50, 5)
-            v_par, _ = timed_latency(rt, np, scheduled, 1, xc, 50, 5)
-            variants[name] = {'sequential_ms': v_seq['wall'], 'greedy_ms': v_par['wall']}
-            if args.search_variants:
-                rt.set_option('executor', args.search_executor)
-                t0 = time.time()
-                searched = ios.optimize(make(init_seed=0, init_scheme='he_normal'), batch_size=1, opt_type='dp_parallel', compute_weight=True,
-                                        warmup=2, number=6, repeat=3, max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
-                variants[name]['search_seconds'] = time.time() - t0
-                rt.set_option('executor', args.executor)
-                v_dp, _ = timed_latency(rt, np, searched, 1, xc, 50, 5)
-                variants[name]['dp_parallel_ms'] = v_dp['wall']
-        result['reference_table_variants_batch1'] = variants
+        if not args.no_extras:
+            # the model variants the reference's own result table uses (its large RandWire / NASNet and SqueezeNet 1.0 with
+            # bypass), sequential and greedy schedules: points of comparison with that table, not part of the metric
+            variants = {}
+            for name, make in (('squeezenet', ios.models.squeezenet), ('randwire_large', ios.models.randwire_large),
+                               ('nasnet_large', ios.models.nasnet_large)):
+                g = make(init_seed=0, init_scheme='he_normal')
+                g.sequential_schedule()
+                scheduled = make(init_seed=0, init_scheme='he_normal')
+                scheduled.greedy_schedule(4)
+                xc = np.random.default_rng(1).standard_normal((1, *g.enter_node.output_shape)).astype(np.float32)
+                v_seq, _ = timed_latency(rt, np, g, 1, xc, 50, 5)
+                v_par, _ = timed_latency(rt, np, scheduled, 1, xc, 50, 5)
+                variants[name] = {'sequential_ms': v_seq['wall'], 'greedy_ms': v_par['wall']}
+                if args.search_variants:
+                    rt.set_option('executor', args.search_executor)
+                    t0 = time.time()
+                    searched = ios.optimize(make(init_seed=0, init_scheme='he_normal'), batch_size=1, opt_type='dp_parallel', compute_weight=True,
+                                            warmup=2, number=6, repeat=3, max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
+                    variants[name]['search_seconds'] = time.time() - t0
+                    rt.set_option('executor', args.executor)
+                    v_dp, _ = timed_latency(rt, np, searched, 1, xc, 50, 5)
+                    variants[name]['dp_parallel_ms'] = v_dp['wall']
+            result['reference_table_variants_batch1'] = variants
 
     if not args.no_cpu:
         import torch
-        from oracle import ios_oracle
         threads = torch.get_num_threads()
         config, weights = graph.export_config(), ios_oracle.graph_weights(graph)
         ios_oracle.run_graph(config, weights, x)
@@ -388,11 +533,11 @@ def main():
             cpu_out = ios_oracle.run_graph(config, weights, x)
             runs += 1
         cpu_ms = (time.perf_counter() - t) / runs * 1e3
-        err = np.abs(opt_out - cpu_out)
         result['cpu_baseline'] = {'value': batch / (cpu_ms * 1e-3), 'unit': 'images/s', 'cores': threads, 'kind': 'port',
                                   'sample': f'{runs} forward passes of the same graph, weights and input on the CPU oracle '
                                             f'(torch-CPU fp32, {threads} threads), {cpu_ms:.1f} ms each'}
-        result['matches_cpu_oracle'] = bool((err <= 1e-4 + 1e-3 * np.abs(cpu_out)).all())
+        result['oracle'] = oracle_check(np, opt_out, cpu_out)
+        result['matches_cpu_oracle'] = result['oracle']['matches_cpu_oracle']
     print(json.dumps(result))
 
 

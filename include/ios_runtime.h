@@ -122,6 +122,13 @@ int ios_session_describe(ios_session *session, char *buf, int cap);         /* l
 /* ms[num_ops]: mean HIP-event time of each device operation launched `repeat` times back to back on one stream. */
 int ios_session_profile_ops(ios_session *session, int warmup, int repeat, float *ms);
 
+/* The kernel launches of one forward pass as the executor in force issues them (one per level of a multi-group stage
+ * under the fused executors), in issue order, as a JSON array into buf: kernel name, stage, blocks, threads, the
+ * operations behind it and their algorithmic flops and bytes.  Returns the length like ios_plan_describe. */
+int ios_session_describe_launches(ios_session *session, char *buf, int cap);
+/* ms[i] (capacity entries available): mean HIP-event time of launch i issued `repeat` times back to back on the launch stream. */
+int ios_session_profile_launches(ios_session *session, int warmup, int repeat, float *ms, int capacity);
+
 #ifdef __cplusplus
 }
 #endif

@@ -253,4 +253,21 @@ int ios_session_profile_ops(ios_session *s, int warmup, int repeat, float *ms) {
     });
 }
 
+int ios_session_describe_launches(ios_session *s, char *buf, int cap) {
+    int needed = -1;
+    guarded([&]() {
+        const std::string text = unbox(s).describe_launches();
+        needed = (int)text.size();
+        if (buf != nullptr && cap > needed) memcpy(buf, text.c_str(), text.size() + 1);
+    });
+    return needed;
+}
+
+int ios_session_profile_launches(ios_session *s, int warmup, int repeat, float *ms, int capacity) {
+    return guarded([&]() {
+        if (ms == nullptr) throw std::runtime_error("output pointer is null");
+        unbox(s).profile_launches(warmup, repeat, ms, capacity);
+    });
+}
+
 }  // extern "C"

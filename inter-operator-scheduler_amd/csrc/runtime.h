@@ -124,6 +124,20 @@ public:
     // reference timing protocol for stage probes: `number` back-to-back passes in one bracket
     void measure_back_to_back(int warmup, int number, int repeat, float *results);
     void profile_ops(int warmup, int repeat, float *ms);
+    // The kernel launches of one forward pass as the executor in force issues them (fused executors: one launch per
+    // level of a multi-group stage, stand-alone kernels for single-group stages; stream executors: one per operation),
+    // in issue order.
+    struct LaunchRecord {
+        int stage = 0;
+        std::string kernel;      // e.g. "fused_kernel<512>", "conv_kernel<wq_m32n16_w8_t16>", "pool_kernel"
+        std::vector<int> ops;    // indices into plan().ops
+        int blocks = 0, threads = 0;
+        int fused_level = -1;    // index into the stage's fused launches, -1 for a stand-alone kernel
+    };
+    std::vector<LaunchRecord> launches();
+    std::string describe_launches();   // JSON array with the algorithmic flops and bytes of every launch
+    // ms[i]: mean HIP-event time of launch i issued `repeat` times back to back on the launch stream
+    void profile_launches(int warmup, int repeat, float *ms, int capacity);
 
 private:
     void setup();
@@ -152,6 +166,7 @@ private:
     struct FusedLaunch {
         int threads, first_item, num_items, total_blocks, smem_bytes;
         FusedHeader header;
+        std::vector<int> ops;   // plan operations behind the items (a two-kernel split-K reduction names its convolution)
     };
     std::vector<std::vector<FusedLaunch>> fused_stages_;   // per stage; empty for single-group stages
     void *fused_items_ = nullptr;                          // device copy of all work items

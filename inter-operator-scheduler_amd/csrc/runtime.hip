@@ -618,6 +618,7 @@ void Session::build_fused() {
         WorkItem item;
         int threads;     // 0: any block size
         int smem_bytes;
+        int op;          // plan operation behind the item
     };
     for (size_t s = 0; s < plan_.stages.size(); s++) {
         const auto &groups = plan_.stages[s];
@@ -630,6 +631,7 @@ void Session::build_fused() {
                 memset(&pend.item, 0, sizeof(WorkItem));
                 pend.threads = 0;
                 pend.smem_bytes = 0;
+                pend.op = index;
                 int blocks = 0;
                 switch (op.kind) {
                     case OpKind::ConvMfma: {
@@ -656,6 +658,7 @@ void Session::build_fused() {
                             red.item.reduce = d.reduce;
                             red.threads = 0;
                             red.smem_bytes = 0;
+                            red.op = index;
                             chains[g].push_back(red);
                         }
                         continue;
@@ -709,8 +712,9 @@ void Session::build_fused() {
             widest = std::max(widest, 256);   // narrowest instantiation of the fused kernel
             // one launch per level, as wide as its widest convolution body
             if (here.size() > (size_t)kMaxFusedItems) throw std::runtime_error("fused launch: too many groups in a stage");
-            FusedLaunch launch{widest, (int)items.size(), 0, 0, 0, {}};
+            FusedLaunch launch{widest, (int)items.size(), 0, 0, 0, {}, {}};
             for (Pending *pend : here) {
+                launch.ops.push_back(pend->op);
                 WorkItem item = pend->item;
                 item.threads = pend->threads == 0 ? widest : pend->threads;
                 if (pend->threads == 0) item.num_blocks = std::max(1, (item.num_blocks * 256 + widest - 1) / widest);
@@ -866,6 +870,108 @@ void Session::profile_ops(int warmup, int repeat, float *ms_out) {
         IOS_HIP(hipStreamSynchronize(main));
         IOS_HIP(hipEventRecord(start_, main));
         for (int r = 0; r < repeat; r++) launch_op(op, main);
+        IOS_HIP(hipEventRecord(stop_, main));
+        IOS_HIP(hipEventSynchronize(stop_));
+        float ms = 0.f;
+        IOS_HIP(hipEventElapsedTime(&ms, start_, stop_));
+        ms_out[i] = ms / (float)repeat;
+    }
+}
+
+// ---- per-launch view of a pass -------------------------------------------------------------------------------------------
+static std::string op_kernel_name(const Plan &plan, const PlanOp &op) {
+    switch (op.kind) {
+        case OpKind::ConvMfma: return std::string("conv_kernel<") + conv_variant(plan.convs[op.conv].launch.variant).name + ">";
+        case OpKind::ConvDepthwise: return "dwconv_kernel";
+        case OpKind::ConvDirect: return "conv_direct_kernel";
+        case OpKind::Pool: return "pool_kernel";
+        case OpKind::GlobalPool: return "global_pool_kernel";
+        case OpKind::Nary:
+        case OpKind::Unary: return "nary_kernel";
+    }
+    return "?";
+}
+
+std::vector<Session::LaunchRecord> Session::launches() {
+    const ExecMode mode = ctx_.exec_mode();
+    const bool fused = !static_ && (mode == ExecMode::Fused || mode == ExecMode::FusedGraph);
+    if (fused) build_fused();
+    std::vector<LaunchRecord> out;
+    for (size_t s = 0; s < plan_.stages.size(); s++) {
+        const auto &groups = plan_.stages[s];
+        if (fused && groups.size() > 1) {
+            for (size_t l = 0; l < fused_stages_[s].size(); l++) {
+                const FusedLaunch &f = fused_stages_[s][l];
+                LaunchRecord r;
+                r.stage = (int)s;
+                r.kernel = "fused_kernel<" + std::to_string(f.threads) + ">";
+                r.ops = f.ops;
+                r.blocks = f.total_blocks;
+                r.threads = f.threads;
+                r.fused_level = (int)l;
+                out.push_back(r);
+            }
+            continue;
+        }
+        for (const auto &group : groups)
+            for (int index : group) {
+                LaunchRecord r;
+                r.stage = (int)s;
+                r.kernel = op_kernel_name(plan_, plan_.ops[index]);
+                r.ops = {index};
+                out.push_back(r);
+            }
+    }
+    return out;
+}
+
+std::string Session::describe_launches() {
+    std::ostringstream os;
+    os << '[';
+    bool first = true;
+    for (const LaunchRecord &r : launches()) {
+        double flops = 0.0, bytes = 0.0, conv_flops = 0.0;
+        std::vector<int> seen;
+        for (int index : r.ops) {
+            if (std::find(seen.begin(), seen.end(), index) != seen.end()) continue;
+            seen.push_back(index);
+            flops += plan_.ops[index].flops;
+            bytes += plan_.ops[index].bytes;
+            if (plan_.ops[index].kind == OpKind::ConvMfma) conv_flops += plan_.ops[index].flops;
+        }
+        os << (first ? "" : ",") << "{\"stage\":" << r.stage << ",\"kernel\":\"" << r.kernel << "\",\"fused_level\":" << r.fused_level
+           << ",\"blocks\":" << r.blocks << ",\"threads\":" << r.threads << ",\"flops\":" << flops << ",\"matrix_flops\":" << conv_flops
+           << ",\"bytes\":" << bytes << ",\"ops\":[";
+        for (size_t i = 0; i < seen.size(); i++) os << (i ? "," : "") << seen[i];
+        os << "]}";
+        first = false;
+    }
+    os << ']';
+    return os.str();
+}
+
+void Session::profile_launches(int warmup, int repeat, float *ms_out, int capacity) {
+    if (static_) throw std::runtime_error("a session in the static scratch has no timers");
+    if (repeat < 1 || warmup < 0) throw std::runtime_error("profile_launches: warmup >= 0 and repeat >= 1 required");
+    const std::vector<LaunchRecord> list = launches();
+    if ((int)list.size() > capacity) throw std::runtime_error("profile_launches: output array too small");
+    hipStream_t main = ctx_.stream(0);
+    run();   // every launch sees the inputs it has in a real pass
+    const WorkItem *items = static_cast<const WorkItem *>(fused_items_);
+    for (size_t i = 0; i < list.size(); i++) {
+        const LaunchRecord &r = list[i];
+        auto issue = [&]() {
+            if (r.fused_level >= 0) {
+                const FusedLaunch &l = fused_stages_[r.stage][r.fused_level];
+                launch_fused(l.threads, items + l.first_item, l.header, l.total_blocks, l.smem_bytes, main);
+            } else {
+                launch_op(plan_.ops[r.ops[0]], main);
+            }
+        };
+        for (int w = 0; w < warmup; w++) issue();
+        IOS_HIP(hipStreamSynchronize(main));
+        IOS_HIP(hipEventRecord(start_, main));
+        for (int k = 0; k < repeat; k++) issue();
         IOS_HIP(hipEventRecord(stop_, main));
         IOS_HIP(hipEventSynchronize(stop_));
         float ms = 0.f;

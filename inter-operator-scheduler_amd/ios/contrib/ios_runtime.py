@@ -75,9 +75,12 @@ def _declare(handle):
     handle.ios_session_num_ops.argtypes = [vp]
     handle.ios_session_describe.argtypes = [vp, ctypes.c_char_p, i]
     handle.ios_session_profile_ops.argtypes = [vp, i, i, f32p]
+    handle.ios_session_describe_launches.argtypes = [vp, ctypes.c_char_p, i]
+    handle.ios_session_profile_launches.argtypes = [vp, i, i, f32p, i]
     for name in ('ios_session_set_conv_weights', 'ios_session_set_input', 'ios_session_run',
                  'ios_session_get_output', 'ios_session_get_tensor', 'ios_session_measure',
-                 'ios_session_num_ops', 'ios_session_describe', 'ios_session_profile_ops'):
+                 'ios_session_num_ops', 'ios_session_describe', 'ios_session_profile_ops',
+                 'ios_session_describe_launches', 'ios_session_profile_launches'):
         getattr(handle, name).restype = i
     return handle
 
@@ -319,6 +322,26 @@ class Session:
             if need < cap:
                 return json.loads(buf.value.decode())
             cap = need + 1
+
+    def launches(self) -> List[dict]:
+        """The kernel launches of one pass under the executor in force: kernel name, stage, operations, flops, bytes."""
+        cap = 1 << 16
+        while True:
+            buf = ctypes.create_string_buffer(cap)
+            need = self._lib.ios_session_describe_launches(self._handle, buf, c_int(cap))
+            if need < 0:
+                _check(1, 'ios_session_describe_launches')
+            if need < cap:
+                return json.loads(buf.value.decode())
+            cap = need + 1
+
+    def profile_launches(self, warmup=2, repeat=10) -> List[float]:
+        """Mean milliseconds of every launch of the pass (see ``launches``) issued back to back, HIP-event timed."""
+        n = len(self.launches())
+        out = c_float_array(max(1, n))
+        _check(self._lib.ios_session_profile_launches(self._handle, c_int(warmup), c_int(repeat), out, c_int(n)),
+               'ios_session_profile_launches')
+        return [float(v) for v in out][:n]
 
     def profile_ops(self, warmup=2, repeat=10) -> List[float]:
         """Mean milliseconds of every device operation run alone on one stream, HIP-event timed."""
