@@ -71,8 +71,7 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fus
             break;
         }
         case WORK_DWCONV: {
-            const DirectConvArgs a = item.direct;
-            dwconv_dispatch(a, local, num_blocks);
+            dwconv_dispatch(item.direct, local, num_blocks);   // (the table of summed inputs is read in place)
             break;
         }
         case WORK_CONV_DIRECT: {

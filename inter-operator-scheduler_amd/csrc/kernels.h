@@ -14,6 +14,8 @@ namespace ios {
 
 enum Act : int { ACT_NONE = 0, ACT_RELU = 1, ACT_TANH = 2, ACT_SIGMOID = 3 };
 
+constexpr int kMaxNaryInputs = 8;   // views one launch adds (or multiplies)
+
 struct TensorView {
     float *ptr = nullptr;  // element (0, 0, 0, 0)
     int C = 0, H = 0, W = 0;
@@ -91,9 +93,11 @@ void launch_pack_filters(const ConvProblem &p, const ConvLaunch &l, const float 
 void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
                       const float *bias, const TensorView &y, float *workspace, unsigned *counters, hipStream_t stream);
 
-// Depth-wise convolution (groups == IC == OC), filters in their original [C][1][KH][KW] layout.
+// Depth-wise convolution (groups == IC == OC), filters in their original [C][1][KH][KW] layout.  With `more`, the input is
+// x + more[0] + ... + more[nmore - 1] (at most kMaxNaryInputs views in all, added left to right before the folded ReLU).
 void launch_dwconv(const ConvProblem &p, const TensorView &x, const float *w, const float *bias,
-                   const TensorView &y, hipStream_t stream);
+                   const TensorView &y, hipStream_t stream, const TensorView *more = nullptr, int nmore = 0);
+bool dwconv_sums_inputs(const ConvProblem &p);   // the kernel for this window can add further inputs in its loader (3 x 3, 5 x 5)
 
 // Direct convolution for any geometry (one thread per output element); used for grouped convolutions
 // whose groups are too thin for the matrix path.
@@ -110,7 +114,6 @@ void launch_pool(const PoolProblem &p, const TensorView &x, const TensorView &y,
 void launch_global_pool(const PoolProblem &p, const TensorView &x, const TensorView &y, hipStream_t stream);
 
 // ---- element-wise -----------------------------------------------------------------------------------
-constexpr int kMaxNaryInputs = 8;
 struct NaryArgs {
     const float *src[kMaxNaryInputs];
     long long src_bstride[kMaxNaryInputs];

@@ -48,6 +48,11 @@ struct PNode {
     int parent = -1, parent_begin = 0;
     bool pre_relu_alias = false;   // elided ReLU: consumers must apply max(x, 0) themselves
     int fused_into = -1;           // concat (identity) node whose buffer holds this node's output
+    bool no_storage = false;       // ReLU whose inputs the consumer reads itself: never materialised
+    // depth-wise convolution that adds the values of a sum in its loader: the node whose single term
+    // holds them (the convolution itself, or the private ReLU in front of it, which is then applied after the sum)
+    int sum_front = -1;
+    bool sum_relu = false;
     int references = 0;            // number of input values that name this node
 };
 
@@ -301,6 +306,7 @@ private:
                 }
             }
         }
+        find_depthwise_sums();
         for (PNode &n : nodes_) {
             if (n.type == NodeType::Identity && single_value(n)) {
                 n.parent = n.inputs[0][0].node;
@@ -328,7 +334,57 @@ private:
             }
         }
         for (PNode &n : nodes_)
-            if (n.parent < 0) n.own = true;
+            if (n.parent < 0 && !n.no_storage) n.own = true;
+    }
+
+    ConvProblem problem_of(const PNode &n) const {
+        int C, H, W;
+        input_shape(n, C, H, W);
+        const Json &cfg = *n.cfg;
+        ConvProblem p;
+        p.B = batch_;
+        p.IC = C; p.H = H; p.W = W;
+        p.OC = n.C; p.OH = n.H; p.OW = n.W;
+        p.KH = cfg["kernel"][0].as_int(); p.KW = cfg["kernel"][1].as_int();
+        p.sh = cfg["stride"][0].as_int(); p.sw = cfg["stride"][1].as_int();
+        p.ph = cfg["padding"][0].as_int(); p.pw = cfg["padding"][1].as_int();
+        p.groups = cfg["groups"].as_int();
+        p.act = act_code(cfg["act"].as_string());
+        p.pre_relu = 0;
+        return p;
+    }
+
+    // Sequential children [(ReLU,) depth-wise K x K convolution, ...] whose input is one term that sums k > 1 values, read by
+    // nobody else: the depth-wise kernel adds the k values (and applies the ReLU) in its loader, so the summing launch and its
+    // output tensor disappear (the reference adds them with a kernel of its own, src/ios/ios_runtime.cu:1047-1057).
+    void find_depthwise_sums() {
+        for (const auto &seq : sequentials_) {
+            for (int i = seq.first; i <= seq.second; i++) {
+                PNode &dw = nodes_[i];
+                if (dw.type != NodeType::Conv) continue;
+                const ConvProblem pd = problem_of(dw);
+                if (!pd.is_depthwise() || !dwconv_sums_inputs(pd)) continue;
+                int front = i;   // node whose inputs are the sources
+                bool relu = false;
+                if (single_value(dw) && i > seq.first && dw.inputs[0][0].node == i - 1) {
+                    const PNode &r = nodes_[i - 1];
+                    const bool whole = dw.inputs[0][0].begin == 0 && dw.inputs[0][0].end == r.C;
+                    if (r.type == NodeType::Relu && r.references == 1 && whole && r.inputs.size() == 1) {
+                        front = i - 1;
+                        relu = true;
+                    }
+                }
+                const PNode &f = nodes_[front];
+                if (f.inputs.size() != 1 || f.inputs[0].size() < 2 || f.inputs[0].size() > (size_t)kMaxNaryInputs) continue;
+                dw.sum_front = front;
+                dw.sum_relu = relu;
+                if (front != i) {
+                    PNode &r = nodes_[front];
+                    r.no_storage = true;   // the convolution reads the ReLU's inputs itself
+                    r.parent = -1;
+                }
+            }
+        }
     }
 
     int resolve_sequential(int index) const {
@@ -436,6 +492,7 @@ private:
     void emit(int index) {
         PNode &n = nodes_[index];
         if (n.type == NodeType::Placeholder || n.type == NodeType::Sequential) return;
+        if (n.no_storage) return;   // ReLU in front of a depth-wise convolution that reads the summed inputs itself
         int C, H, W;
         input_shape(n, C, H, W);
         const Json &cfg = *n.cfg;
@@ -469,24 +526,31 @@ private:
         }
     }
 
-    void emit_conv(PNode &n, const Json &cfg, int C, int H, int W, int index) {
-        bool pre_relu = false;
-        const ViewRef in = input_view(n, C, H, W, &pre_relu);
+    int add_plan_conv(const PNode &n, const ConvProblem &p) {
         PlanConv conv;
         conv.name = n.name;
-        ConvProblem &p = conv.problem;
-        p.B = batch_;
-        p.IC = C; p.H = H; p.W = W;
-        p.OC = n.C; p.OH = n.H; p.OW = n.W;
-        p.KH = cfg["kernel"][0].as_int(); p.KW = cfg["kernel"][1].as_int();
-        p.sh = cfg["stride"][0].as_int(); p.sw = cfg["stride"][1].as_int();
-        p.ph = cfg["padding"][0].as_int(); p.pw = cfg["padding"][1].as_int();
-        p.groups = cfg["groups"].as_int();
-        p.act = act_code(cfg["act"].as_string());
-        p.pre_relu = pre_relu ? 1 : 0;
+        conv.problem = p;
         conv.weight_off = reserve((size_t)p.OC * p.K());
         conv.bias_off = reserve((size_t)p.OC);
+        if (plan_.conv_index.count(n.name)) throw std::runtime_error("duplicate convolution name '" + n.name + "'");
+        plan_.conv_index[n.name] = static_cast<int>(plan_.convs.size());
+        plan_.convs.push_back(conv);
+        return static_cast<int>(plan_.convs.size()) - 1;
+    }
+
+    void emit_conv(PNode &n, const Json &cfg, int C, int H, int W, int index) {
+        (void)cfg;
+        bool pre_relu = false;
+        std::vector<ViewRef> sum_srcs;
+        if (n.sum_front >= 0) {
+            for (const Val &v : nodes_[n.sum_front].inputs[0]) sum_srcs.push_back(view_of(v.node).window(v.begin, v.end));
+            pre_relu = n.sum_relu;
+        }
+        const ViewRef in = n.sum_front >= 0 ? sum_srcs[0] : input_view(n, C, H, W, &pre_relu);
+        ConvProblem p = problem_of(n);
+        p.pre_relu = pre_relu ? 1 : 0;
         OpKind kind;
+        bool matrix_path = false;
         if (p.is_depthwise()) {
             kind = OpKind::ConvDepthwise;
         } else if ((p.groups > 1 && (p.ICg() < 4 || p.OCg() < 8)) || !conv_matrix_path_supported(p) ||
@@ -495,18 +559,19 @@ private:
             kind = OpKind::ConvDirect;
         } else {
             kind = OpKind::ConvMfma;
-            conv.matrix_path = true;
+            matrix_path = true;
             // the kernel configuration depends on how many groups share the stage: chosen in finish()
         }
-        if (plan_.conv_index.count(n.name)) throw std::runtime_error("duplicate convolution name '" + n.name + "'");
-        plan_.conv_index[n.name] = static_cast<int>(plan_.convs.size());
-        plan_.convs.push_back(conv);
+        const int conv = add_plan_conv(n, p);
+        plan_.convs[conv].matrix_path = matrix_path;
         PlanOp &op = push(kind, n);
         op.in = in;
         op.out = view_of(index);
-        op.conv = static_cast<int>(plan_.convs.size()) - 1;
-        op.flops = p.flops();
-        op.bytes = 4.0 * ((double)batch_ * C * H * W + (double)p.OC * p.K() + p.OC + (double)batch_ * p.OC * p.OH * p.OW);
+        op.conv = conv;
+        op.srcs = sum_srcs;
+        const double k = sum_srcs.empty() ? 1.0 : (double)sum_srcs.size();
+        op.flops = p.flops() + (k - 1.0) * (double)batch_ * C * H * W;
+        op.bytes = 4.0 * (k * (double)batch_ * C * H * W + (double)p.OC * p.K() + p.OC + (double)batch_ * p.OC * p.OH * p.OW);
     }
 
     void emit_pool(PNode &n, const Json &cfg, int C, int H, int W, int index) {
@@ -590,7 +655,7 @@ private:
     void finish() {
         for (size_t i = 0; i < nodes_.size(); i++) {
             const PNode &n = nodes_[i];
-            if (n.pre_relu_alias) continue;   // never materialised
+            if (n.pre_relu_alias || n.no_storage) continue;   // never materialised
             plan_.tensors[n.name] = view_of(static_cast<int>(i));
         }
         plan_.input = view_of(0);
@@ -677,6 +742,7 @@ std::string describe_plan(const Plan &plan) {
             }
         }
         if (op.kind == OpKind::Nary) os << ",\"inputs\":" << op.srcs.size() << ",\"accumulate\":" << op.accumulate;
+        if (op.kind == OpKind::ConvDepthwise) os << ",\"inputs\":" << (op.srcs.empty() ? 1 : op.srcs.size());
         if (op.kind == OpKind::Nary || op.kind == OpKind::Unary) os << ",\"act\":" << op.act;
         os << '}';
     }

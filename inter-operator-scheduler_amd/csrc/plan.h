@@ -60,7 +60,7 @@ struct PlanOp {
     ViewRef in, out;
     int conv = -1;        // index into Plan::convs
     PoolProblem pool{};
-    std::vector<ViewRef> srcs;   // Nary
+    std::vector<ViewRef> srcs;   // Nary: inputs; ConvDepthwise of a sum: the views it adds in its loader (else empty)
     int multiply = 0, accumulate = 0, act = 0;
     double flops = 0.0, bytes = 0.0;
 };

@@ -10,7 +10,7 @@ namespace ios {
 
 __global__ void pool_kernel(PoolArgs a) { pool_body(a, blockIdx.x, gridDim.x); }
 __global__ void global_pool_kernel(PoolArgs a) { global_pool_body(a, blockIdx.x, gridDim.x); }
-__global__ void dwconv_kernel(DirectConvArgs a) { dwconv_dispatch(a, blockIdx.x, gridDim.x); }
+__global__ void dwconv_kernel(DirectConvArgs a) { dwconv_dispatch<true>(a, blockIdx.x, gridDim.x); }
 __global__ void conv_direct_kernel(DirectConvArgs a) { conv_direct_body(a, blockIdx.x, gridDim.x); }
 __global__ void nary_kernel(NaryKernelArgs a) { nary_dispatch(a, blockIdx.x, gridDim.x); }
 
@@ -61,8 +61,31 @@ DirectConvArgs make_direct_conv_args(const ConvProblem &p, const TensorView &x, 
     a.p = p;
     const unsigned long long x_bytes = ((unsigned long long)(p.B - 1) * x.bstride + (unsigned long long)p.IC * p.H * p.W) * 4ull;
     a.x_bytes = x_bytes < (1ull << 31) ? (unsigned)x_bytes : 0u;
+    a.nmore = 0;
+    for (int s = 0; s < kMaxNaryInputs - 1; s++) {
+        a.more[s] = x.ptr;
+        a.more_bs[s] = x.bstride;
+        a.more_bytes[s] = 0;
+    }
     *blocks = blocks_for((long long)p.B * p.OC * p.OH * p.OW, 256, 8192);
     return a;
+}
+
+bool dwconv_sums_inputs(const ConvProblem &p) { return p.is_depthwise() && p.KH == p.KW && (p.KH == 3 || p.KH == 5); }
+
+void add_dwconv_sources(DirectConvArgs &a, const TensorView *more, int count) {
+    if (count < 0 || count > kMaxNaryInputs - 1) throw std::runtime_error("dwconv: too many summed inputs");
+    const ConvProblem &p = a.p;
+    if (count > 0 && !dwconv_sums_inputs(p)) throw std::runtime_error("dwconv: this window does not add inputs in its loader");
+    for (int s = 0; s < count; s++) {
+        if (more[s].C != p.IC || more[s].H != p.H || more[s].W != p.W) throw std::runtime_error("dwconv: summed inputs of different shapes");
+        const unsigned long long bytes = ((unsigned long long)(p.B - 1) * more[s].bstride + (unsigned long long)p.IC * p.H * p.W) * 4ull;
+        if (bytes >= (1ull << 31) || a.x_bytes == 0) throw std::runtime_error("dwconv: summed inputs beyond 31-bit offsets");
+        a.more[s] = more[s].ptr;
+        a.more_bs[s] = more[s].bstride;
+        a.more_bytes[s] = (unsigned)bytes;
+    }
+    a.nmore = count;
 }
 
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -101,10 +124,11 @@ void launch_global_pool(const PoolProblem &p, const TensorView &x, const TensorV
 }
 
 void launch_dwconv(const ConvProblem &p, const TensorView &x, const float *w, const float *bias, const TensorView &y,
-                   hipStream_t stream) {
+                   hipStream_t stream, const TensorView *more, int nmore) {
     if (!p.is_depthwise()) throw std::runtime_error("dwconv: not a depth-wise problem");
     int blocks;
-    const DirectConvArgs a = make_direct_conv_args(p, x, w, bias, y, &blocks);
+    DirectConvArgs a = make_direct_conv_args(p, x, w, bias, y, &blocks);
+    add_dwconv_sources(a, more, nmore);
     hipLaunchKernelGGL(dwconv_kernel, dim3(blocks), dim3(256), 0, stream, a);
 }
 

@@ -157,6 +157,12 @@ struct DirectConvArgs {
     long long x_bs, y_bs;
     ConvProblem p;
     unsigned x_bytes;   // extent of the input view in bytes when it is below 2^31 (branch-free depth-wise loads), else 0
+    // depth-wise convolution of a sum: the input is x + more[0] + ... + more[nmore - 1] (added left to right, then the
+    // folded ReLU), every view of the shape of x; the reference adds them with a kernel of its own (src/ios/ops.cu:26-48)
+    const float *more[kMaxNaryInputs - 1];
+    long long more_bs[kMaxNaryInputs - 1];
+    unsigned more_bytes[kMaxNaryInputs - 1];
+    int nmore;
 };
 
 // raw buffer loads as in the matrix-path convolution: an offset with the top bit set is out of range and reads zero
@@ -164,7 +170,8 @@ __device__ __forceinline__ float pw_buffer_load(__amdgpu_buffer_rsrc_t r, unsign
     return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_offset, 0, 0));
 }
 
-template <int KH, int KW>
+// SUM: the instantiation that adds further inputs in its loader (kept apart so that the common single-input form stays small)
+template <int KH, int KW, bool SUM = false>
 __device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, int num_blocks) {
     const ConvProblem &p = a.p;
     const int kh_n = KH > 0 ? KH : p.KH, kw_n = KW > 0 ? KW : p.KW;
@@ -197,6 +204,39 @@ __device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, 
                     v[i2 * KW + j] = pw_buffer_load(xr, (base + (unsigned)(i2 * p.W + j) * 4u) | kill);
                 }
             }
+            // further inputs of the sum (windows up to 5 x 5; the host refuses larger ones): two at a time for 3 x 3 windows,
+            // where a missing second one has extent zero and reads zeros, one at a time for 5 x 5
+            if constexpr (SUM && KH * KW <= 25) {
+                constexpr int PAIR = KH * KW <= 9 ? 2 : 1;
+                // unrolled with wavefront-uniform guards: indexing the argument arrays with a loop variable would move them to scratch memory
+#pragma unroll
+                for (int s = 0; s < kMaxNaryInputs - 1; s += PAIR) {
+                    if (s >= a.nmore) break;
+                    float u[PAIR][KH > 0 ? KH * KW : 1];
+#pragma unroll
+                    for (int e = 0; e < PAIR; e++) {
+                        constexpr int kLast = kMaxNaryInputs - 2;
+                        const int se = s + e < kLast ? s + e : kLast;
+                        const __amdgpu_buffer_rsrc_t sr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a.more[se]), 0,
+                                                                                             s + e < a.nmore ? a.more_bytes[se] : 0u, 0x00020000);
+                        const unsigned sbase = (unsigned)(((long long)b * a.more_bs[se] + (long long)c * p.H * p.W + (long long)h0 * p.W + w0) * 4);
+#pragma unroll
+                        for (int i2 = 0; i2 < KH; i2++) {
+                            const unsigned row_kill = (unsigned)(h0 + i2) < (unsigned)p.H ? 0u : 0x80000000u;
+#pragma unroll
+                            for (int j = 0; j < KW; j++) {
+                                const unsigned kill = (unsigned)(w0 + j) < (unsigned)p.W ? row_kill : 0x80000000u;
+                                u[e][i2 * KW + j] = pw_buffer_load(sr, (sbase + (unsigned)(i2 * p.W + j) * 4u) | kill);
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int t = 0; t < KH * KW; t++) {
+                        v[t] += u[0][t];
+                        if (PAIR > 1 && s + 1 < a.nmore) v[t] += u[PAIR - 1][t];   // wavefront-uniform; skipping keeps -0.0 + 0.0 out of the sum
+                    }
+                }
+            }
 #pragma unroll
             for (int t = 0; t < KH * KW; t++) acc = fmaf(__int_as_float(max(__float_as_int(v[t]), relu_floor)), wc[t], acc);
         } else {
@@ -217,8 +257,18 @@ __device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, 
     }
 }
 
+// WITH_SUM: the caller may hold launches that add further inputs in the loader (their 5 x 5 form needs more registers than
+// the fused stage kernel of the matrix-path convolutions grants, so that kernel is built without them)
+template <bool WITH_SUM = true>
 __device__ __forceinline__ void dwconv_dispatch(const DirectConvArgs &a, int block, int num_blocks) {
     const ConvProblem &p = a.p;
+    if (a.nmore > 0) {   // the host only builds such launches for 3 x 3 and 5 x 5 windows
+        if constexpr (WITH_SUM) {
+            if (p.KH == 3) dwconv_body<3, 3, true>(a, block, num_blocks);
+            else dwconv_body<5, 5, true>(a, block, num_blocks);
+        }
+        return;
+    }
     if (p.KH == 3 && p.KW == 3) dwconv_body<3, 3>(a, block, num_blocks);
     else if (p.KH == 5 && p.KW == 5) dwconv_body<5, 5>(a, block, num_blocks);
     else if (p.KH == 7 && p.KW == 7) dwconv_body<7, 7>(a, block, num_blocks);

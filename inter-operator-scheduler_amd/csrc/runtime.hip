@@ -543,7 +543,10 @@ void Session::launch_op(const PlanOp &op, hipStream_t stream) {
         }
         case OpKind::ConvDepthwise: {
             const PlanConv &c = plan_.convs[op.conv];
-            launch_dwconv(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), stream);
+            TensorView more[kMaxNaryInputs];
+            for (size_t i = 1; i < op.srcs.size(); i++) more[i - 1] = tv(op.srcs[i]);
+            launch_dwconv(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), stream, more,
+                          op.srcs.empty() ? 0 : (int)op.srcs.size() - 1);
             break;
         }
         case OpKind::ConvDirect: {
@@ -668,6 +671,11 @@ void Session::build_fused() {
                         const PlanConv &c = plan_.convs[op.conv];
                         pend.item.kind = op.kind == OpKind::ConvDepthwise ? WORK_DWCONV : WORK_CONV_DIRECT;
                         pend.item.direct = make_direct_conv_args(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), &blocks);
+                        if (op.kind == OpKind::ConvDepthwise && op.srcs.size() > 1) {
+                            TensorView more[kMaxNaryInputs];
+                            for (size_t i = 1; i < op.srcs.size(); i++) more[i - 1] = tv(op.srcs[i]);
+                            add_dwconv_sources(pend.item.direct, more, (int)op.srcs.size() - 1);
+                        }
                         break;
                     }
                     case OpKind::Pool:

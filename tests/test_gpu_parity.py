@@ -300,6 +300,70 @@ def test_sequential_units_and_folded_relu():
         assert_close(got, want, 'sequential units')
 
 
+def separable_graph(in_shape, inputs, relu, oc, window, stride):
+    """`inputs` 1x1 convolutions of the placeholder feed one (ReLU,) depth-wise, 1x1 unit whose output sits in a concat."""
+    def build(b, v):
+        parts = [ios.conv2d(b, [[v]], in_shape[0], (1, 1), act='identity') for _ in range(inputs)]
+        pad = (window // 2, window // 2)
+        make = ios.relu_sep_conv if relu else ios.sep_conv
+        unit = make(b, [parts], oc, (window, window), (stride, stride), pad)
+        other = ios.conv2d(b, [[unit]], 6, (1, 1))
+        ios.identity(b, [[other], [unit]], is_exit=True)      # the unit writes into a channel window of this buffer
+    return single_op_graph(in_shape, build)
+
+
+def test_depthwise_kernel_adds_up_to_eight_inputs_in_its_loader():
+    """(sum of k values,) (ReLU,) depth-wise convolution: no summing launch, no sum tensor (3 x 3 and 5 x 5 windows)."""
+    for in_shape, inputs, relu, oc, window, stride, batch in [((312, 7, 7), 8, True, 312, 3, 1, 1), ((200, 9, 9), 3, True, 64, 3, 2, 2),
+                                                              ((78, 28, 28), 2, True, 78, 3, 1, 2), ((21, 9, 9), 2, False, 33, 3, 2, 3),
+                                                              ((176, 7, 7), 2, False, 176, 5, 1, 1), ((96, 8, 8), 5, True, 96, 5, 1, 3),
+                                                              ((3, 6, 6), 7, True, 5, 5, 2, 1), ((64, 10, 10), 2, True, 64, 7, 1, 1)]:
+        graph = separable_graph(in_shape, inputs, relu, oc, window, stride)
+        ops = rt.plan_describe(graph, batch)
+        kinds = [op['kind'] for op in ops]
+        dw = [op for op in ops if op['kind'] == 'conv_depthwise']
+        assert len(dw) == 1
+        if window <= 5:
+            assert dw[0]['inputs'] == inputs and 'nary' not in kinds and dw[0]['conv']['pre_relu'] == int(relu)
+        else:
+            assert dw[0]['inputs'] == 1 and kinds.count('nary') == 1      # 7 x 7 windows keep the summing launch
+        x = np.random.default_rng(14).standard_normal((batch, *in_shape)).astype(np.float32)
+        want = ios_oracle.run(graph, x)
+        outs = {}
+        for executor in ('streams', 'fused'):
+            rt.set_option('executor', executor)
+            outs[executor] = rt.graph_inference(graph, batch, x)
+            assert_close(outs[executor], want, f'depth-wise sum {in_shape} k={inputs} {window}x{window} {executor}')
+        np.testing.assert_array_equal(outs['fused'], outs['streams'])
+
+
+def test_depthwise_sums_share_fused_launches_with_other_operators():
+    """A stage whose groups hold depth-wise convolutions of sums (3 x 3, 5 x 5), a matrix-path convolution, a pool and a sum."""
+    def build(b, v):
+        a = ios.conv2d(b, [[v]], 20, (1, 1), act='identity')
+        c = ios.conv2d(b, [[v]], 20, (1, 1), act='identity')
+        u3 = ios.relu_sep_conv(b, [[a, c, v]], 24, (3, 3), (1, 1), (1, 1))
+        u5 = ios.sep_conv(b, [[a, c]], 24, (5, 5), (1, 1), (2, 2))
+        u7 = ios.relu_sep_conv(b, [[a, v]], 24, (7, 7), (1, 1), (3, 3))
+        e = ios.conv2d(b, [[a]], 24, (3, 3), padding=(1, 1))
+        f = ios.pool2d(b, [[c]], 'avg', (3, 3), (1, 1), (1, 1))
+        s = ios.identity(b, [[a, c]])
+        ios.identity(b, [[u3], [u5], [u7], [e], [f], [s]], is_exit=True)
+    graph = single_op_graph((20, 14, 14), build)
+    names = [n.name for n in graph.blocks[0].inner_nodes]
+    graph.blocks[0].stages = [[[names[0]], [names[1]]], [[n] for n in names[2:8]], [[graph.blocks[0].exit_node.name]]]
+    for batch in (1, 2):
+        x = np.random.default_rng(13).standard_normal((batch, 20, 14, 14)).astype(np.float32)
+        want = ios_oracle.run(graph, x)
+        outs = {}
+        for executor in ('streams', 'fused', 'fused_graph', 'graph'):
+            rt.set_option('executor', executor)
+            outs[executor] = rt.graph_inference(graph, batch, x)
+            assert_close(outs[executor], want, f'{executor} batch {batch}')
+        for executor in ('fused', 'fused_graph', 'graph'):
+            np.testing.assert_array_equal(outs[executor], outs['streams'])
+
+
 def model_cases():
     # (id, constructor, batch, strict tolerance).  Seeded non-zero biases everywhere; RandWire in the folded-batch-norm
     # form its configuration describes; NASNet both under the He-normal initialisation its configuration names (scaled

@@ -50,9 +50,15 @@ def test_host_planner_fuses_concats_and_folds_relus():
 
     rw = ios.models.randwire_small()
     rw.sequential_schedule()
-    kinds = collections.Counter(op['kind'] for op in rt.plan_describe(rw, 1))
+    ops = rt.plan_describe(rw, 1)
+    kinds = collections.Counter(op['kind'] for op in ops)
     assert kinds['conv_depthwise'] == 96 and kinds['conv_mfma'] == 99
-    folded = [op for op in rt.plan_describe(rw, 1) if op['kind'] == 'conv_depthwise' and op['conv']['pre_relu']]
+    # a node's depth-wise convolution adds the node's predecessors (and applies the ReLU) in its loader: the only summing
+    # launches left are the stage outputs
+    assert kinds['nary'] == 3 and sum(kinds.values()) == 200
+    depthwise = [op for op in ops if op['kind'] == 'conv_depthwise']
+    assert max(op['inputs'] for op in depthwise) >= 5 and all(op['conv']['pre_relu'] for op in depthwise if op['inputs'] > 1)
+    folded = [op for op in depthwise if op['inputs'] == 1 and op['conv']['pre_relu']]
     assert len(folded) > 0      # single-input nodes fold their ReLU into the depth-wise convolution
     nm = ios.models.nasnet_mobile()
     nm.sequential_schedule()
