@@ -440,6 +440,8 @@ private:
         op.kind = kind;
         op.node = owner.name;
         op.unit = owner.unit;
+        op.level = level_base_;
+        level_top_ = std::max(level_top_, op.level + 1);
         plan_.ops.push_back(op);
         return plan_.ops.back();
     }
@@ -465,6 +467,8 @@ private:
             op.act = last == term.size() ? act : ACT_NONE;
             op.flops = elems * (double)(last - first - (first > 0 ? 0 : 1));
             op.bytes = 4.0 * elems * (double)(last - first + 1 + (first > 0 ? 1 : 0));
+            op.level = level_base_ + (int)(first / kMaxNaryInputs);   // accumulation chunks of one term follow each other
+            level_top_ = std::max(level_top_, op.level + 1);
         }
     }
 
@@ -486,6 +490,7 @@ private:
             materialise_term(n, term, temp.window(offset, offset + len), ACT_NONE, false);
             offset += len;
         }
+        level_base_ = level_top_;   // the operator itself reads what the terms wrote
         return temp;
     }
 
@@ -493,6 +498,12 @@ private:
         PNode &n = nodes_[index];
         if (n.type == NodeType::Placeholder || n.type == NodeType::Sequential) return;
         if (n.no_storage) return;   // ReLU in front of a depth-wise convolution that reads the summed inputs itself
+        // levels count inside a schedule unit; the members of a Sequential follow each other
+        if (n.unit != level_unit_) {
+            level_unit_ = n.unit;
+            level_top_ = 0;
+        }
+        level_base_ = level_top_;
         int C, H, W;
         input_shape(n, C, H, W);
         const Json &cfg = *n.cfg;
@@ -690,6 +701,7 @@ private:
     }
 
     int batch_;
+    int level_unit_ = -2, level_base_ = 0, level_top_ = 0;   // PlanOp::level of the operations being emitted
     const LaunchChooser &chooser_;
     Plan plan_;
     std::vector<PNode> nodes_;
@@ -744,6 +756,7 @@ std::string describe_plan(const Plan &plan) {
         if (op.kind == OpKind::Nary) os << ",\"inputs\":" << op.srcs.size() << ",\"accumulate\":" << op.accumulate;
         if (op.kind == OpKind::ConvDepthwise) os << ",\"inputs\":" << (op.srcs.empty() ? 1 : op.srcs.size());
         if (op.kind == OpKind::Nary || op.kind == OpKind::Unary) os << ",\"act\":" << op.act;
+        os << ",\"level\":" << op.level;
         os << '}';
     }
     os << ']';

@@ -57,6 +57,9 @@ struct PlanOp {
     std::string node;     // operator name in the document
     int unit = -1;        // schedule unit (top-level operator) this op belongs to
     int stage = -1, group = -1;
+    // position in the dependency order of the operations of its unit: operations of one unit on the same level are independent
+    // of each other (the terms of a concatenation) and may run concurrently, a higher level reads what the lower ones wrote
+    int level = 0;
     ViewRef in, out;
     int conv = -1;        // index into Plan::convs
     PoolProblem pool{};

@@ -165,10 +165,11 @@ private:
     hipEvent_t start_ = nullptr, stop_ = nullptr;
     struct FusedLaunch {
         int threads, first_item, num_items, total_blocks, smem_bytes;
+        int single_op;   // >= 0: no fused launch, this plan operation is launched with its stand-alone kernel
         FusedHeader header;
         std::vector<int> ops;   // plan operations behind the items (a two-kernel split-K reduction names its convolution)
     };
-    std::vector<std::vector<FusedLaunch>> fused_stages_;   // per stage; empty for single-group stages
+    std::vector<std::vector<FusedLaunch>> fused_stages_;   // per stage; empty for stages whose operations all follow each other
     void *fused_items_ = nullptr;                          // device copy of all work items
     bool fused_built_ = false;
     hipGraph_t graph_ = nullptr;

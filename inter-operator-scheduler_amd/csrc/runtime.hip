@@ -610,9 +610,11 @@ void Session::enqueue(bool stage_events) {
 }
 
 // ---- fused stage launches -----------------------------------------------------------------------------------------
-// A multi-group stage is cut into levels: level l holds the l-th kernel of every group (a split-K convolution
-// contributes its main kernel and, one level later, its reduction).  The kernels of one level are independent
-// and become work items of one fused launch; levels follow each other on the main stream.
+// A stage is cut into levels: the operations of a group follow each other, except that operations of one unit on the same
+// PlanOp::level (the terms of a concatenation) share a level; a split-K convolution contributes its main kernel and, with
+// the two-kernel reduction, one level later its reduction.  The kernels of one level are independent and become work items
+// of one fused launch; levels follow each other on the main stream.  A single-group stage keeps its stand-alone kernels on
+// the levels that hold one operation.
 void Session::build_fused() {
     if (fused_built_) return;
     std::vector<WorkItem> items;
@@ -622,12 +624,35 @@ void Session::build_fused() {
         int threads;     // 0: any block size
         int smem_bytes;
         int op;          // plan operation behind the item
+        bool fusable;
     };
     for (size_t s = 0; s < plan_.stages.size(); s++) {
         const auto &groups = plan_.stages[s];
-        if (groups.size() <= 1) continue;
-        std::vector<std::vector<Pending>> chains(groups.size());
+        const bool solo = groups.size() <= 1;
+        if (solo) {
+            bool shared_level = false;
+            for (const auto &group : groups)
+                for (size_t i = 1; i < group.size(); i++) {
+                    const PlanOp &a = plan_.ops[group[i - 1]], &b = plan_.ops[group[i]];
+                    if (a.unit == b.unit && a.level == b.level) shared_level = true;
+                }
+            if (!shared_level) continue;
+        }
+        std::vector<std::vector<std::vector<Pending>>> chains(groups.size());   // group, level, items
         for (size_t g = 0; g < groups.size(); g++) {
+            auto &chain = chains[g];
+            int unit = -2;
+            size_t base = 0, shift = 0;
+            auto level_of = [&](const PlanOp &op) -> std::vector<Pending> & {
+                if (op.unit != unit) {
+                    unit = op.unit;
+                    base = chain.size();
+                    shift = 0;
+                }
+                const size_t at = base + shift + (size_t)op.level;
+                if (chain.size() <= at) chain.resize(at + 1);
+                return chain[at];
+            };
             for (int index : groups[g]) {
                 const PlanOp &op = plan_.ops[index];
                 Pending pend;
@@ -635,13 +660,15 @@ void Session::build_fused() {
                 pend.threads = 0;
                 pend.smem_bytes = 0;
                 pend.op = index;
+                pend.fusable = true;
                 int blocks = 0;
                 switch (op.kind) {
                     case OpKind::ConvMfma: {
                         const PlanConv &c = plan_.convs[op.conv];
                         const ConvDispatch d = make_conv_dispatch(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off,
                                                                   tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr, counters_of(c));
-                        if (!conv_variant(d.variant).fusable())
+                        pend.fusable = conv_variant(d.variant).fusable();
+                        if (!pend.fusable && !solo)
                             throw std::runtime_error(std::string("convolution kernel configuration ") + conv_variant(d.variant).name +
                                                      " cannot run inside a fused stage launch");
                         pend.item.kind = WORK_CONV;
@@ -652,8 +679,9 @@ void Session::build_fused() {
                         pend.item.conv = d.args;
                         pend.threads = d.threads;
                         pend.smem_bytes = d.smem_bytes;
-                        chains[g].push_back(pend);
-                        if (d.has_reduce) {
+                        if (d.has_reduce && solo) pend.fusable = false;   // launched stand-alone, reduction included
+                        level_of(op).push_back(pend);
+                        if (d.has_reduce && !solo) {
                             Pending red;
                             memset(&red.item, 0, sizeof(WorkItem));
                             red.item.kind = WORK_REDUCE;
@@ -662,7 +690,9 @@ void Session::build_fused() {
                             red.threads = 0;
                             red.smem_bytes = 0;
                             red.op = index;
-                            chains[g].push_back(red);
+                            red.fusable = true;
+                            shift++;
+                            level_of(op).push_back(red);
                         }
                         continue;
                     }
@@ -704,7 +734,7 @@ void Session::build_fused() {
                     }
                 }
                 pend.item.num_blocks = blocks;   // sized for 256-thread blocks, rescaled below
-                chains[g].push_back(pend);
+                level_of(op).push_back(pend);
             }
         }
         size_t depth = 0;
@@ -712,29 +742,40 @@ void Session::build_fused() {
         for (size_t level = 0; level < depth; level++) {
             std::vector<Pending *> here;
             int widest = 0;
+            bool all_fusable = true;
             for (auto &chain : chains)
-                if (level < chain.size()) {
-                    here.push_back(&chain[level]);
-                    widest = std::max(widest, chain[level].threads);
-                }
-            widest = std::max(widest, 256);   // narrowest instantiation of the fused kernel
-            // one launch per level, as wide as its widest convolution body
-            if (here.size() > (size_t)kMaxFusedItems) throw std::runtime_error("fused launch: too many groups in a stage");
-            FusedLaunch launch{widest, (int)items.size(), 0, 0, 0, {}, {}};
-            for (Pending *pend : here) {
-                launch.ops.push_back(pend->op);
-                WorkItem item = pend->item;
-                item.threads = pend->threads == 0 ? widest : pend->threads;
-                if (pend->threads == 0) item.num_blocks = std::max(1, (item.num_blocks * 256 + widest - 1) / widest);
-                item.first_block = launch.total_blocks;
-                if (launch.num_items < kFusedHeaderItems) launch.header.first_block[launch.num_items] = item.first_block;
-                launch.total_blocks += item.num_blocks;
-                launch.smem_bytes = std::max(launch.smem_bytes, pend->smem_bytes);
-                launch.num_items++;
-                items.push_back(item);
+                if (level < chain.size())
+                    for (Pending &pend : chain[level]) {
+                        here.push_back(&pend);
+                        widest = std::max(widest, pend.threads);
+                        all_fusable = all_fusable && pend.fusable;
+                    }
+            if (here.empty()) continue;
+            if (solo && (here.size() == 1 || !all_fusable)) {
+                for (Pending *pend : here) fused_stages_[s].push_back(FusedLaunch{0, 0, 0, 0, 0, pend->op, {}, {pend->op}});
+                continue;
             }
-            launch.header.num_items = launch.num_items;
-            fused_stages_[s].push_back(launch);
+            widest = std::max(widest, 256);   // narrowest instantiation of the fused kernel
+            // one launch per level, as wide as its widest convolution body; more items than a launch holds: several launches
+            for (size_t first = 0; first < here.size(); first += kMaxFusedItems) {
+                const size_t last = std::min(here.size(), first + (size_t)kMaxFusedItems);
+                FusedLaunch launch{widest, (int)items.size(), 0, 0, 0, -1, {}, {}};
+                for (size_t i = first; i < last; i++) {
+                    Pending *pend = here[i];
+                    launch.ops.push_back(pend->op);
+                    WorkItem item = pend->item;
+                    item.threads = pend->threads == 0 ? widest : pend->threads;
+                    if (pend->threads == 0) item.num_blocks = std::max(1, (item.num_blocks * 256 + widest - 1) / widest);
+                    item.first_block = launch.total_blocks;
+                    if (launch.num_items < kFusedHeaderItems) launch.header.first_block[launch.num_items] = item.first_block;
+                    launch.total_blocks += item.num_blocks;
+                    launch.smem_bytes = std::max(launch.smem_bytes, pend->smem_bytes);
+                    launch.num_items++;
+                    items.push_back(item);
+                }
+                launch.header.num_items = launch.num_items;
+                fused_stages_[s].push_back(launch);
+            }
         }
     }
     if (!items.empty()) {
@@ -751,13 +792,14 @@ void Session::enqueue_fused(bool stage_events) {
     hipStream_t main = ctx_.stream(0);
     const WorkItem *items = static_cast<const WorkItem *>(fused_items_);
     for (size_t s = 0; s < plan_.stages.size(); s++) {
-        const auto &groups = plan_.stages[s];
-        if (groups.size() <= 1) {
-            for (const auto &group : groups)
+        if (fused_stages_[s].empty()) {
+            for (const auto &group : plan_.stages[s])
                 for (int op : group) launch_op(plan_.ops[op], main);
         } else {
-            for (const FusedLaunch &l : fused_stages_[s])
-                launch_fused(l.threads, items + l.first_item, l.header, l.total_blocks, l.smem_bytes, main);
+            for (const FusedLaunch &l : fused_stages_[s]) {
+                if (l.single_op >= 0) launch_op(plan_.ops[l.single_op], main);
+                else launch_fused(l.threads, items + l.first_item, l.header, l.total_blocks, l.smem_bytes, main);
+            }
         }
         if (stage_events) IOS_HIP(hipEventRecord(stage_events_[s], main));
     }
@@ -907,11 +949,17 @@ std::vector<Session::LaunchRecord> Session::launches() {
     std::vector<LaunchRecord> out;
     for (size_t s = 0; s < plan_.stages.size(); s++) {
         const auto &groups = plan_.stages[s];
-        if (fused && groups.size() > 1) {
+        if (fused && !fused_stages_[s].empty()) {
             for (size_t l = 0; l < fused_stages_[s].size(); l++) {
                 const FusedLaunch &f = fused_stages_[s][l];
                 LaunchRecord r;
                 r.stage = (int)s;
+                if (f.single_op >= 0) {
+                    r.kernel = op_kernel_name(plan_, plan_.ops[f.single_op]);
+                    r.ops = {f.single_op};
+                    out.push_back(r);
+                    continue;
+                }
                 r.kernel = "fused_kernel<" + std::to_string(f.threads) + ">";
                 r.ops = f.ops;
                 r.blocks = f.total_blocks;

@@ -62,7 +62,16 @@ def test_host_planner_fuses_concats_and_folds_relus():
     assert len(folded) > 0      # single-input nodes fold their ReLU into the depth-wise convolution
     nm = ios.models.nasnet_mobile()
     nm.sequential_schedule()
-    assert len(rt.plan_describe(nm, 1)) > 400
+    ops = rt.plan_describe(nm, 1)
+    assert len(ops) > 400
+    # the sums of a cell's output concatenation are independent of each other: same unit, same level (one fused launch);
+    # the 1x1 convolution of a separable unit follows its depth-wise convolution
+    exit_sums = collections.defaultdict(list)
+    for op in ops:
+        if op['kind'] == 'nary':
+            exit_sums[op['node']].append(op['level'])
+    assert max(len(levels) for levels in exit_sums.values()) == 5 and all(set(levels) == {0} for levels in exit_sums.values())
+    assert all(op['level'] == 1 for op in ops if op['kind'] == 'conv_mfma' and op['conv']['kh'] == 1 and ops[ops.index(op) - 1]['kind'] == 'conv_depthwise')
 
 
 def test_host_planner_rejects_bad_documents():
