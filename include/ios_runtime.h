@@ -85,6 +85,10 @@ const char *ios_last_error(void);
  *       | "kernel" (a second kernel adds them); same results bit for bit;
  *   "precision" = "fp32" | "bf16": reduced-precision mode of the matrix-path convolutions (bfloat16 operands, fp32
  *       accumulation), the counterpart of the reference's USE_FLOAT16 build option (src/ios/ios_runtime.cu:19-43);
+ *   "arena_reuse" = "1" (default) | "0": operator outputs, temporaries and split-K partial tiles whose lifetimes (first to
+ *       last stage that touches them) do not intersect share device memory; the network input and the result never do.
+ *       The reference allocates every output for the lifetime of the graph (src/ios/ios_runtime.cu:1273-1285, 1318-1327).
+ *       With "0" every operator output survives the pass (ios_session_get_tensor on any node); needs no device;
  *   "conv_variant" = index or -1 and "conv_split_k" = count or 0 force one convolution kernel configuration (testing). */
 int ios_set_option(const char *key, const char *value);
 

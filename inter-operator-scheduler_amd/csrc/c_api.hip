@@ -127,6 +127,7 @@ const char *ios_last_error(void) { return g_last_error.c_str(); }
 int ios_set_option(const char *key, const char *value) {
     return guarded([&]() {
         if (key == nullptr || value == nullptr) throw std::runtime_error("option key or value is null");
+        if (ios::set_planner_option(key, value)) return;   // needs no device
         ios::DeviceContext::get().set_option(key, value);
     });
 }

@@ -5,6 +5,8 @@
 // three document kinds, :623-812 for the input algebra, :1047-1057 for pooling types).
 #include "plan.h"
 
+#include <climits>
+
 #include <algorithm>
 #include <cstdio>
 #include <set>
@@ -392,15 +394,119 @@ private:
         return index;
     }
 
+    // persistent storage (filters, biases, packed filters, ticket counters): final offsets, handed out front to back
     size_t reserve(size_t floats) {
         const size_t at = plan_.arena_floats;
         plan_.arena_floats += (floats + 63) & ~size_t(63);
         return at;
     }
 
+    // Storage with a lifetime (operator outputs, temporaries, split-K partial tiles): a region in a virtual address space,
+    // marked by kRegionTag in its offsets, that place_regions() maps behind the persistent storage once the stages are known.
+    static constexpr size_t kRegionTag = size_t(1) << 62;
+    struct Region {
+        size_t voff, floats;
+        int first = INT_MAX, last = -1;   // stages that touch it
+        bool pinned = false;              // lives for the whole pass (inputs, the result)
+        size_t at = 0;                    // final offset
+    };
+    size_t reserve_region(size_t floats, bool pinned = false) {
+        Region r;
+        r.voff = region_floats_;
+        r.floats = (std::max<size_t>(floats, 1) + 63) & ~size_t(63);
+        r.pinned = pinned;
+        region_floats_ += r.floats;
+        regions_.push_back(r);
+        return r.voff | kRegionTag;
+    }
+    Region *region_of(size_t offset) {
+        if (!(offset & kRegionTag)) return nullptr;
+        const size_t v = offset & ~kRegionTag;
+        auto it = std::upper_bound(regions_.begin(), regions_.end(), v, [](size_t value, const Region &r) { return value < r.voff; });
+        if (it == regions_.begin()) throw std::runtime_error("internal: view outside every region");
+        --it;
+        if (v >= it->voff + it->floats) throw std::runtime_error("internal: view outside its region");
+        return &*it;
+    }
+    void touch(size_t offset, int stage) {
+        if (Region *r = region_of(offset)) {
+            r->first = std::min(r->first, stage);
+            r->last = std::max(r->last, stage);
+        }
+    }
+    size_t placed(size_t offset) {
+        Region *r = region_of(offset);
+        return r ? r->at + ((offset & ~kRegionTag) - r->voff) : offset;
+    }
+
+    // Lifetimes from the stages of the operations that read or write a region; then first-fit placement, largest regions
+    // first, where two regions may share addresses when their lifetimes do not intersect (all operations of a stage have
+    // finished before the next stage starts, under every executor); finally every offset of the plan is rewritten.
+    void place_regions() {
+        const int last_stage = (int)plan_.stages.size() - 1;
+        for (const PlanOp &op : plan_.ops) {
+            touch(op.in.offset, op.stage);
+            touch(op.out.offset, op.stage);
+            for (const ViewRef &v : op.srcs) touch(v.offset, op.stage);
+            if (op.conv >= 0 && plan_.convs[op.conv].ws_floats > 0) touch(plan_.convs[op.conv].ws_off, op.stage);
+        }
+        if (Region *r = region_of(plan_.output.offset)) r->pinned = true;
+        const bool reuse = planner_arena_reuse();
+        for (Region &r : regions_)
+            if (r.pinned || !reuse || r.last < 0) {   // (an untouched region belongs to an operator nobody reads: keep it apart)
+                r.first = 0;
+                r.last = last_stage;
+            }
+        std::vector<Region *> order;
+        for (Region &r : regions_) order.push_back(&r);
+        std::stable_sort(order.begin(), order.end(), [](const Region *a, const Region *b) { return a->floats > b->floats; });
+        std::vector<Region *> done;
+        size_t extent = 0;
+        for (Region *r : order) {
+            // candidate offsets: 0 and the end of every placed region that is alive at the same time
+            std::vector<std::pair<size_t, size_t>> busy;   // [begin, end) of conflicting regions
+            for (Region *o : done)
+                if (o->first <= r->last && r->first <= o->last) busy.push_back({o->at, o->at + o->floats});
+            std::sort(busy.begin(), busy.end());
+            size_t at = 0;
+            for (const auto &b : busy) {
+                if (at + r->floats <= b.first) break;
+                at = std::max(at, b.second);
+            }
+            r->at = at;
+            extent = std::max(extent, at + r->floats);
+            done.push_back(r);
+        }
+        const size_t base = plan_.arena_floats;
+        plan_.persistent_floats = base;
+        plan_.activation_floats_without_reuse = region_floats_;
+        for (Region &r : regions_) r.at += base;
+        plan_.arena_floats = base + extent;
+        // names of the outputs that a later region overwrites
+        for (auto &entry : plan_.tensors) {
+            const Region *r = region_of(entry.second.offset);
+            if (r == nullptr) continue;
+            for (const Region &o : regions_)
+                if (&o != r && o.first > r->last && o.at < r->at + r->floats && r->at < o.at + o.floats) {
+                    plan_.overwritten.insert(entry.first);
+                    break;
+                }
+        }
+        for (PlanOp &op : plan_.ops) {
+            op.in.offset = placed(op.in.offset);
+            op.out.offset = placed(op.out.offset);
+            for (ViewRef &v : op.srcs) v.offset = placed(v.offset);
+        }
+        for (PlanConv &c : plan_.convs)
+            if (c.ws_floats > 0) c.ws_off = placed(c.ws_off);
+        for (auto &entry : plan_.tensors) entry.second.offset = placed(entry.second.offset);
+        plan_.input.offset = placed(plan_.input.offset);
+        plan_.output.offset = placed(plan_.output.offset);
+    }
+
     void allocate_outputs() {
         for (PNode &n : nodes_)
-            if (n.own) n.own_offset = reserve((size_t)batch_ * n.C * n.H * n.W);
+            if (n.own) n.own_offset = reserve_region((size_t)batch_ * n.C * n.H * n.W, /*pinned=*/n.type == NodeType::Placeholder);
     }
 
     ViewRef view_of(int index) const {
@@ -426,7 +532,7 @@ private:
 
     ViewRef dense_temp(int C, int H, int W) {
         ViewRef v;
-        v.offset = reserve((size_t)batch_ * C * H * W);
+        v.offset = reserve_region((size_t)batch_ * C * H * W);
         v.C = C;
         v.H = H;
         v.W = W;
@@ -694,10 +800,11 @@ private:
             conv.launch = chooser_(conv.problem, share[i]);
             conv.packed_off = reserve(conv_packed_floats(conv.problem, conv.launch));
             conv.ws_floats = conv_workspace_floats(conv.problem, conv.launch);
-            if (conv.ws_floats > 0) conv.ws_off = reserve(conv.ws_floats);
+            if (conv.ws_floats > 0) conv.ws_off = reserve_region(conv.ws_floats);
             conv.ctr_count = conv_counter_count(conv.problem, conv.launch);
             if (conv.ctr_count > 0) conv.ctr_off = reserve(conv.ctr_count);
         }
+        place_regions();
     }
 
     int batch_;
@@ -710,6 +817,8 @@ private:
     std::vector<int> unit_result_;
     struct SeqRange { int first, second; };
     std::vector<SeqRange> sequentials_;
+    std::vector<Region> regions_;   // ascending virtual offsets
+    size_t region_floats_ = 0;
 };
 
 void json_escape(std::ostringstream &os, const std::string &s) {
@@ -723,6 +832,20 @@ void json_escape(std::ostringstream &os, const std::string &s) {
 }
 
 }  // namespace
+
+namespace {
+bool g_arena_reuse = true;
+}
+
+bool set_planner_option(const std::string &key, const std::string &value) {
+    if (key == "arena_reuse") {
+        g_arena_reuse = !(value == "0" || value == "false" || value == "off" || value.empty());
+        return true;
+    }
+    return false;
+}
+
+bool planner_arena_reuse() { return g_arena_reuse; }
 
 Plan build_plan(PlanMode mode, const Json &doc, const Json *extra, int batch, const LaunchChooser &chooser) {
     Planner planner(batch, chooser);
@@ -757,6 +880,23 @@ std::string describe_plan(const Plan &plan) {
         if (op.kind == OpKind::ConvDepthwise) os << ",\"inputs\":" << (op.srcs.empty() ? 1 : op.srcs.size());
         if (op.kind == OpKind::Nary || op.kind == OpKind::Unary) os << ",\"act\":" << op.act;
         os << ",\"level\":" << op.level;
+        // arena extents in floats, one [begin, end) per image: what the operation writes and what it reads
+        auto ranges = [&](const char *key, const std::vector<ViewRef> &views) {
+            os << ",\"" << key << "\":[";
+            bool first_range = true;
+            for (const ViewRef &v : views)
+                for (int n = 0; n < plan.batch; n++) {
+                    const size_t begin = v.offset + (size_t)n * (size_t)v.bstride;
+                    os << (first_range ? "" : ",") << '[' << begin << ',' << begin + v.image_floats() << ']';
+                    first_range = false;
+                }
+            os << ']';
+        };
+        std::vector<ViewRef> reads = op.srcs;
+        if (op.kind != OpKind::Nary && op.srcs.empty()) reads.push_back(op.in);
+        if (op.kind == OpKind::Nary && op.accumulate) reads.push_back(op.out);
+        ranges("writes", {op.out});
+        ranges("reads", reads);
         os << '}';
     }
     os << ']';

@@ -13,6 +13,7 @@
 
 #include <functional>
 #include <map>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -79,6 +80,13 @@ struct Plan {
     ViewRef input, output;
     std::string input_name, output_name;
     size_t arena_floats = 0;
+    // layout of the arena: [0, persistent_floats) filters, biases, packed filters and split-K ticket counters, which live as
+    // long as the plan; behind them the regions of operator outputs, temporaries and split-K partial tiles.  With reuse
+    // (planner option "arena_reuse"), regions whose lifetimes (first to last stage that touches them) do not intersect share
+    // addresses; `overwritten` names the operators whose output does not survive to the end of a pass for that reason.
+    size_t persistent_floats = 0;
+    size_t activation_floats_without_reuse = 0;
+    std::set<std::string> overwritten;
     bool output_single_group = true;                     // the last stage has one group
 };
 
@@ -95,5 +103,9 @@ typedef std::function<ConvLaunch(const ConvProblem &, int share)> LaunchChooser;
 Plan build_plan(PlanMode mode, const Json &doc, const Json *extra, int batch, const LaunchChooser &chooser);
 
 std::string describe_plan(const Plan &plan);   // JSON array, one object per op
+
+// Planner options that need no device: "arena_reuse" = "1" (default) | "0".  Returns false for an unknown key.
+bool set_planner_option(const std::string &key, const std::string &value);
+bool planner_arena_reuse();
 
 }  // namespace ios

@@ -382,6 +382,7 @@ std::string DeviceContext::info_json() const {
        << ",\"executor\":\"" << (exec_mode_ == ExecMode::Graph ? "graph" : exec_mode_ == ExecMode::Fused ? "fused" : exec_mode_ == ExecMode::FusedGraph ? "fused_graph" : "streams") << "\",\"autotune\":" << (autotune_ ? "true" : "false")
        << ",\"split_k_reduce\":\"" << (inline_reduce_ ? "inline" : "kernel") << "\""
        << ",\"precision\":\"" << (bf16_ ? "bf16" : "fp32") << "\""
+       << ",\"arena_reuse\":" << (planner_arena_reuse() ? "true" : "false")
        << ",\"max_groups\":" << kMaxGroups << ",\"conv_variants\":[";
     for (int i = 0; i < conv_num_variants(); i++) os << (i ? "," : "") << '"' << conv_variant(i).name << '"';
     os << "]}";
@@ -525,6 +526,9 @@ void Session::get_output(float *host) {
 void Session::get_tensor(const std::string &name, float *host) {
     auto it = plan_.tensors.find(name);
     if (it == plan_.tensors.end()) throw std::runtime_error("operator '" + name + "' has no materialised output");
+    if (plan_.overwritten.count(name))
+        throw std::runtime_error("the output of operator '" + name + "' shares its memory with a later operator and does not survive the pass "
+                                 "(option arena_reuse=0 keeps every output)");
     copy_out(it->second, host);
 }
 

@@ -38,7 +38,9 @@ def default_options():
     rt.set_option('autotune', 0)            # closed-form kernel configurations keep the suite short and repeatable
     rt.set_option('split_k_reduce', 'inline')
     rt.set_option('precision', 'fp32')
+    rt.set_option('arena_reuse', 1)
     yield
+    rt.set_option('arena_reuse', 1)
     rt.set_option('precision', 'fp32')
     rt.set_option('autotune', 0)
     rt.set_option('conv_variant', -1)
@@ -235,12 +237,28 @@ def test_input_algebra_sum_concat_slice_activation_element():
     for batch in (1, 3):
         x = np.random.default_rng(4).standard_normal((batch, 5, 11, 11)).astype(np.float32)
         want = ios_oracle.run(graph, x, keep_all=True)
+        rt.set_option('arena_reuse', 0)      # every operator's output survives the pass
         with rt.Session(graph, batch) as session:
             session.load_weights()
             session.set_input(x)
             session.run()
             for node in list(graph.nodes())[1:]:
                 assert_close(session.tensor(node), want[node.name], f'node {node.name} ({node.type}) batch {batch}')
+        rt.set_option('arena_reuse', 1)
+        with rt.Session(graph, batch) as session:
+            session.load_weights()
+            session.set_input(x)
+            for _ in range(2):      # the second pass finds the input where the first one left it
+                session.run()
+            assert_close(session.output(), want[graph.exit_node.name], f'shared arena, batch {batch}')
+            unreadable = 0
+            for node in list(graph.nodes())[1:]:
+                try:
+                    assert_close(session.tensor(node), want[node.name], f'node {node.name} ({node.type}) batch {batch}, shared arena')
+                except RuntimeError as error:      # refused, not garbage: the node's memory was given to a later operator
+                    assert 'does not survive' in str(error)
+                    unreadable += 1
+            assert unreadable > 0
 
 
 def test_fused_stage_launch_covers_every_operator_kind():
@@ -400,6 +418,7 @@ def test_network_matches_oracle_under_every_schedule_and_executor(name, make, ba
     x = np.random.default_rng(1).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
     want_all = ios_oracle.run(graph, x, keep_all=True)
     want = want_all[graph.exit_node.name]
+    rt.set_option('arena_reuse', 0)      # node by node: every operator's output has to survive the pass
     with rt.Session(graph, batch) as session:
         session.load_weights()
         session.set_input(x)
@@ -421,6 +440,7 @@ def test_network_matches_oracle_under_every_schedule_and_executor(name, make, ba
             assert all(ulps <= 64.0 for _, _, _, ulps in report), report
     assert_close(got, want, name, scaled=not strict)
     assert np.isfinite(got).all() and np.abs(got).max() > 0
+    rt.set_option('arena_reuse', 1)      # everything below runs in the shared arena
 
     big = name.startswith(('randwire', 'nasnet'))
     greedy = make()

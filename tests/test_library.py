@@ -4,6 +4,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 
 import ios
@@ -201,3 +202,67 @@ def test_bench_refuses_more_than_one_gpu():
     done = subprocess.run([sys.executable, os.path.join(root, 'bench.py'), '--gpus', '2'], capture_output=True, text=True, timeout=60)
     assert done.returncode != 0
     assert 'single-GPU' in done.stderr
+
+
+def _simulate(ops):
+    """Runs a plan symbolically: every float of the arena remembers the operation that wrote it last.  Returns, per
+    operation, the writers it sees in what it reads; fails when two groups of one stage touch each other's memory."""
+    end = max(r[1] for op in ops for key in ('writes', 'reads') for r in op[key])
+    writer = np.full(end, -1, dtype=np.int32)
+    seen = []
+    stages = {}
+    for index, op in enumerate(ops):
+        stages.setdefault(op['stage'], []).append(index)
+    for stage in sorted(stages):
+        members = stages[stage]
+        # concurrency inside the stage: what one group writes, no other group reads or writes
+        mark = {}
+        for index in members:
+            for begin, stop in ops[index]['writes']:
+                mark.setdefault(ops[index]['group'], []).append((begin, stop))
+        for index in members:
+            op = ops[index]
+            for group, ranges in mark.items():
+                if group == op['group']:
+                    continue
+                for begin, stop in ranges:
+                    for b, e in op['reads'] + op['writes']:
+                        assert e <= begin or stop <= b, (op['node'], 'overlaps group', group, 'in stage', stage)
+        for index in members:       # launch order inside a stage: groups one after the other is one valid order
+            op = ops[index]
+            found = set()
+            for begin, stop in op['reads']:
+                found.update(np.unique(writer[begin:stop]).tolist())
+            seen.append(tuple(sorted(found)))
+            for begin, stop in op['writes']:
+                writer[begin:stop] = index
+    return seen
+
+
+@pytest.mark.parametrize('name,batch,schedule', [('squeezenet_1_1', 2, 'sequential'), ('squeezenet_1_1', 1, 'greedy'),
+                                                 ('randwire_small', 1, 'greedy'), ('nasnet_mobile', 1, 'greedy'),
+                                                 ('nasnet_mobile', 2, 'sequential'), ('inception_v3', 1, 'greedy')])
+def test_arena_reuse_never_lets_an_operator_read_what_another_overwrote(name, batch, schedule):
+    graph = getattr(ios.models, name)()
+    if schedule == 'greedy':
+        graph.greedy_schedule(8)
+    else:
+        graph.sequential_schedule()
+    try:
+        rt.set_option('arena_reuse', 0)
+        plain = rt.plan_describe(graph, batch)
+        plain_bytes = rt.plan_arena_bytes(graph, batch)
+        rt.set_option('arena_reuse', 1)
+        shared = rt.plan_describe(graph, batch)
+        shared_bytes = rt.plan_arena_bytes(graph, batch)
+    finally:
+        rt.set_option('arena_reuse', 1)
+    assert [(op['node'], op['kind']) for op in plain] == [(op['node'], op['kind']) for op in shared]
+    assert shared_bytes < 0.9 * plain_bytes
+    # every operation reads values written by exactly the same operations (or by nobody: the input, filters) in both plans
+    assert _simulate(shared) == _simulate(plain)
+    # the network input is never overwritten: no operation writes where the first operation reads
+    first_reads = shared[0]['reads']
+    for op in shared:
+        for begin, stop in op['writes']:
+            assert all(e <= begin or stop <= b for b, e in first_reads), op['node']
