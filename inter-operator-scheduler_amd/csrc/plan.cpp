@@ -481,7 +481,9 @@ private:
         plan_.persistent_floats = base;
         plan_.activation_floats_without_reuse = region_floats_;
         for (Region &r : regions_) r.at += base;
-        plan_.arena_floats = base + extent;
+        // (the vectorised pooling kernel reads up to eight floats past the end of a tensor and discards them: the arena ends
+        // in padding so that such a read stays inside the allocation)
+        plan_.arena_floats = base + extent + 64;
         // names of the outputs that a later region overwrites
         for (auto &entry : plan_.tensors) {
             const Region *r = region_of(entry.second.offset);

@@ -32,6 +32,7 @@ PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorV
     a.y_bs = y.bstride;
     a.p = p;
     a.strip_rows = 0;
+    a.vec_columns = 1;
     if (global) {
         *blocks = blocks_for((long long)p.B * p.C, 4, 4096);
     } else if (p.KH == 3 && p.KW == 3 && (p.sh == 1 || p.sh == 2)) {
@@ -39,7 +40,19 @@ PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorV
         int rows = kPoolStripRows;
         while (rows > 1 && (long long)p.B * p.C * ((p.OH + rows - 1) / rows) * p.OW < (1LL << 20)) rows >>= 1;
         a.strip_rows = rows;
-        *blocks = blocks_for((long long)p.B * p.C * ((p.OH + rows - 1) / rows) * p.OW, 256, 16384);
+        long long threads = (long long)p.B * p.C * ((p.OH + rows - 1) / rows) * p.OW;
+        // large tensors: four output columns per thread (16-byte loads and stores) while that leaves half a million threads
+        if ((p.sw == 1 || p.sw == 2) && p.pw <= 1 && p.W >= 8) {
+            auto quads = [&](int r) { return (long long)p.B * p.C * ((p.OH + r - 1) / r) * ((p.OW + kPoolVecColumns - 1) / kPoolVecColumns); };
+            int vrows = kPoolStripRows;
+            while (vrows > 1 && quads(vrows) < (1LL << 19)) vrows >>= 1;
+            if (quads(vrows) >= (1LL << 19)) {
+                a.vec_columns = kPoolVecColumns;
+                a.strip_rows = vrows;
+                threads = quads(vrows);
+            }
+        }
+        *blocks = blocks_for(threads, 256, 16384);
     } else {
         *blocks = blocks_for((long long)p.B * p.C * p.OH * p.OW, 256, 8192);
     }

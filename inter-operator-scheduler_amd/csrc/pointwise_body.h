@@ -25,6 +25,7 @@ struct PoolArgs {
     long long x_bs, y_bs;
     PoolProblem p;
     int strip_rows;   // 3 x 3 windows: output rows per thread (see pool3x3_body); 0 selects the generic body
+    int vec_columns;  // 3 x 3 windows: output columns per thread, 1 or kPoolVecColumns (see pool3x3_vec_body)
 };
 
 __device__ __forceinline__ void pool_generic_body(const PoolArgs &a, int block, int num_blocks) {
@@ -120,9 +121,110 @@ __device__ __forceinline__ void pool3x3_body(const PoolArgs &a, int block, int n
     }
 }
 
+// The same strips, four output columns wide: the form for large tensors, where the load instructions per byte decide.  A
+// thread reads an input row of its strip with one clamped scalar load and one (stride 1) or two (stride 2) 16-byte loads
+// at any 4-byte alignment instead of three loads per output column, and stores four outputs with one 16-byte store.  The
+// 16-byte loads may run up to eight elements past the end of a row; what they bring from there (the next row, the next
+// plane, or the padding that ends every arena) is replaced by the neutral element.  SW: stride along w (1 or 2), the
+// padding along w is at most 1.
+typedef float pw_floatx4_u __attribute__((ext_vector_type(4), aligned(4)));
+constexpr int kPoolVecColumns = 4;
+
+template <int SW>
+__device__ __forceinline__ void pool3x3_vec_body(const PoolArgs &a, int block, int num_blocks) {
+    const PoolProblem &p = a.p;
+    const int R = a.strip_rows;
+    constexpr int V = kPoolVecColumns;
+    constexpr int IN = SW * (V - 1) + 3;   // input columns of a row a thread reads: 6 or 9
+    const unsigned strips = (unsigned)((p.OH + R - 1) / R);
+    const unsigned quads = (unsigned)((p.OW + V - 1) / V);
+    const unsigned per_plane = strips * quads;
+    const unsigned total = per_plane * (unsigned)(p.C * p.B);
+    const bool is_max = p.is_max != 0;
+    const float neutral = is_max ? -INFINITY : 0.f;
+    for (unsigned i = block * blockDim.x + threadIdx.x; i < total; i += num_blocks * blockDim.x) {
+        const unsigned pc = i / per_plane;
+        const unsigned rest = i - pc * per_plane;
+        const unsigned strip = rest / quads;
+        const int ow0 = (int)(rest - strip * quads) * V;
+        const unsigned b = pc / (unsigned)p.C;
+        const unsigned c = pc - b * (unsigned)p.C;
+        const float *xc = a.x + (long long)b * a.x_bs + (long long)c * p.H * p.W;
+        float *yc = a.y + (long long)b * a.y_bs + (long long)c * p.OH * p.OW + ow0;
+        const int w0 = ow0 * SW - p.pw;          // first input column (-1 at the left edge with padding)
+        const int w0c = max(w0, 0);
+        // horizontal results of one input row for the four windows
+        auto row = [&](int h, float (&out)[V]) {
+            const bool in_h = (unsigned)h < (unsigned)p.H;
+            const float *xr = xc + min(max(h, 0), p.H - 1) * p.W;
+            float v[IN];
+            v[0] = xr[w0c];
+            const pw_floatx4_u q0 = *reinterpret_cast<const pw_floatx4_u *>(xr + w0 + 1);
+            v[1] = q0.x; v[2] = q0.y; v[3] = q0.z; v[4] = q0.w;
+            if constexpr (SW == 1) {
+                v[5] = xr[min(w0 + 5, p.W - 1)];
+            } else {
+                const pw_floatx4_u q1 = *reinterpret_cast<const pw_floatx4_u *>(xr + w0 + 5);
+                v[5] = q1.x; v[6] = q1.y; v[7] = q1.z; v[8] = q1.w;
+            }
+#pragma unroll
+            for (int j = 0; j < IN; j++) v[j] = (in_h && (unsigned)(w0 + j) < (unsigned)p.W) ? v[j] : neutral;
+#pragma unroll
+            for (int k = 0; k < V; k++)
+                out[k] = is_max ? fmaxf(fmaxf(v[SW * k], v[SW * k + 1]), v[SW * k + 2]) : (v[SW * k] + v[SW * k + 1]) + v[SW * k + 2];
+        };
+        auto store = [&](int oh, const float (&r0)[V], const float (&r1)[V], const float (&r2)[V]) {
+            float o[V];
+#pragma unroll
+            for (int k = 0; k < V; k++) o[k] = is_max ? fmaxf(fmaxf(r0[k], r1[k]), r2[k]) : ((r0[k] + r1[k]) + r2[k]) * (1.0f / 9.0f);
+            float *yr = yc + oh * p.OW;
+            if (ow0 + V <= p.OW) {
+                pw_floatx4_u q;
+                q.x = o[0]; q.y = o[1]; q.z = o[2]; q.w = o[3];
+                *reinterpret_cast<pw_floatx4_u *>(yr) = q;
+            } else {
+#pragma unroll
+                for (int k = 0; k < V; k++)
+                    if (ow0 + k < p.OW) yr[k] = o[k];
+            }
+        };
+        const int oh_begin = (int)strip * R;
+        const int oh_end = min(p.OH, oh_begin + R);
+        float r0[V], r1[V], r2[V];
+        if (p.sh == 1) {
+            row(oh_begin - p.ph, r0);
+            row(oh_begin - p.ph + 1, r1);
+            for (int oh = oh_begin; oh < oh_end; oh++) {
+                row(oh - p.ph + 2, r2);
+                store(oh, r0, r1, r2);
+#pragma unroll
+                for (int k = 0; k < V; k++) {
+                    r0[k] = r1[k];
+                    r1[k] = r2[k];
+                }
+            }
+        } else {
+            row(oh_begin * 2 - p.ph, r0);
+            for (int oh = oh_begin; oh < oh_end; oh++) {
+                row(oh * 2 - p.ph + 1, r1);
+                row(oh * 2 - p.ph + 2, r2);
+                store(oh, r0, r1, r2);
+#pragma unroll
+                for (int k = 0; k < V; k++) r0[k] = r2[k];
+            }
+        }
+    }
+}
+
 __device__ __forceinline__ void pool_body(const PoolArgs &a, int block, int num_blocks) {
-    if (a.strip_rows > 0) pool3x3_body(a, block, num_blocks);
-    else pool_generic_body(a, block, num_blocks);
+    if (a.strip_rows > 0 && a.vec_columns > 1) {
+        if (a.p.sw == 1) pool3x3_vec_body<1>(a, block, num_blocks);
+        else pool3x3_vec_body<2>(a, block, num_blocks);
+    } else if (a.strip_rows > 0) {
+        pool3x3_body(a, block, num_blocks);
+    } else {
+        pool_generic_body(a, block, num_blocks);
+    }
 }
 
 // window == whole map: one wavefront reduces one (image, channel) plane

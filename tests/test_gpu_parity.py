@@ -220,6 +220,37 @@ def test_pool_matches_oracle(case):
     assert_close(got, want, f'pool {case}')
 
 
+LARGE_POOLS = [
+    # tensors large enough for the form with four output columns per thread (16-byte loads at any alignment, reads past
+    # the end of a row that must be discarded): in_shape, type, stride, padding, batch
+    ((128, 35, 35), 'avg', 1, 1, 16),       # OW = 35: the last thread of a row holds three columns
+    ((128, 35, 35), 'max', 1, 1, 16),
+    ((96, 71, 71), 'max', 2, 0, 8),         # Inception-v3 reduction pools: odd width, no padding
+    ((176, 56, 56), 'avg', 2, 1, 16),       # NASNet: stride 2 with padding, even width
+    ((176, 56, 56), 'max', 2, 1, 16),
+    ((640, 9, 10), 'avg', 1, 1, 32),        # rows shorter than three threads' worth, width != height
+    ((512, 17, 17), 'max', 1, 0, 16),       # no padding: OW = 15
+]
+
+
+@pytest.mark.parametrize('case', LARGE_POOLS)
+def test_large_pool_with_four_columns_per_thread_matches_oracle(case):
+    in_shape, kind, stride, pad, batch = case
+    def build(b, v):
+        # the pool reads a channel window of the input and writes into a channel window of the concatenation
+        mid = Value(v.node, 3, in_shape[0] - 2)
+        a = ios.pool2d(b, [[mid]], kind, (3, 3), (stride, stride), (pad, pad))
+        c = ios.pool2d(b, [[Value(v.node, 0, 4)]], 'max' if kind == 'avg' else 'avg', (3, 3), (stride, stride), (pad, pad))
+        ios.identity(b, [[c], [a]], is_exit=True)
+    graph = single_op_graph(in_shape, build)
+    x = np.random.default_rng(5).standard_normal((batch, *in_shape)).astype(np.float32) - 2.0
+    want = ios_oracle.run(graph, x)
+    for executor in ('streams', 'fused'):
+        rt.set_option('executor', executor)
+        got = rt.graph_inference(graph, batch, x)
+        assert_close(got, want, f'large pool {case} {executor}')
+
+
 def test_input_algebra_sum_concat_slice_activation_element():
     def build(b, v):
         a = ios.conv2d(b, [[v]], 12, (1, 1), act='identity')
