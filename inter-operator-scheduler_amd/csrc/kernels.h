@@ -100,9 +100,11 @@ void launch_dwconv(const ConvProblem &p, const TensorView &x, const float *w, co
 bool dwconv_sums_inputs(const ConvProblem &p);   // the kernel for this window can add further inputs in its loader (3 x 3, 5 x 5)
 
 // Direct convolution for any geometry (one thread per output element); used for grouped convolutions
-// whose groups are too thin for the matrix path.
+// whose groups are too thin for the matrix path.  `thin` selects the form for 3 x 3 convolutions of 3-channel images
+// (conv_thin_applies), which is bound by the bytes of its output and serves first layers at large batches.
+inline bool conv_thin_applies(const ConvProblem &p) { return p.groups == 1 && p.IC == 3 && p.KH == 3 && p.KW == 3; }
 void launch_conv_direct(const ConvProblem &p, const TensorView &x, const float *w, const float *bias,
-                        const TensorView &y, hipStream_t stream);
+                        const TensorView &y, hipStream_t stream, bool thin = false);
 
 // ---- pooling ----------------------------------------------------------------------------------------
 struct PoolProblem {

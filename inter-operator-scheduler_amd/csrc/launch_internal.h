@@ -20,7 +20,7 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
                                 const float *bias, const TensorView &y, float *workspace, unsigned *counters);
 PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorView &y, bool global, int *blocks);
 DirectConvArgs make_direct_conv_args(const ConvProblem &p, const TensorView &x, const float *w, const float *bias,
-                                     const TensorView &y, int *blocks);
+                                     const TensorView &y, int *blocks, bool thin = false);
 // further inputs of a depth-wise convolution of a sum (see DirectConvArgs::more)
 void add_dwconv_sources(DirectConvArgs &a, const TensorView *more, int count);
 NaryKernelArgs make_nary_args(const NaryArgs &in, int multiply, int accumulate, int act, int B, long long chw,

@@ -683,6 +683,10 @@ private:
         }
         const int conv = add_plan_conv(n, p);
         plan_.convs[conv].matrix_path = matrix_path;
+        // K = 27: bound by the bytes of the output; from this size on the direct kernel with coalesced stores wins.  It is
+        // not part of the fused stage kernel, so finish() keeps the matrix path when the stage turns out to have several groups.
+        plan_.convs[conv].thin = matrix_path && conv_thin_applies(p) && planner_thin_conv_min_pixels() >= 0 &&
+                                 p.Npix() >= planner_thin_conv_min_pixels() && p.Npix() * p.OC < (1LL << 31);
         PlanOp &op = push(kind, n);
         op.in = in;
         op.out = view_of(index);
@@ -796,6 +800,16 @@ private:
                     for (const auto &other : stage) busy += other.size() > pos ? 1 : 0;
                     share[op.conv] = stage.size() > 1 ? std::max(2, busy) : 1;
                 }
+        for (PlanOp &op : plan_.ops) {
+            if (op.conv < 0 || !plan_.convs[op.conv].thin) continue;
+            PlanConv &conv = plan_.convs[op.conv];
+            if (plan_.stages[op.stage].size() == 1) {
+                conv.matrix_path = false;
+                op.kind = OpKind::ConvDirect;
+            } else {
+                conv.thin = false;
+            }
+        }
         for (size_t i = 0; i < plan_.convs.size(); i++) {
             PlanConv &conv = plan_.convs[i];
             if (!conv.matrix_path) continue;
@@ -837,6 +851,7 @@ void json_escape(std::ostringstream &os, const std::string &s) {
 
 namespace {
 bool g_arena_reuse = true;
+long long g_thin_conv_min_pixels = 1LL << 18;
 }
 
 bool set_planner_option(const std::string &key, const std::string &value) {
@@ -844,10 +859,15 @@ bool set_planner_option(const std::string &key, const std::string &value) {
         g_arena_reuse = !(value == "0" || value == "false" || value == "off" || value.empty());
         return true;
     }
+    if (key == "thin_conv_min_pixels") {
+        g_thin_conv_min_pixels = atoll(value.c_str());
+        return true;
+    }
     return false;
 }
 
 bool planner_arena_reuse() { return g_arena_reuse; }
+long long planner_thin_conv_min_pixels() { return g_thin_conv_min_pixels; }
 
 Plan build_plan(PlanMode mode, const Json &doc, const Json *extra, int batch, const LaunchChooser &chooser) {
     Planner planner(batch, chooser);
@@ -873,6 +893,7 @@ std::string describe_plan(const Plan &plan) {
             os << ",\"conv\":{\"ic\":" << p.IC << ",\"h\":" << p.H << ",\"w\":" << p.W << ",\"oc\":" << p.OC << ",\"kh\":" << p.KH
                << ",\"kw\":" << p.KW << ",\"sh\":" << p.sh << ",\"sw\":" << p.sw << ",\"ph\":" << p.ph << ",\"pw\":" << p.pw
                << ",\"groups\":" << p.groups << ",\"act\":" << p.act << ",\"pre_relu\":" << p.pre_relu << "}";
+            if (op.kind == OpKind::ConvDirect) os << ",\"thin\":" << (c.thin ? "true" : "false");
             if (c.matrix_path) {
                 os << ",\"variant\":\"" << conv_variant(c.launch.variant).name << "\",\"split_k\":" << c.launch.split_k
                    << ",\"fusable\":" << (conv_variant(c.launch.variant).fusable() ? "true" : "false");

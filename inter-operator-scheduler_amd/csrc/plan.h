@@ -51,6 +51,7 @@ struct PlanConv {
     size_t ctr_off = 0, ctr_count = 0;         // split-K ticket counters (32-bit words at float offsets), zeroed at session setup
     ConvLaunch launch;
     bool matrix_path = false;
+    bool thin = false;   // direct path: the kernel for 3 x 3 convolutions of 3-channel images (first layers at large batches)
 };
 
 struct PlanOp {
@@ -104,8 +105,11 @@ Plan build_plan(PlanMode mode, const Json &doc, const Json *extra, int batch, co
 
 std::string describe_plan(const Plan &plan);   // JSON array, one object per op
 
-// Planner options that need no device: "arena_reuse" = "1" (default) | "0".  Returns false for an unknown key.
+// Planner options that need no device: "arena_reuse" = "1" (default) | "0"; "thin_conv_min_pixels" = least number of output
+// pixels (batch x OH x OW) from which a 3 x 3 convolution of a 3-channel image takes the output-bound direct kernel instead
+// of the matrix path (default 2^18; a negative value disables it).  Returns false for an unknown key.
 bool set_planner_option(const std::string &key, const std::string &value);
 bool planner_arena_reuse();
+long long planner_thin_conv_min_pixels();
 
 }  // namespace ios

@@ -12,6 +12,10 @@ __global__ void pool_kernel(PoolArgs a) { pool_body(a, blockIdx.x, gridDim.x); }
 __global__ void global_pool_kernel(PoolArgs a) { global_pool_body(a, blockIdx.x, gridDim.x); }
 __global__ void dwconv_kernel(DirectConvArgs a) { dwconv_dispatch<true>(a, blockIdx.x, gridDim.x); }
 __global__ void conv_direct_kernel(DirectConvArgs a) { conv_direct_body(a, blockIdx.x, gridDim.x); }
+__global__ __launch_bounds__(256) void conv_thin_kernel(DirectConvArgs a) {
+    __shared__ float filters[kThinConvSmemFloats];
+    conv_thin_body(a, filters, blockIdx.x, gridDim.x);
+}
 __global__ void nary_kernel(NaryKernelArgs a) { nary_dispatch(a, blockIdx.x, gridDim.x); }
 
 static int blocks_for(long long n, int per_block, int cap) {
@@ -60,7 +64,7 @@ PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorV
 }
 
 DirectConvArgs make_direct_conv_args(const ConvProblem &p, const TensorView &x, const float *w, const float *bias,
-                                     const TensorView &y, int *blocks) {
+                                     const TensorView &y, int *blocks, bool thin) {
     if (x.C != p.IC || x.H != p.H || x.W != p.W || y.C != p.OC || y.H != p.OH || y.W != p.OW)
         throw std::runtime_error("conv: tensor views do not match the problem");
     if ((long long)p.B * p.OC * p.OH * p.OW >= (1LL << 31)) throw std::runtime_error("conv: tensor too large for 32-bit indexing");
@@ -81,6 +85,14 @@ DirectConvArgs make_direct_conv_args(const ConvProblem &p, const TensorView &x, 
         a.more_bytes[s] = 0;
     }
     *blocks = blocks_for((long long)p.B * p.OC * p.OH * p.OW, 256, 8192);
+    a.thin = 0;
+    if (thin) {
+        if (!conv_thin_applies(p)) throw std::runtime_error("conv: the thin-input kernel serves 3 x 3 convolutions of 3-channel inputs");
+        a.thin = 1;
+        // one block per 256 pixels and 32 output channels (sized for 256-thread blocks like the other bodies)
+        const long long units = (((long long)p.B * p.OH * p.OW + 255) / 256) * ((p.OC + kThinConvChannels - 1) / kThinConvChannels);
+        *blocks = (int)std::min<long long>(units, 1 << 20);
+    }
     return a;
 }
 
@@ -146,10 +158,11 @@ void launch_dwconv(const ConvProblem &p, const TensorView &x, const float *w, co
 }
 
 void launch_conv_direct(const ConvProblem &p, const TensorView &x, const float *w, const float *bias, const TensorView &y,
-                        hipStream_t stream) {
+                        hipStream_t stream, bool thin) {
     int blocks;
-    const DirectConvArgs a = make_direct_conv_args(p, x, w, bias, y, &blocks);
-    hipLaunchKernelGGL(conv_direct_kernel, dim3(blocks), dim3(256), 0, stream, a);
+    const DirectConvArgs a = make_direct_conv_args(p, x, w, bias, y, &blocks, thin);
+    if (thin) hipLaunchKernelGGL(conv_thin_kernel, dim3(blocks), dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL(conv_direct_kernel, dim3(blocks), dim3(256), 0, stream, a);
 }
 
 void launch_nary(const NaryArgs &in, int multiply, int accumulate, int act, int B, long long chw, const TensorView &y,

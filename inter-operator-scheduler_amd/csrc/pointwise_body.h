@@ -259,6 +259,7 @@ struct DirectConvArgs {
     long long x_bs, y_bs;
     ConvProblem p;
     unsigned x_bytes;   // extent of the input view in bytes when it is below 2^31 (branch-free depth-wise loads), else 0
+    int thin;           // direct convolution: 1 selects conv_thin_body (needs kThinConvSmemFloats floats of LDS)
     // depth-wise convolution of a sum: the input is x + more[0] + ... + more[nmore - 1] (added left to right, then the
     // folded ReLU), every view of the shape of x; the reference adds them with a kernel of its own (src/ios/ops.cu:26-48)
     const float *more[kMaxNaryInputs - 1];
@@ -375,6 +376,88 @@ __device__ __forceinline__ void dwconv_dispatch(const DirectConvArgs &a, int blo
     else if (p.KH == 5 && p.KW == 5) dwconv_body<5, 5>(a, block, num_blocks);
     else if (p.KH == 7 && p.KW == 7) dwconv_body<7, 7>(a, block, num_blocks);
     else dwconv_body<0, 0>(a, block, num_blocks);
+}
+
+// 3 x 3 convolution of a 3-channel image (the first layer of an image network) for large batches: K is 27, so the layer is
+// bound by the bytes of its output, not by arithmetic.  A block takes blockDim.x consecutive output pixels and kThinConvChannels
+// output channels: their 27 x 32 filter taps wait transposed in LDS and are read as broadcasts, a thread walks the nine filter rows with the three
+// input values of the next row in flight (clamped addresses, zeros selected for the padding), keeps 32 accumulators, and
+// every store instruction of a wavefront writes 64 consecutive pixels of one output channel.  Sum order: bias, then taps in
+// (channel, kh, kw) order, like the direct kernel.  `smem`: kThinConvSmemFloats floats.
+constexpr int kThinConvChannels = 32;
+constexpr int kThinConvTaps = 27;
+constexpr int kThinConvSmemFloats = (kThinConvTaps + 1) * kThinConvChannels;
+
+__device__ __forceinline__ void conv_thin_body(const DirectConvArgs &a, float *smem, int block, int num_blocks) {
+    const ConvProblem &p = a.p;
+    constexpr int OCB = kThinConvChannels, K = kThinConvTaps;
+    const unsigned ohw = (unsigned)(p.OH * p.OW);
+    const unsigned npix = ohw * (unsigned)p.B;
+    const unsigned pix_blocks = (npix + blockDim.x - 1) / blockDim.x;
+    const unsigned chunks = (unsigned)(p.OC + OCB - 1) / OCB;
+    const unsigned units = pix_blocks * chunks;
+    for (unsigned u = block; u < units; u += num_blocks) {
+        const unsigned chunk = u / pix_blocks;   // consecutive blocks share their filters
+        const unsigned pb = u - chunk * pix_blocks;
+        const int oc0 = (int)chunk * OCB;
+        __syncthreads();   // the previous unit's filters are no longer read
+        for (int i = threadIdx.x; i < (K + 1) * OCB; i += blockDim.x) {
+            const int t = i / OCB, o = i - t * OCB;
+            const int oc = min(oc0 + o, p.OC - 1);
+            smem[i] = t < K ? a.w[(size_t)oc * K + t] : a.bias[oc];
+        }
+        __syncthreads();
+        const unsigned n = pb * blockDim.x + threadIdx.x;
+        const bool valid = n < npix;
+        const unsigned nn = min(n, npix - 1);
+        const unsigned b = nn / ohw;
+        const unsigned r = nn - b * ohw;
+        const int oh = (int)(r / (unsigned)p.OW);
+        const int ow = (int)r - oh * p.OW;
+        const int h0 = oh * p.sh - p.ph, w0 = ow * p.sw - p.pw;
+        const float *xb = a.x + (long long)b * a.x_bs;
+        auto tap = [&](int c, int i2, int j) -> float {
+            const int h = h0 + i2, w = w0 + j;
+            const bool inside = (unsigned)h < (unsigned)p.H && (unsigned)w < (unsigned)p.W;
+            const float l = xb[(c * p.H + min(max(h, 0), p.H - 1)) * p.W + min(max(w, 0), p.W - 1)];
+            const float value = inside ? l : 0.f;
+            return p.pre_relu ? fmaxf(value, 0.f) : value;
+        };
+        float acc[OCB];
+#pragma unroll
+        for (int o = 0; o < OCB; o++) acc[o] = smem[K * OCB + o];
+        // a rolled loop over the taps (unrolled, the compiler fetches all 27 x 32 filter values first and spills them); the
+        // input values of one filter row (three taps) are requested while the previous row is being used
+        float v0 = tap(0, 0, 0), v1 = tap(0, 0, 1), v2 = tap(0, 0, 2);
+#pragma unroll 1
+        for (int row = 0; row < 9; row++) {
+            const int next = min(row + 1, 8);
+            const int nc = next / 3, ni = next - nc * 3;
+            const float n0 = tap(nc, ni, 0), n1 = tap(nc, ni, 1), n2 = tap(nc, ni, 2);
+            const pw_floatx4 *wt = reinterpret_cast<const pw_floatx4 *>(smem + row * 3 * OCB);
+#pragma unroll
+            for (int j = 0; j < 3; j++) {
+                const float value = j == 0 ? v0 : (j == 1 ? v1 : v2);
+#pragma unroll
+                for (int q = 0; q < OCB / 4; q++) {
+                    const pw_floatx4 w4 = wt[j * (OCB / 4) + q];
+                    acc[q * 4 + 0] = fmaf(value, w4.x, acc[q * 4 + 0]);
+                    acc[q * 4 + 1] = fmaf(value, w4.y, acc[q * 4 + 1]);
+                    acc[q * 4 + 2] = fmaf(value, w4.z, acc[q * 4 + 2]);
+                    acc[q * 4 + 3] = fmaf(value, w4.w, acc[q * 4 + 3]);
+                }
+            }
+            v0 = n0;
+            v1 = n1;
+            v2 = n2;
+        }
+        if (valid) {
+            float *yb = a.y + (long long)b * a.y_bs + r;
+#pragma unroll
+            for (int o = 0; o < OCB; o++)
+                if (oc0 + o < p.OC) yb[(long long)(oc0 + o) * ohw] = act_apply(acc[o], p.act);
+        }
+    }
 }
 
 __device__ __forceinline__ void conv_direct_body(const DirectConvArgs &a, int block, int num_blocks) {

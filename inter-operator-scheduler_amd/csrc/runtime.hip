@@ -555,7 +555,7 @@ void Session::launch_op(const PlanOp &op, hipStream_t stream) {
         }
         case OpKind::ConvDirect: {
             const PlanConv &c = plan_.convs[op.conv];
-            launch_conv_direct(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), stream);
+            launch_conv_direct(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), stream, c.thin);
             break;
         }
         case OpKind::Pool: launch_pool(op.pool, tv(op.in), tv(op.out), stream); break;
@@ -704,6 +704,7 @@ void Session::build_fused() {
                     case OpKind::ConvDirect: {
                         const PlanConv &c = plan_.convs[op.conv];
                         pend.item.kind = op.kind == OpKind::ConvDepthwise ? WORK_DWCONV : WORK_CONV_DIRECT;
+                        if (c.thin) throw std::runtime_error("internal: the thin-input convolution kernel is planned for single-group stages only");
                         pend.item.direct = make_direct_conv_args(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), &blocks);
                         if (op.kind == OpKind::ConvDepthwise && op.srcs.size() > 1) {
                             TensorView more[kMaxNaryInputs];
@@ -937,7 +938,7 @@ static std::string op_kernel_name(const Plan &plan, const PlanOp &op) {
     switch (op.kind) {
         case OpKind::ConvMfma: return std::string("conv_kernel<") + conv_variant(plan.convs[op.conv].launch.variant).name + ">";
         case OpKind::ConvDepthwise: return "dwconv_kernel";
-        case OpKind::ConvDirect: return "conv_direct_kernel";
+        case OpKind::ConvDirect: return plan.convs[op.conv].thin ? "conv_thin_kernel" : "conv_direct_kernel";
         case OpKind::Pool: return "pool_kernel";
         case OpKind::GlobalPool: return "global_pool_kernel";
         case OpKind::Nary:

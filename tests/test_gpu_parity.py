@@ -39,8 +39,10 @@ def default_options():
     rt.set_option('split_k_reduce', 'inline')
     rt.set_option('precision', 'fp32')
     rt.set_option('arena_reuse', 1)
+    rt.set_option('thin_conv_min_pixels', 1 << 18)
     yield
     rt.set_option('arena_reuse', 1)
+    rt.set_option('thin_conv_min_pixels', 1 << 18)
     rt.set_option('precision', 'fp32')
     rt.set_option('autotune', 0)
     rt.set_option('conv_variant', -1)
@@ -218,6 +220,55 @@ def test_pool_matches_oracle(case):
     got = rt.graph_inference(graph, batch, x)
     want = ios_oracle.run(graph, x)
     assert_close(got, want, f'pool {case}')
+
+
+THIN_CONVS = [
+    # 3 x 3 convolutions of 3-channel images on the output-bound direct kernel: in_shape, out_channels, stride, padding, act, batch
+    ((3, 31, 31), 32, 2, 0, 'relu', 2),
+    ((3, 30, 33), 40, 2, 1, 'relu', 3),         # output channels that do not fill the second block of 32, padding
+    ((3, 19, 17), 70, 1, 1, 'identity', 1),
+    ((3, 64, 64), 24, 1, 0, 'tanh', 5),         # fewer than 32 output channels
+    ((3, 299, 299), 32, 2, 0, 'relu', 4),       # Inception-v3's first layer, above the default size threshold
+]
+
+
+@pytest.mark.parametrize('case', THIN_CONVS)
+def test_first_layer_kernel_for_three_channel_images_matches_oracle(case):
+    in_shape, oc, stride, pad, act, batch = case
+    def build(b, v):
+        a = ios.conv2d(b, [[v]], oc, (3, 3), (stride, stride), (pad, pad), act=act)
+        c = ios.conv2d(b, [[a]], 8, (1, 1))
+        ios.identity(b, [[c], [a]], is_exit=True)       # the convolution stores into a channel window
+    graph = single_op_graph(in_shape, build)
+    rt.set_option('thin_conv_min_pixels', 0 if in_shape[1] < 100 else 1 << 16)
+    first = rt.plan_describe(graph, batch)[0]
+    assert first['kind'] == 'conv_direct' and first['thin'] is True
+    x = np.random.default_rng(6).standard_normal((batch, *in_shape)).astype(np.float32)
+    want = ios_oracle.run(graph, x)
+    outs = {}
+    for executor in ('streams', 'fused', 'fused_graph'):
+        rt.set_option('executor', executor)
+        outs[executor] = rt.graph_inference(graph, batch, x)
+        assert_close(outs[executor], want, f'thin conv {case} {executor}')
+    rt.set_option('thin_conv_min_pixels', -1)
+    assert rt.plan_describe(graph, batch)[0]['kind'] == 'conv_mfma'
+    assert_close(rt.graph_inference(graph, batch, x), want, f'matrix path {case}')
+
+
+def test_first_layer_kernel_stays_out_of_stages_with_several_groups():
+    def build(b, v):
+        a = ios.conv2d(b, [[v]], 32, (3, 3), (2, 2))
+        c = ios.conv2d(b, [[v]], 16, (3, 3), (2, 2))
+        ios.identity(b, [[a], [c]], is_exit=True)
+    graph = single_op_graph((3, 40, 40), build)
+    rt.set_option('thin_conv_min_pixels', 0)
+    assert [op['kind'] for op in rt.plan_describe(graph, 2)] == ['conv_direct', 'conv_direct']
+    names = [n.name for n in graph.blocks[0].inner_nodes]
+    graph.blocks[0].stages = [[[names[0]], [names[1]]], [[graph.blocks[0].exit_node.name]]]
+    assert [op['kind'] for op in rt.plan_describe(graph, 2)] == ['conv_mfma', 'conv_mfma']
+    x = np.random.default_rng(8).standard_normal((2, 3, 40, 40)).astype(np.float32)
+    rt.set_option('executor', 'fused')
+    assert_close(rt.graph_inference(graph, 2, x), ios_oracle.run(graph, x), 'parallel first layers')
 
 
 LARGE_POOLS = [

@@ -97,10 +97,12 @@ def test_reference_schedule_files_load_round_trip_and_plan(name):
     ops = rt.plan_describe(graph, reference_schedules.TUNED_BATCH[name])
     # slices of merged convolutions are read in place by convolutions and pools; only a slice that is itself a term of a
     # block's concatenation is copied there (at most one per merged convolution)
-    assert {op['kind'] for op in ops} <= {'conv_mfma', 'pool', 'global_pool', 'unary'}
+    # (at the batch sizes 16 ... 128 the first layer, a 3 x 3 convolution of the 3-channel image, takes the direct kernel)
+    assert {op['kind'] for op in ops} <= {'conv_mfma', 'conv_direct', 'pool', 'global_pool', 'unary'}
+    assert [op['kind'] for op in ops].count('conv_direct') <= 1
     merged = sum(' ' in n.hint_name for n in graph.nodes())
     assert sum(op['kind'] == 'unary' for op in ops) <= merged
-    assert sum(op['kind'] == 'conv_mfma' for op in ops) == sum(n.type == 'conv' for n in graph.nodes())
+    assert sum(op['kind'] in ('conv_mfma', 'conv_direct') for op in ops) == sum(n.type == 'conv' for n in graph.nodes())
 
 
 def test_reference_schedule_weights_from_the_plain_model_reproduce_its_output_on_the_oracle():
