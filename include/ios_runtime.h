@@ -89,6 +89,9 @@ const char *ios_last_error(void);
  *       last stage that touches them) do not intersect share device memory; the network input and the result never do.
  *       The reference allocates every output for the lifetime of the graph (src/ios/ios_runtime.cu:1273-1285, 1318-1327).
  *       With "0" every operator output survives the pass (ios_session_get_tensor on any node); needs no device;
+ *   "thin_conv_min_pixels" = count (default 262144; negative: never): a 3 x 3 convolution of a 3-channel image with at least
+ *       this many output pixels (batch x OH x OW) that has its stage to itself runs on a direct kernel bound by the bytes of
+ *       its output instead of the matrix path (first layers at large batches); needs no device;
  *   "conv_variant" = index or -1 and "conv_split_k" = count or 0 force one convolution kernel configuration (testing). */
 int ios_set_option(const char *key, const char *value);
 
