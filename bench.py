@@ -452,18 +452,19 @@ def main():
                 sweep[str(b)]['oracle'] = dict(oracle_check(np, out_own[sample], ios_oracle.run(graph, xb[sample])), images_checked=sample)
         result['batch_sweep'] = sweep
         if not args.no_extras:
-            # reduced-precision mode (bfloat16 operands, fp32 accumulation): not the headline metric, reported beside it
-            rt.set_option('precision', 'bf16')
-            reduced = {}
-            for b in (1, 64):
-                xb = np.random.default_rng(1).standard_normal((b, 3, 299, 299)).astype(np.float32)
-                r_seq, out_b = timed_latency(rt, np, graph, b, xb, max(10, args.steps // (b * 2)), 3)
-                reduced[str(b)] = {'sequential_ms': r_seq['wall'], 'images_per_s': b / (r_seq['wall'] * 1e-3)}
-                if b == 1:
-                    reduced[str(b)]['max_abs_diff_to_fp32'] = float(np.abs(out_b - seq_out).max())
-                    reduced[str(b)]['fp32_output_scale'] = float(np.abs(seq_out).max())
-            rt.set_option('precision', 'fp32')
-            result['reduced_precision_bf16'] = reduced
+            # reduced-precision modes (bfloat16 / half operands, fp32 accumulation): not the headline metric, reported beside it
+            for precision in ('bf16', 'fp16'):
+                rt.set_option('precision', precision)
+                reduced = {}
+                for b in (1, 64):
+                    xb = np.random.default_rng(1).standard_normal((b, 3, 299, 299)).astype(np.float32)
+                    r_seq, out_b = timed_latency(rt, np, graph, b, xb, max(10, args.steps // (b * 2)), 3)
+                    reduced[str(b)] = {'sequential_ms': r_seq['wall'], 'images_per_s': b / (r_seq['wall'] * 1e-3)}
+                    if b == 1:
+                        reduced[str(b)]['max_abs_diff_to_fp32'] = float(np.abs(out_b - seq_out).max())
+                        reduced[str(b)]['fp32_output_scale'] = float(np.abs(seq_out).max())
+                rt.set_option('precision', 'fp32')
+                result['reduced_precision_' + precision] = reduced
 
     if not args.no_configs:
         configs = {}

@@ -83,8 +83,9 @@ const char *ios_last_error(void);
  *       cudnnFind-based selection (src/ios/ios_runtime.cu:150-205); "clear_tuning" = anything forgets them;
  *   "split_k_reduce" = "inline" (the last block of a tile adds the split-K slices inside the convolution kernel)
  *       | "kernel" (a second kernel adds them); same results bit for bit;
- *   "precision" = "fp32" | "bf16": reduced-precision mode of the matrix-path convolutions (bfloat16 operands, fp32
- *       accumulation), the counterpart of the reference's USE_FLOAT16 build option (src/ios/ios_runtime.cu:19-43);
+ *   "precision" = "fp32" | "bf16" | "fp16": reduced-precision modes of the matrix-path convolutions (bfloat16 or IEEE half
+ *       operands, fp32 accumulation and outputs); "fp16" is the counterpart of the reference's USE_FLOAT16 build option
+ *       (src/ios/ios_runtime.cu:19-43), with its range (operands beyond 65504 become infinite);
  *   "arena_reuse" = "1" (default) | "0": operator outputs, temporaries and split-K partial tiles whose lifetimes (first to
  *       last stage that touches them) do not intersect share device memory; the network input and the result never do.
  *       The reference allocates every output for the lifetime of the graph (src/ios/ios_runtime.cu:1273-1285, 1318-1327).

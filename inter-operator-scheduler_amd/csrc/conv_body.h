@@ -127,6 +127,7 @@ __device__ __forceinline__ floatx4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, u
 
 typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uintx2 buffer_load_u32x2(__amdgpu_buffer_rsrc_t r, unsigned byte_offset, unsigned scalar_offset = 0) {
     return __builtin_amdgcn_raw_buffer_load_b64(r, byte_offset, scalar_offset, 0);
@@ -502,7 +503,7 @@ __device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int bloc
 //
 // CP: channel padding of the packed filters when it should differ from the default (8, or the batch with QUAD); 4 serves
 // layers with a handful of input channels (the first layer of an image network), whose K would otherwise be mostly padding.
-template <int MT, int TM, int TN, int NW, int U, bool QUAD = false, int D = 2, bool BF16 = false, int CP = 0>
+template <int MT, int TM, int TN, int NW, int U, bool QUAD = false, int D = 2, int RP = 0, int CP = 0>
 struct ConvWsplit {
     using M = Mfma<MT>;
     static constexpr int BM = TM * MT, BN = TN * MT;
@@ -515,9 +516,9 @@ struct ConvWsplit {
     // accumulators + staged operands per lane decide whether the body fits the register budget of a fused launch
     // (the channel-padding-4 forms serve first layers, which are stages of their own: kept out of the fused launches)
     static constexpr bool FUSABLE = CP == 0 && E + D * U * (TM + TN) <= (QUAD ? 56 : 48);   // per-step addressing of the plain layout needs more registers
-    static constexpr bool KBF16 = BF16;                    // packed filters hold bfloat16
+    static constexpr int KREDUCED = RP;                    // 0: fp32 filters; 1: packed filters hold bfloat16; 2: IEEE half
     static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
-    static_assert(!BF16 || (QUAD && MT == 16 && U == 4), "the bfloat16 path is the 16 x 16 x 16 form of the quad layout");
+    static_assert(RP >= 0 && RP <= 2 && (RP == 0 || (QUAD && MT == 16 && U == 4)), "the 16-bit paths are the 16 x 16 x 16 form of the quad layout");
 
     __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *red, int tile, int g, int z) {
 
@@ -566,7 +567,7 @@ struct ConvWsplit {
         w_kill[i] = m0 + i * MT + lc < a.OCgP ? 0u : kOutOfRange;
         // byte offsets below 2^31 (checked on the host)
         if (QUAD)   // [g][k / 4][m][4]: this lane's first quad of a batch is row (U / 4) * lk
-            w_lane[i] = (((unsigned)g * ((unsigned)a.Kq >> 2) + (unsigned)((U / 4) * lk)) * (unsigned)a.OCgP + (unsigned)(m0 + i * MT + lc)) * (BF16 ? 8u : 16u);
+            w_lane[i] = (((unsigned)g * ((unsigned)a.Kq >> 2) + (unsigned)((U / 4) * lk)) * (unsigned)a.OCgP + (unsigned)(m0 + i * MT + lc)) * (RP != 0 ? 8u : 16u);
         else
             w_lane[i] = (((unsigned)g * (unsigned)a.Kq + (unsigned)lk) * (unsigned)a.OCgP + (unsigned)(m0 + i * MT + lc)) * 4u;
     }
@@ -597,7 +598,7 @@ struct ConvWsplit {
     struct FilterStageBf16 {
         uintx2 v[TM];
     };
-    using FilterStage = std::conditional_t<BF16, FilterStageBf16, FilterStageF32>;
+    using FilterStage = std::conditional_t<(RP != 0), FilterStageBf16, FilterStageF32>;
     FilterStage av[D];
     float bv[D][U][TN];
 
@@ -612,7 +613,7 @@ struct ConvWsplit {
         q_cb = kb - tap * a.ICgP;
         q_kh = a.KW == 1 ? tap : (int)__umulhi((unsigned)tap, a.magic_kw);
         q_kw = tap - q_kh * a.KW;
-        q_w = (unsigned)((kb / 4) * a.OCgP) * (BF16 ? 8u : 16u);
+        q_w = (unsigned)((kb / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
     }
     auto load_batch = [&](int s0, FilterStage &A, float(&B)[U][TN]) {
         if constexpr (QUAD) {
@@ -621,9 +622,9 @@ struct ConvWsplit {
             // offsets go into the vector operand of the buffer loads, the per-batch / per-step parts into the scalar
             // operand: a filter load costs no VALU instruction, an input load one add + one or per batch and tile.
             (void)s0;
-            if constexpr (BF16) {
+            if constexpr (RP != 0) {
 #pragma unroll
-                for (int i = 0; i < TM; i++) {   // four bfloat16 = the lane's four k of this batch
+                for (int i = 0; i < TM; i++) {   // four 16-bit values = the lane's four k of this batch
                     A.v[i] = buffer_load_u32x2(wr, w_lane[i] | w_kill[i], q_w);
                 }
             } else {
@@ -662,7 +663,7 @@ struct ConvWsplit {
                     for (int j = 0; j < TN; j++) B[u][j] = buffer_load_f32(xr, voff[j], x_chan + (unsigned)(u * a.HW) * 4u);
             }
             // next batch
-            q_w += (unsigned)((U * M::KSTEP / 4) * a.OCgP) * (BF16 ? 8u : 16u);
+            q_w += (unsigned)((U * M::KSTEP / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
             q_cb += U * M::KSTEP;
             if (q_cb >= a.ICgP) {
                 q_cb = 0;
@@ -700,15 +701,21 @@ struct ConvWsplit {
     // folded ReLU of the producer: as integers, negative floats are below 0 and everything is above INT_MIN
     const int relu_floor = a.pre_relu ? 0 : (int)0x80000000;
     auto compute = [&](const FilterStage &A, const float(&B)[U][TN]) {
-        if constexpr (BF16) {
+        if constexpr (RP != 0) {
 #pragma unroll
             for (int j = 0; j < TN; j++) {
                 const floatx4 b32 = {__int_as_float(max(__float_as_int(B[0][j]), relu_floor)), __int_as_float(max(__float_as_int(B[1][j]), relu_floor)),
                                      __int_as_float(max(__float_as_int(B[2][j]), relu_floor)), __int_as_float(max(__float_as_int(B[3][j]), relu_floor))};
-                const bf16x4 b4 = __builtin_convertvector(b32, bf16x4);   // round to nearest even
+                if constexpr (RP == 1) {
+                    const bf16x4 b4 = __builtin_convertvector(b32, bf16x4);   // round to nearest even
 #pragma unroll
-                for (int i = 0; i < TM; i++) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(bf16x4, A.v[i]), b4, acc[i][j], 0, 0, 0);
+                    for (int i = 0; i < TM; i++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(bf16x4, A.v[i]), b4, acc[i][j], 0, 0, 0);
+                } else {
+                    const halfx4 b4 = __builtin_convertvector(b32, halfx4);   // round to nearest even, overflow to infinity
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(halfx4, A.v[i]), b4, acc[i][j], 0, 0, 0);
                 }
             }
             return;
@@ -903,6 +910,19 @@ struct ConvWsplit {
     X(66, "wq_m64n32_w8_t32_u4", 32, 2, 1, 8, 4, true, 2, false)     \
     X(67, "wq_m64n64_w4_t32_u4", 32, 2, 2, 4, 4, true, 2, false)     \
     X(68, "wq_m64n32_w4_t32_u4_d4", 32, 2, 1, 4, 4, true, 4, false)
-constexpr int kNumConvVariants = 69;
+// X(index, name, MT, TM, TN, NW, U, QUAD, D, RP): the reduced-precision configurations once more with IEEE half operands
+// (RP = 2, option precision=fp16), the literal counterpart of the reference's USE_FLOAT16 build
+#define IOS_WSPLIT_F16_VARIANTS(X)                          \
+    X(69, "wh_m16n16_w16", 16, 1, 1, 16, 4, true, 2, 2)     \
+    X(70, "wh_m16n16_w8_d4", 16, 1, 1, 8, 4, true, 4, 2)    \
+    X(71, "wh_m32n16_w8", 16, 2, 1, 8, 4, true, 2, 2)       \
+    X(72, "wh_m32n16_w16", 16, 2, 1, 16, 4, true, 2, 2)     \
+    X(73, "wh_m32n32_w8", 16, 2, 2, 8, 4, true, 2, 2)       \
+    X(74, "wh_m32n32_w4_d4", 16, 2, 2, 4, 4, true, 4, 2)    \
+    X(75, "wh_m64n16_w8", 16, 4, 1, 8, 4, true, 2, 2)       \
+    X(76, "wh_m64n32_w8", 16, 4, 2, 8, 4, true, 2, 2)       \
+    X(77, "wh_m64n32_w4_d4", 16, 4, 2, 4, 4, true, 4, 2)    \
+    X(78, "wh_m64n64_w4", 16, 4, 4, 4, 4, true, 2, 2)
+constexpr int kNumConvVariants = 79;
 
 }  // namespace ios

@@ -41,7 +41,7 @@ struct VariantEntry {
 
 static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)
                                              IOS_WSPLIT_C4_VARIANTS(IOS_WSPLIT_C4_ENTRY)
-                                             IOS_WSPLIT_T32_VARIANTS(IOS_WSPLIT_ENTRY)};
+                                             IOS_WSPLIT_T32_VARIANTS(IOS_WSPLIT_ENTRY) IOS_WSPLIT_F16_VARIANTS(IOS_WSPLIT_ENTRY)};
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 static_assert(kNumVariants == kNumConvVariants, "variant lists and count disagree");
 
@@ -90,7 +90,7 @@ static int variant_by_name(const char *name) {
     throw std::runtime_error(std::string("conv: no kernel configuration named ") + name);
 }
 
-ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only, bool bf16) {
+ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only, int precision) {
     // Closed-form model distilled from measured choices on Inception-v3 at batch 1, 16 and 64: problems that fill
     // the device several times over with 64 x 64 tiles take the LDS-tiled kernel (the largest tile that still
     // offers two blocks per compute unit); smaller ones take the wave-split kernel with the largest tile that
@@ -101,16 +101,23 @@ ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only
         return (long long)ceil_div(M, v.BM) * ceil_div(N, v.BN) * p.groups;
     };
     ConvLaunch best;
-    if (bf16) {
+    if (precision != PREC_FP32) {
         // reduced precision: wave-split configurations only, the largest tile that offers two blocks per compute unit
-        static const int large_to_small[] = {variant_by_name("wb_m64n64_w4"), variant_by_name("wb_m64n32_w8"),
-                                             variant_by_name("wb_m32n32_w8"), variant_by_name("wb_m32n16_w8")};
-        for (int idx : large_to_small)
+        static const int bf16_large_to_small[] = {variant_by_name("wb_m64n64_w4"), variant_by_name("wb_m64n32_w8"),
+                                                  variant_by_name("wb_m32n32_w8"), variant_by_name("wb_m32n16_w8"),
+                                                  variant_by_name("wb_m16n16_w16")};
+        static const int fp16_large_to_small[] = {variant_by_name("wh_m64n64_w4"), variant_by_name("wh_m64n32_w8"),
+                                                  variant_by_name("wh_m32n32_w8"), variant_by_name("wh_m32n16_w8"),
+                                                  variant_by_name("wh_m16n16_w16")};
+        const int *large_to_small = precision == PREC_BF16 ? bf16_large_to_small : fp16_large_to_small;
+        for (int i = 0; i < 4; i++) {
+            const int idx = large_to_small[i];
             if ((!fusable_only || kVariants[idx].v.fusable()) && blocks_of(idx) >= 2LL * num_cus) {
                 best.variant = idx;
                 return best;
             }
-        best.variant = variant_by_name("wb_m16n16_w16");
+        }
+        best.variant = large_to_small[4];
         const ConvVariant &v = kVariants[best.variant].v;
         const long long blocks = blocks_of(best.variant);
         const int batches = ceil_div(p.Kq(v.cpad), v.BK);
@@ -183,7 +190,7 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     a.HW = p.H * p.W; a.OHW = p.OH * p.OW; a.groups = p.groups;
     a.x_bs = x.bstride; a.y_bs = y.bstride;
     const unsigned long long x_bytes = ((unsigned long long)(p.B - 1) * x.bstride + (unsigned long long)p.IC * p.H * p.W) * 4ull;
-    const unsigned long long w_bytes = (unsigned long long)p.groups * p.Kq(e.v.cpad) * p.OCgP() * (e.v.bf16 ? 2ull : 4ull);
+    const unsigned long long w_bytes = (unsigned long long)p.groups * p.Kq(e.v.cpad) * p.OCgP() * (e.v.precision != PREC_FP32 ? 2ull : 4ull);
     if (x_bytes >= (1ull << 31) || w_bytes >= (1ull << 31)) throw std::runtime_error("conv: tensor too large for 31-bit buffer offsets");
     a.x_bytes = (unsigned)x_bytes;
     a.w_bytes = (unsigned)w_bytes;
@@ -247,7 +254,7 @@ void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorVie
 
 // ---- filter packing ------------------------------------------------------------------------
 __global__ void pack_filters_kernel(const float *w, float *packed, int OCg, int OCgP, int ICg, int ICgP, int taps, int groups, int kquad,
-                                    int bf16) {
+                                    int precision) {
     // packed[g][k][m] = w[g * OCg + m][c][tap] with k = tap * ICgP + c;  rows with c >= ICg and columns with m >= OCg are zero.
     // kquad: packed[g][k / 4][m][k % 4] instead (ICgP is a multiple of 4)
     const size_t total = (size_t)groups * taps * ICgP * OCgP;
@@ -267,7 +274,8 @@ __global__ void pack_filters_kernel(const float *w, float *packed, int OCg, int 
         const int tap = (int)(gt % taps);
         const int g = (int)(gt / taps);
         const float value = (m < OCg && c < ICg) ? w[(((size_t)g * OCg + m) * ICg + c) * taps + tap] : 0.f;
-        if (bf16) reinterpret_cast<__bf16 *>(packed)[i] = (__bf16)value;   // round to nearest even
+        if (precision == PREC_BF16) reinterpret_cast<__bf16 *>(packed)[i] = (__bf16)value;   // round to nearest even
+        else if (precision == PREC_FP16) reinterpret_cast<_Float16 *>(packed)[i] = (_Float16)value;   // round to nearest even
         else packed[i] = value;
     }
 }
@@ -275,7 +283,7 @@ __global__ void pack_filters_kernel(const float *w, float *packed, int OCg, int 
 size_t conv_packed_floats(const ConvProblem &p, const ConvLaunch &l) {
     if (l.variant < 0 || l.variant >= kNumVariants) throw std::runtime_error("conv: bad variant");
     const size_t elements = (size_t)p.groups * p.Kq(kVariants[l.variant].v.cpad) * p.OCgP();
-    return kVariants[l.variant].v.bf16 ? (elements + 1) / 2 : elements;
+    return kVariants[l.variant].v.precision != PREC_FP32 ? (elements + 1) / 2 : elements;
 }
 
 size_t conv_packed_floats_max(const ConvProblem &p) {
@@ -289,7 +297,7 @@ void launch_pack_filters(const ConvProblem &p, const ConvLaunch &l, const float 
     const size_t total = (size_t)p.groups * p.Kq(cpad) * p.OCgP();   // elements
     const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 65535);
     hipLaunchKernelGGL(pack_filters_kernel, dim3(blocks), dim3(256), 0, stream, w, packed, p.OCg(), p.OCgP(), p.ICg(), p.ICgP(cpad),
-                       p.KH * p.KW, p.groups, kVariants[l.variant].v.kquad ? 1 : 0, kVariants[l.variant].v.bf16 ? 1 : 0);
+                       p.KH * p.KW, p.groups, kVariants[l.variant].v.kquad ? 1 : 0, kVariants[l.variant].v.precision);
 }
 
 }  // namespace ios

@@ -48,6 +48,7 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fus
                 IOS_WSPLIT_VARIANTS(IOS_CASE_WSPLIT)
                 IOS_WSPLIT_C4_VARIANTS(IOS_CASE_WSPLIT_C4)
                 IOS_WSPLIT_T32_VARIANTS(IOS_CASE_WSPLIT)
+                IOS_WSPLIT_F16_VARIANTS(IOS_CASE_WSPLIT)
 #undef IOS_CASE_WSPLIT_C4
 #undef IOS_CASE_TILED
 #undef IOS_CASE_WSPLIT

@@ -13,6 +13,7 @@
 namespace ios {
 
 enum Act : int { ACT_NONE = 0, ACT_RELU = 1, ACT_TANH = 2, ACT_SIGMOID = 3 };
+enum Precision : int { PREC_FP32 = 0, PREC_BF16 = 1, PREC_FP16 = 2 };   // operand type of the matrix-path convolutions
 
 constexpr int kMaxNaryInputs = 8;   // views one launch adds (or multiplies)
 
@@ -51,7 +52,7 @@ struct ConvVariant {
     bool kquad; // packed filters are [k / 4][m][4] (16-byte loads along k) instead of [k][m]
     int threads() const { return 64 * WM * WN * WK; }
     bool fusable_;   // light enough on registers to run inside a fused stage launch
-    bool bf16;       // reduced-precision mode: bfloat16 filters and inputs, fp32 accumulation
+    int precision;   // PREC_FP32, or a reduced-precision mode: bfloat16 / IEEE half filters and inputs, fp32 accumulation
     bool fusable() const { return fusable_; }
 };
 
@@ -75,12 +76,12 @@ bool conv_matrix_path_supported(const ConvProblem &p);
 
 // Default configuration from a closed-form occupancy model (num_cus = compute units of the device);
 // fusable_only restricts the choice to configurations that can run inside a fused stage launch.
-// bf16 selects among the reduced-precision configurations.
-ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only = false, bool bf16 = false);
+// precision selects the family of configurations (fp32, bfloat16 or half operands).
+ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only = false, int precision = PREC_FP32);
 
 // Filter packing for a kernel configuration: w[OC][ICg][KH][KW] -> packed[g][k = (kh*KW + kw)*ICgP + c][OCgP]
 // (or [g][k / 4][OCgP][k % 4] for kquad configurations), ICgP = ICg rounded up to the configuration's channel
-// padding (zero rows), OCgP = OCg rounded up to 4.  bf16 configurations pack bfloat16 (round to nearest even), two
+// padding (zero rows), OCgP = OCg rounded up to 4.  16-bit configurations pack bfloat16 or half (round to nearest even), two
 // per float of the returned size.
 size_t conv_packed_floats(const ConvProblem &p, const ConvLaunch &l);
 size_t conv_packed_floats_max(const ConvProblem &p);   // over all configurations

@@ -73,7 +73,7 @@ private:
     unsigned *tune_counters_ = nullptr;
     size_t tune_counter_count_ = 0;
     bool inline_reduce_ = true;
-    bool bf16_ = false;   // reduced-precision mode for matrix-path convolutions
+    int precision_ = PREC_FP32;   // operand type of the matrix-path convolutions (reduced-precision modes: PREC_BF16, PREC_FP16)
     bool share_cost_rule_ = true;   // share classes weigh time by the held share of the device (false: hard footprint budgets)
     int share_threads_per_cu_ = 1024;   // resident threads per compute unit the share-class budgets assume (four wavefronts per SIMD)
     void load_tune_cache();

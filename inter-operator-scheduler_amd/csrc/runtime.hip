@@ -113,7 +113,9 @@ void DeviceContext::load_tune_cache() {
         std::ostringstream os;
         for (int i = 0; i < 12; i++) os << (i ? " " : "") << v[i];
         os << ' ' << token;
-        if (conv_variant(entry.best[0].variant).bf16) os << " bf16";   // reduced-precision entries have their own keys
+        // reduced-precision entries have their own keys
+        if (conv_variant(entry.best[0].variant).precision == PREC_BF16) os << " bf16";
+        if (conv_variant(entry.best[0].variant).precision == PREC_FP16) os << " fp16";
         tuned[os.str()] = entry;
     }
     fclose(f);
@@ -200,7 +202,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     float fastest = 1e30f;
     for (int v = 0; v < conv_num_variants(); v++) {
         const ConvVariant &cv = conv_variant(v);
-        if (cv.bf16 != bf16_) continue;   // the precision mode decides which family of configurations competes
+        if (cv.precision != precision_) continue;   // the precision mode decides which family of configurations competes
         // tiles more than twice as tall / wide as the problem only waste lanes
         if (cv.BM >= 2 * p.OCg() + 32 || cv.BN >= 2 * p.Npix() + 32) continue;
         int last_effective = -1;
@@ -271,7 +273,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
                 }
             }
         }
-        if (!found[c]) result.best[c] = conv_pick_launch(p, std::max(1, num_cus_ >> c), c > 0, bf16_);
+        if (!found[c]) result.best[c] = conv_pick_launch(p, std::max(1, num_cus_ >> c), c > 0, precision_);
     }
     if (!tune_cache_path_.empty()) {
         FILE *f = fopen(tune_cache_path_.c_str(), "a");
@@ -291,7 +293,7 @@ ConvLaunch DeviceContext::choose_launch(const ConvProblem &p, int share, bool al
     ConvLaunch launch;
     bool chosen = false;
     if (autotune_) {
-        const std::string key = conv_signature(p) + " " + settings_token() + (bf16_ ? " bf16" : "");
+        const std::string key = conv_signature(p) + " " + settings_token() + (precision_ == PREC_BF16 ? " bf16" : precision_ == PREC_FP16 ? " fp16" : "");
         auto it = tuned.find(key);
         if (it == tuned.end() && allow_tuning) it = tuned.emplace(key, tune_conv(p)).first;
         if (it != tuned.end()) {
@@ -300,7 +302,7 @@ ConvLaunch DeviceContext::choose_launch(const ConvProblem &p, int share, bool al
         }
     }
     if (!chosen) {
-        launch = conv_pick_launch(p, std::max(1, num_cus_ >> cls), cls > 0, bf16_);
+        launch = conv_pick_launch(p, std::max(1, num_cus_ >> cls), cls > 0, precision_);
     }
     if (forced_variant_ >= 0) launch.variant = forced_variant_;
     if (forced_split_k_ > 0) launch.split_k = forced_split_k_;
@@ -362,9 +364,10 @@ void DeviceContext::set_option(const std::string &key, const std::string &value)
         if (v < 64 || v > 4096) throw std::runtime_error("option share_threads_per_cu: expected 64..4096");
         share_threads_per_cu_ = v;
     } else if (key == "precision") {
-        if (value == "fp32") bf16_ = false;
-        else if (value == "bf16") bf16_ = true;
-        else throw std::runtime_error("option precision: expected fp32 or bf16, got '" + value + "'");
+        if (value == "fp32") precision_ = PREC_FP32;
+        else if (value == "bf16") precision_ = PREC_BF16;
+        else if (value == "fp16") precision_ = PREC_FP16;
+        else throw std::runtime_error("option precision: expected fp32, bf16 or fp16, got '" + value + "'");
     } else if (key == "split_k_reduce") {
         if (value == "inline") inline_reduce_ = true;
         else if (value == "kernel") inline_reduce_ = false;
@@ -381,7 +384,7 @@ std::string DeviceContext::info_json() const {
     os << "{\"name\":\"" << name_ << "\",\"arch\":\"" << arch_ << "\",\"compute_units\":" << num_cus_
        << ",\"executor\":\"" << (exec_mode_ == ExecMode::Graph ? "graph" : exec_mode_ == ExecMode::Fused ? "fused" : exec_mode_ == ExecMode::FusedGraph ? "fused_graph" : "streams") << "\",\"autotune\":" << (autotune_ ? "true" : "false")
        << ",\"split_k_reduce\":\"" << (inline_reduce_ ? "inline" : "kernel") << "\""
-       << ",\"precision\":\"" << (bf16_ ? "bf16" : "fp32") << "\""
+       << ",\"precision\":\"" << (precision_ == PREC_BF16 ? "bf16" : precision_ == PREC_FP16 ? "fp16" : "fp32") << "\""
        << ",\"arena_reuse\":" << (planner_arena_reuse() ? "true" : "false")
        << ",\"max_groups\":" << kMaxGroups << ",\"conv_variants\":[";
     for (int i = 0; i < conv_num_variants(); i++) os << (i ? "," : "") << '"' << conv_variant(i).name << '"';

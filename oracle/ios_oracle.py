@@ -74,12 +74,17 @@ def to_bf16(t):
     return t.to(torch.bfloat16).to(torch.float32)
 
 
-def eval_node(config, outputs, weights: Weights, bf16_convs=frozenset()):
+def to_fp16(t):
+    """Round to IEEE half (nearest even, overflow to infinity) and back: the operand view of the precision=fp16 mode."""
+    return t.to(torch.float16).to(torch.float32)
+
+
+def eval_node(config, outputs, weights: Weights, bf16_convs=frozenset(), fp16_convs=frozenset()):
     kind = config['type']
     if kind == 'sequential':
         out = None
         for child in config['nodes']:
-            out = eval_node(child, outputs, weights, bf16_convs)
+            out = eval_node(child, outputs, weights, bf16_convs, fp16_convs)
             outputs[child['name']] = out
         return out
     x = gather_input(config['inputs'], outputs, multiply=(kind == 'element' and config['op_type'] == 'mul'))
@@ -88,6 +93,8 @@ def eval_node(config, outputs, weights: Weights, bf16_convs=frozenset()):
         w = torch.from_numpy(np.ascontiguousarray(w, dtype=np.float32))
         if config['name'] in bf16_convs:   # bfloat16 operands, fp32 accumulation
             x, w = to_bf16(x), to_bf16(w)
+        elif config['name'] in fp16_convs:   # half operands, fp32 accumulation
+            x, w = to_fp16(x), to_fp16(w)
         return conv2d(x, w,
                       torch.from_numpy(np.ascontiguousarray(b, dtype=np.float32)),
                       config['stride'], config['padding'], config['groups'], config['act'])
@@ -103,11 +110,12 @@ def eval_node(config, outputs, weights: Weights, bf16_convs=frozenset()):
 
 
 def run_graph(graph_config: dict, weights: Weights, x: np.ndarray, keep_all=False, num_threads: Optional[int] = None,
-              bf16_convs=frozenset()):
+              bf16_convs=frozenset(), fp16_convs=frozenset()):
     """
     Evaluate an exported graph on input ``x`` (batch, C, H, W).  Returns the exit operator's output as a
     float32 array, or a dict name -> array of every operator when ``keep_all``.  Convolutions named in
-    ``bf16_convs`` see their input and filters rounded to bfloat16 (the runtime's reduced-precision mode).
+    ``bf16_convs`` / ``fp16_convs`` see their input and filters rounded to bfloat16 / IEEE half (the runtime's
+    reduced-precision modes).
     """
     if num_threads is not None:
         torch.set_num_threads(num_threads)
@@ -116,7 +124,7 @@ def run_graph(graph_config: dict, weights: Weights, x: np.ndarray, keep_all=Fals
     with torch.no_grad():
         for block in graph_config['blocks']:
             for config in block['inner_nodes'] + [block['exit_node']]:
-                outputs[config['name']] = eval_node(config, outputs, weights, bf16_convs)
+                outputs[config['name']] = eval_node(config, outputs, weights, bf16_convs, fp16_convs)
                 last = config['name']
     if keep_all:
         return {name: t.numpy() for name, t in outputs.items()}
@@ -128,6 +136,6 @@ def graph_weights(graph) -> Weights:
     return {conv.name: (conv.weight, conv.bias) for conv in graph.conv_nodes()}
 
 
-def run(graph, x: np.ndarray, keep_all=False, num_threads=None, bf16_convs=frozenset()):
+def run(graph, x: np.ndarray, keep_all=False, num_threads=None, bf16_convs=frozenset(), fp16_convs=frozenset()):
     """Evaluate an ``ios.Graph`` object with the weights stored in its convolutions."""
-    return run_graph(graph.export_config(), graph_weights(graph), x, keep_all, num_threads, bf16_convs)
+    return run_graph(graph.export_config(), graph_weights(graph), x, keep_all, num_threads, bf16_convs, fp16_convs)

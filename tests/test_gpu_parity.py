@@ -684,29 +684,36 @@ def assert_close_reduced(got, want, what=''):
     assert err.max() <= 3e-2 * scale, f'{what}: max abs err {err.max():.3e} at scale {scale:.3e}'
 
 
+REDUCED = [('bf16', 'wb_', 'bf16_convs'), ('fp16', 'wh_', 'fp16_convs')]
+
+
+@pytest.mark.parametrize('mode', REDUCED, ids=[m[0] for m in REDUCED])
 @pytest.mark.parametrize('case', [c for c in CONVS if c[5] == 1])
-def test_reduced_precision_conv_matches_the_bfloat16_oracle(case):
-    """precision=bf16: bit-level agreement is not expected (summation order), but against an oracle that rounds the
-    same operands to bfloat16 the fp32 tolerance holds; against the fp32 oracle the error is that of the rounding."""
+def test_reduced_precision_conv_matches_the_rounding_oracle(case, mode):
+    """precision=bf16 / fp16: bit-level agreement is not expected (summation order), but against an oracle that rounds the
+    same operands to bfloat16 / half the fp32 tolerance holds; against the fp32 oracle the error is that of the rounding."""
+    precision, _, oracle_key = mode
     in_shape, oc, k, s, p, g, act, batch = case
     graph = single_op_graph(in_shape, lambda b, v: ios.conv2d(b, [[v]], oc, k, s, p, g, act, is_exit=True))
     x = np.random.default_rng(1).standard_normal((batch, *in_shape)).astype(np.float32)
-    rt.set_option('precision', 'bf16')
+    rt.set_option('precision', precision)
     convs = matrix_path_convs(graph, batch)
     assert convs, 'expected a matrix-path convolution'
     got = rt.graph_inference(graph, batch, x)
-    assert_close(got, ios_oracle.run(graph, x, bf16_convs=convs), f'bf16 conv {case}')
-    assert_close_reduced(got, ios_oracle.run(graph, x), f'bf16 conv {case} against fp32')
+    assert_close(got, ios_oracle.run(graph, x, **{oracle_key: convs}), f'{precision} conv {case}')
+    assert_close_reduced(got, ios_oracle.run(graph, x), f'{precision} conv {case} against fp32')
     rt.set_option('precision', 'fp32')
     assert not np.array_equal(got, rt.graph_inference(graph, batch, x))     # the mode really changes the arithmetic
 
 
-def test_every_reduced_precision_kernel_configuration():
+@pytest.mark.parametrize('mode', REDUCED, ids=[m[0] for m in REDUCED])
+def test_every_reduced_precision_kernel_configuration(mode):
+    precision, prefix, oracle_key = mode
     names = rt.device_info()['conv_variants']
-    rt.set_option('precision', 'bf16')
+    rt.set_option('precision', precision)
     tried = 0
     for index, name in enumerate(names):
-        if not name.startswith('wb_'):
+        if not name.startswith(prefix):
             continue
         tried += 1
         rt.set_option('conv_variant', index)
@@ -718,22 +725,24 @@ def test_every_reduced_precision_kernel_configuration():
                 graph = single_op_graph(in_shape, lambda b, v: ios.conv2d(b, [[v]], oc, k, s, p, 1, 'relu', is_exit=True))
                 x = np.random.default_rng(1).standard_normal((batch, *in_shape)).astype(np.float32)
                 got = rt.graph_inference(graph, batch, x)
-                want = ios_oracle.run(graph, x, bf16_convs=matrix_path_convs(graph, batch))
+                want = ios_oracle.run(graph, x, **{oracle_key: matrix_path_convs(graph, batch)})
                 assert_close(got, want, f'{name} split {split} conv {in_shape}->{oc} {k}')
                 np.testing.assert_array_equal(got, rt.graph_inference(graph, batch, x))
-    assert tried >= 5
+    assert tried >= 10
 
 
-def test_reduced_precision_network_under_parallel_schedules():
+@pytest.mark.parametrize('mode', REDUCED, ids=[m[0] for m in REDUCED])
+def test_reduced_precision_network_under_parallel_schedules(mode):
+    precision, _, oracle_key = mode
     graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias')
     graph.sequential_schedule()
     greedy = ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias')
     greedy.greedy_schedule(8)
     x = np.random.default_rng(1).standard_normal((2, *graph.enter_node.output_shape)).astype(np.float32)
-    rt.set_option('precision', 'bf16')
+    rt.set_option('precision', precision)
     convs = matrix_path_convs(graph, 2)
     assert len(convs) == 94
-    want = ios_oracle.run(graph, x, bf16_convs=convs)
+    want = ios_oracle.run(graph, x, **{oracle_key: convs})
     want_fp32 = ios_oracle.run(graph, x)
     for executor, g in (('streams', graph), ('fused', greedy), ('fused_graph', greedy)):
         rt.set_option('executor', executor)
@@ -743,10 +752,10 @@ def test_reduced_precision_network_under_parallel_schedules():
             for _ in range(2):
                 session.run()
             got = session.output()
-        # 94 layers deep, a different rounding of one operand (summation order before it) can flip a bfloat16 rounding
-        # downstream: the bfloat16 oracle is matched at the rounding tolerance, a little tighter than the fp32 one
-        assert_close_reduced(got, want, f'bf16 inception {executor}')
-        assert_close_reduced(got, want_fp32, f'bf16 inception {executor} against fp32')
+        # 94 layers deep, a different rounding of one operand (summation order before it) can flip a 16-bit rounding
+        # downstream: the rounding oracle is matched at the rounding tolerance, a little tighter than the fp32 one
+        assert_close_reduced(got, want, f'{precision} inception {executor}')
+        assert_close_reduced(got, want_fp32, f'{precision} inception {executor} against fp32')
         assert np.abs(got - want).max() <= np.abs(got - want_fp32).max() * 1.5 + 1e-4
 
 

@@ -208,6 +208,39 @@ def test_bf16_rounding_is_round_to_nearest_even():
     np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+def test_fp16_rounding_is_ieee_half_round_to_nearest_even():
+    """The oracle's half view of an operand against numpy's float16 (an independent implementation) and known cases."""
+    import torch
+    rng = np.random.default_rng(12)
+    x = np.concatenate([rng.standard_normal(4096).astype(np.float32) * 10.0 ** rng.integers(-9, 6, 4096),
+                        np.array([0.0, -0.0, 1.0, 1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 65504.0, 65519.9, 65520.0, -1e6, 6e-8, 2.9e-8],
+                                 dtype=np.float32)]).astype(np.float32)
+    got = ios_oracle.to_fp16(torch.from_numpy(x)).numpy()
+    with np.errstate(over='ignore'):
+        want = x.astype(np.float16).astype(np.float32)
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    known = ios_oracle.to_fp16(torch.tensor([1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 65519.9, 65520.0, 2.9e-8])).numpy()
+    # ties go to the even mantissa; 65520 is the first value that rounds to infinity; below half the smallest subnormal: zero
+    np.testing.assert_array_equal(known, np.array([1.0, 1.0 + 2.0 ** -9, 65504.0, np.inf, 0.0], dtype=np.float32))
+    # a convolution named in fp16_convs sees exactly those operands
+    import ios
+    ios.reset_name()
+    v = ios.placeholder((4, 5, 5))
+    block = ios.Block(v.node)
+    ios.conv2d(block, [[v]], 6, (3, 3), (1, 1), (1, 1), 1, 'identity', is_exit=True)
+    graph = ios.Graph('h', v.node, [block])
+    graph.init_weights(seed=3, scheme='he_normal_bias')
+    conv = graph.conv_nodes()[0]
+    xin = rng.standard_normal((2, 4, 5, 5)).astype(np.float32)
+    got = ios_oracle.run(graph, xin, fp16_convs={conv.name})
+    rounded = ios.Graph.from_config(graph.export_config())
+    rounded.conv_nodes()[0].weight = conv.weight.astype(np.float16).astype(np.float32)
+    rounded.conv_nodes()[0].bias = conv.bias
+    want = ios_oracle.run(rounded, xin.astype(np.float16).astype(np.float32))
+    np.testing.assert_array_equal(got, want)
+    assert not np.array_equal(got, ios_oracle.run(graph, xin))
+
+
 def _golden_vectors():
     import os
     import sys
