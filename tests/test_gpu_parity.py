@@ -120,7 +120,7 @@ def test_committed_operator_vectors():
 
 
 # every fp32 kernel configuration the library was built with (host-only query; the bfloat16 ones have their own test)
-FP32_VARIANTS = [name for name in rt.conv_variant_names() if not name.startswith('wb_')]
+FP32_VARIANTS = [name for name in rt.conv_variant_names() if not name.startswith(('wb_', 'wh_'))]
 
 
 @pytest.mark.parametrize('variant_name', FP32_VARIANTS)
