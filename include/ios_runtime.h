@@ -118,7 +118,12 @@ void ios_session_destroy(ios_session *session);
 int ios_session_set_conv_weights(ios_session *session, int num_convs, char **conv_names, float **filter_data,
                                  float **bias_data);
 int ios_session_set_input(ios_session *session, const float *input);
-int ios_session_run(ios_session *session);
+int ios_session_run(ios_session *session);                                  /* one forward pass, waits for it */
+/* One forward pass queued behind the earlier ones without waiting, and the wait for everything queued: K passes
+ * between two synchronisations run back to back on the device, as the reference's timers see them
+ * (src/ios/ios_runtime.cu:1423-1440 takes its events around the device work of a pass). */
+int ios_session_enqueue(ios_session *session);
+int ios_session_synchronize(ios_session *session);
 int ios_session_get_output(ios_session *session, float *output);
 /* Dense copy of any operator's output (batch x C x H x W) after a run. */
 int ios_session_get_tensor(ios_session *session, const char *node_name, float *output);

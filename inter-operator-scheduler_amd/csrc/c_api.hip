@@ -211,6 +211,14 @@ int ios_session_run(ios_session *s) {
     return guarded([&]() { unbox(s).run(); });
 }
 
+int ios_session_enqueue(ios_session *s) {
+    return guarded([&]() { unbox(s).forward(); });
+}
+
+int ios_session_synchronize(ios_session *s) {
+    return guarded([&]() { unbox(s).synchronize(); });
+}
+
 int ios_session_get_output(ios_session *s, float *output) {
     return guarded([&]() { unbox(s).get_output(output); });
 }

@@ -118,6 +118,8 @@ public:
     void get_tensor(const std::string &name, float *host);
 
     void run();   // one forward pass, synchronised
+    void forward();       // one forward pass queued without waiting (stream launches or graph replay, by the execution mode)
+    void synchronize();   // waits for everything queued
     // reference timing protocol for graphs / blocks: per repeat the mean of `number` individually
     // bracketed forward passes; optional per-stage times from events recorded after every stage
     void measure(int warmup, int number, int repeat, bool profile_stage, float *results, float *stage_results);
@@ -149,7 +151,6 @@ private:
     void enqueue_fused(bool stage_events);
     void enqueue_serial();
     void build_fused();
-    void forward();                    // enqueue or graph launch according to the execution mode
     void build_graph();
     void copy_out(const ViewRef &view, float *host);
     TensorView tv(const ViewRef &v) const;

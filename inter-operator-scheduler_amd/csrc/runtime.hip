@@ -854,8 +854,10 @@ void Session::forward() {
 
 void Session::run() {
     forward();
-    IOS_HIP(hipStreamSynchronize(ctx_.stream(0)));
+    synchronize();
 }
+
+void Session::synchronize() { IOS_HIP(hipStreamSynchronize(ctx_.stream(0))); }
 
 void Session::measure(int warmup, int number, int repeat, bool profile_stage, float *results, float *stage_results) {
     if (static_) throw std::runtime_error("a session in the static scratch has no timers");

@@ -69,6 +69,8 @@ def _declare(handle):
                                                     ctypes.POINTER(vp)]
     handle.ios_session_set_input.argtypes = [vp, vp]
     handle.ios_session_run.argtypes = [vp]
+    handle.ios_session_enqueue.argtypes = [vp]
+    handle.ios_session_synchronize.argtypes = [vp]
     handle.ios_session_get_output.argtypes = [vp, vp]
     handle.ios_session_get_tensor.argtypes = [vp, s, vp]
     handle.ios_session_measure.argtypes = [vp, i, i, i, i, f32p, f32p]
@@ -78,7 +80,7 @@ def _declare(handle):
     handle.ios_session_describe_launches.argtypes = [vp, ctypes.c_char_p, i]
     handle.ios_session_profile_launches.argtypes = [vp, i, i, f32p, i]
     for name in ('ios_session_set_conv_weights', 'ios_session_set_input', 'ios_session_run',
-                 'ios_session_get_output', 'ios_session_get_tensor', 'ios_session_measure',
+                 'ios_session_get_output', 'ios_session_get_tensor', 'ios_session_measure', 'ios_session_enqueue', 'ios_session_synchronize',
                  'ios_session_num_ops', 'ios_session_describe', 'ios_session_profile_ops',
                  'ios_session_describe_launches', 'ios_session_profile_launches'):
         getattr(handle, name).restype = i
@@ -286,6 +288,13 @@ class Session:
 
     def run(self):
         _check(self._lib.ios_session_run(self._handle), 'ios_session_run')
+
+    def enqueue(self):
+        """Queue one forward pass behind the earlier ones without waiting (see ``synchronize``)."""
+        _check(self._lib.ios_session_enqueue(self._handle), 'ios_session_enqueue')
+
+    def synchronize(self):
+        _check(self._lib.ios_session_synchronize(self._handle), 'ios_session_synchronize')
 
     def output(self) -> np.ndarray:
         out = np.empty(self.output_shape, dtype=np.float32)

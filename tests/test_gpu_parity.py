@@ -464,6 +464,24 @@ def test_depthwise_sums_share_fused_launches_with_other_operators():
             np.testing.assert_array_equal(outs[executor], outs['streams'])
 
 
+def test_passes_queued_back_to_back_give_the_result_of_a_single_pass():
+    graph = ios.models.squeezenet_1_1(init_seed=0, init_scheme='he_normal_bias')
+    graph.greedy_schedule(8)
+    x = np.random.default_rng(3).standard_normal((2, *graph.enter_node.output_shape)).astype(np.float32)
+    for executor in ('streams', 'fused', 'fused_graph'):
+        rt.set_option('executor', executor)
+        with rt.Session(graph, 2) as session:
+            session.load_weights()
+            session.set_input(x)
+            session.run()
+            single = session.output()
+            for _ in range(7):
+                session.enqueue()
+            session.synchronize()
+            np.testing.assert_array_equal(session.output(), single)
+    assert_close(single, ios_oracle.run(graph, x), 'squeezenet batch 2')
+
+
 def model_cases():
     # (id, constructor, batch, strict tolerance).  Seeded non-zero biases everywhere; RandWire in the folded-batch-norm
     # form its configuration describes; NASNet both under the He-normal initialisation its configuration names (scaled
