@@ -10,7 +10,7 @@ namespace ios {
 
 __global__ void pool_kernel(PoolArgs a) { pool_body(a, blockIdx.x, gridDim.x); }
 __global__ void global_pool_kernel(PoolArgs a) { global_pool_body(a, blockIdx.x, gridDim.x); }
-__global__ void dwconv_kernel(DirectConvArgs a) { dwconv_dispatch<true>(a, blockIdx.x, gridDim.x); }
+__global__ void dwconv_kernel(DirectConvArgs a) { dwconv_dispatch(a, blockIdx.x, gridDim.x); }
 __global__ void conv_direct_kernel(DirectConvArgs a) { conv_direct_body(a, blockIdx.x, gridDim.x); }
 __global__ __launch_bounds__(256) void conv_thin_kernel(DirectConvArgs a) {
     __shared__ float filters[kThinConvSmemFloats];

@@ -360,16 +360,11 @@ __device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, 
     }
 }
 
-// WITH_SUM: the caller may hold launches that add further inputs in the loader (their 5 x 5 form needs more registers than
-// the fused stage kernel of the matrix-path convolutions grants, so that kernel is built without them)
-template <bool WITH_SUM = true>
 __device__ __forceinline__ void dwconv_dispatch(const DirectConvArgs &a, int block, int num_blocks) {
     const ConvProblem &p = a.p;
     if (a.nmore > 0) {   // the host only builds such launches for 3 x 3 and 5 x 5 windows
-        if constexpr (WITH_SUM) {
-            if (p.KH == 3) dwconv_body<3, 3, true>(a, block, num_blocks);
-            else dwconv_body<5, 5, true>(a, block, num_blocks);
-        }
+        if (p.KH == 3) dwconv_body<3, 3, true>(a, block, num_blocks);
+        else dwconv_body<5, 5, true>(a, block, num_blocks);
         return;
     }
     if (p.KH == 3 && p.KW == 3) dwconv_body<3, 3>(a, block, num_blocks);
