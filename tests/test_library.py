@@ -266,3 +266,25 @@ def test_arena_reuse_never_lets_an_operator_read_what_another_overwrote(name, ba
     for op in shared:
         for begin, stop in op['writes']:
             assert all(e <= begin or stop <= b for b, e in first_reads), op['node']
+
+
+def test_planner_options_need_no_device_and_change_the_plan():
+    graph = ios.models.inception_v3()
+    graph.sequential_schedule()
+    try:
+        first = rt.plan_describe(graph, 16)[0]
+        assert first['kind'] == 'conv_direct' and first['thin'] is True      # 16 x 149 x 149 output pixels: the first-layer kernel
+        assert rt.plan_describe(graph, 1)[0]['kind'] == 'conv_mfma'           # batch 1: the matrix path
+        rt.set_option('thin_conv_min_pixels', -1)
+        assert rt.plan_describe(graph, 16)[0]['kind'] == 'conv_mfma'
+        rt.set_option('thin_conv_min_pixels', 0)
+        assert rt.plan_describe(graph, 1)[0]['kind'] == 'conv_direct'
+        # only 3 x 3 convolutions of 3-channel inputs qualify
+        assert sum(op['kind'] == 'conv_direct' for op in rt.plan_describe(graph, 1)) == 1
+        rt.set_option('arena_reuse', 0)
+        plain = rt.plan_arena_bytes(graph, 16)
+        rt.set_option('arena_reuse', 1)
+        assert rt.plan_arena_bytes(graph, 16) < plain
+    finally:
+        rt.set_option('thin_conv_min_pixels', 1 << 18)
+        rt.set_option('arena_reuse', 1)
