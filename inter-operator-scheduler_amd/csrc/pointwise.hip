@@ -45,12 +45,13 @@ PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorV
         while (rows > 1 && (long long)p.B * p.C * ((p.OH + rows - 1) / rows) * p.OW < (1LL << 20)) rows >>= 1;
         a.strip_rows = rows;
         long long threads = (long long)p.B * p.C * ((p.OH + rows - 1) / rows) * p.OW;
-        // large tensors: four output columns per thread (16-byte loads and stores) while that leaves half a million threads
+        // larger tensors: four output columns per thread (16-byte loads and stores) while that leaves 65536 threads
         if ((p.sw == 1 || p.sw == 2) && p.pw <= 1 && p.W >= 8) {
+            const long long kVecMinThreads = 1LL << 16;   // measured: 2^16 beats the one-column form from 64x147x147 at batch 1 on, 2^14 loses
             auto quads = [&](int r) { return (long long)p.B * p.C * ((p.OH + r - 1) / r) * ((p.OW + kPoolVecColumns - 1) / kPoolVecColumns); };
             int vrows = kPoolStripRows;
-            while (vrows > 1 && quads(vrows) < (1LL << 19)) vrows >>= 1;
-            if (quads(vrows) >= (1LL << 19)) {
+            while (vrows > 1 && quads(vrows) < kVecMinThreads) vrows >>= 1;
+            if (quads(vrows) >= kVecMinThreads) {
                 a.vec_columns = kPoolVecColumns;
                 a.strip_rows = vrows;
                 threads = quads(vrows);

@@ -121,7 +121,7 @@ __device__ __forceinline__ void pool3x3_body(const PoolArgs &a, int block, int n
     }
 }
 
-// The same strips, four output columns wide: the form for large tensors, where the load instructions per byte decide.  A
+// The same strips, four output columns wide: the form for all but small tensors, where the load instructions per byte decide.  A
 // thread reads an input row of its strip with one clamped scalar load and one (stride 1) or two (stride 2) 16-byte loads
 // at any 4-byte alignment instead of three loads per output column, and stores four outputs with one 16-byte store.  The
 // 16-byte loads may run up to eight elements past the end of a row; what they bring from there (the next row, the next
