@@ -3,7 +3,9 @@
 set -euo pipefail
 cd "$(dirname "$0")"
 mkdir -p build
-FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclang -packed-fp32-ops -mllvm -amdgpu-mfma-vgpr-form=1 -Wno-unused-result"
+# -amdgpu-kernarg-preload-count: the leading scalar kernel arguments arrive in registers (the fused stage kernel's item
+# starts), which takes one scalar-load round trip out of every fused launch
+FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclang -packed-fp32-ops -mllvm -amdgpu-mfma-vgpr-form=1 -mllvm -amdgpu-kernarg-preload-count=16 -Wno-unused-result"
 pids=()
 for src in conv_mfma.hip pointwise.hip fused.hip runtime.hip c_api.hip; do
     # the resource remarks go to a log: a kernel that spills registers to scratch memory is reported below

@@ -5,11 +5,20 @@
 
 namespace ios {
 
+// The first blocks of the items travel as scalar kernel arguments (b1 ... b7; item 0 starts at block 0): with
+// -amdgpu-kernarg-preload-count the command processor hands them to a wavefront in registers, so a block knows its item
+// without a load and its first load is the item itself.
 template <int T>
-__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fused_kernel(const WorkItem *__restrict__ items, FusedHeader header) {
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fused_kernel(const WorkItem *__restrict__ items, int num_items, int b1, int b2,
+                                                                                            int b3, int b4, int b5, int b6, int b7) {
     extern __shared__ floatx4 fused_smem[];
     float *smem = reinterpret_cast<float *>(fused_smem);
     const int bid = blockIdx.x;
+    FusedHeader header;
+    header.num_items = num_items;
+    header.first_block[0] = 0;
+    header.first_block[1] = b1; header.first_block[2] = b2; header.first_block[3] = b3; header.first_block[4] = b4;
+    header.first_block[5] = b5; header.first_block[6] = b6; header.first_block[7] = b7;
     int index = 0;   // number of further items that start at or before this block
     if (header.num_items <= kFusedHeaderItems) {
 #pragma unroll
@@ -91,10 +100,18 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fus
 void launch_fused(int threads, const WorkItem *device_items, const FusedHeader &header, int total_blocks, int smem_bytes, hipStream_t stream) {
     if (header.num_items < 1 || header.num_items > kMaxFusedItems || total_blocks < 1) throw std::runtime_error("fused launch: bad item count");
     const dim3 grid((unsigned)total_blocks);
+    static_assert(kFusedHeaderItems == 8, "the kernel takes seven first-block arguments");
+    const int *b = header.first_block;
     switch (threads) {
-        case 256: hipLaunchKernelGGL(fused_kernel<256>, grid, dim3(256), smem_bytes, stream, device_items, header); break;
-        case 512: hipLaunchKernelGGL(fused_kernel<512>, grid, dim3(512), smem_bytes, stream, device_items, header); break;
-        case 1024: hipLaunchKernelGGL(fused_kernel<1024>, grid, dim3(1024), smem_bytes, stream, device_items, header); break;
+        case 256:
+            hipLaunchKernelGGL(fused_kernel<256>, grid, dim3(256), smem_bytes, stream, device_items, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7]);
+            break;
+        case 512:
+            hipLaunchKernelGGL(fused_kernel<512>, grid, dim3(512), smem_bytes, stream, device_items, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7]);
+            break;
+        case 1024:
+            hipLaunchKernelGGL(fused_kernel<1024>, grid, dim3(1024), smem_bytes, stream, device_items, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7]);
+            break;
         default: throw std::runtime_error("fused launch: unsupported block size");
     }
 }
