@@ -27,6 +27,17 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fus
         while (index + 1 < header.num_items && bid >= items[index + 1].first_block) index++;
     }
     const WorkItem &item = items[index];
+    // An item spans five 64-byte lines of the scalar cache, and the bodies read its fields in two or three dependent steps
+    // (kind, then configuration, then arguments): one word of every line is requested together with the first step, so
+    // that the later steps find their lines in the cache instead of paying a miss each.  The comparison below never
+    // holds (first_block is not negative) and only keeps the compiler from dropping the loads.
+    {
+        const int *words = reinterpret_cast<const int *>(&item);
+        int touched = 0;
+#pragma unroll
+        for (int line = 1; line * 16 < (int)(sizeof(WorkItem) / sizeof(int)); line++) touched |= words[line * 16];
+        if (item.first_block == -1 && touched == 0x5a5a5a5a) return;
+    }
     const int local = bid - item.first_block;
     const int num_blocks = item.num_blocks;
     switch (item.kind) {
