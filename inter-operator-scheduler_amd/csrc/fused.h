@@ -19,6 +19,7 @@ struct WorkItem {
     int tiles, groups;             // convolution grid decomposition: block = (tile, group, K slice)
     int first_block, num_blocks;   // range of this item inside the fused grid
     int reserved;
+    FastDiv div_tiles, div_groups; // convolution: exact quotients by tiles and by groups without an integer division
     union {
         ConvKernelArgs conv;
         ReduceArgs reduce;
@@ -34,7 +35,7 @@ constexpr int kMaxFusedItems = 16;    // = groups per stage
 constexpr int kFusedHeaderItems = 8;  // the schedule search builds stages of up to 8 groups; wider stages walk the table
 struct FusedHeader {
     int num_items;
-    int first_block[kFusedHeaderItems];   // ascending; entries beyond num_items are unused
+    int first_block[kFusedHeaderItems];   // ascending; entries beyond num_items are INT_MAX (no block reaches them)
 };
 
 // Thread-block sizes the fused kernel is instantiated for.  A launch uses the size of its widest convolution body;

@@ -1,6 +1,7 @@
 // The fused stage kernel: see fused.h.
 #include "fused.h"
 
+#include <climits>
 #include <stdexcept>
 
 namespace ios {
@@ -22,7 +23,7 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fus
     int index = 0;   // number of further items that start at or before this block
     if (header.num_items <= kFusedHeaderItems) {
 #pragma unroll
-        for (int i = 1; i < kFusedHeaderItems; i++) index += (i < header.num_items && bid >= header.first_block[i]) ? 1 : 0;
+        for (int i = 1; i < kFusedHeaderItems; i++) index += bid >= header.first_block[i] ? 1 : 0;   // unused entries are INT_MAX
     } else {
         while (index + 1 < header.num_items && bid >= items[index + 1].first_block) index++;
     }
@@ -44,10 +45,10 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fus
         case WORK_CONV: {
             if ((int)threadIdx.x >= item.threads) return;   // surplus wavefronts of a narrower body
             const ConvKernelArgs &a = item.conv;   // fields are fetched with scalar loads where they are used
-            const int tile = local % item.tiles;
-            const int rest = local / item.tiles;
-            const int g = rest % item.groups;
-            const int z = rest / item.groups;
+            const int rest = (int)fast_div((unsigned)local, item.div_tiles);
+            const int tile = local - rest * item.tiles;
+            const int z = (int)fast_div((unsigned)rest, item.div_groups);
+            const int g = rest - z * item.groups;
             switch (item.variant) {
 #define IOS_CASE_TILED(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                          \
     case IDX:                                                                                              \
@@ -112,7 +113,8 @@ void launch_fused(int threads, const WorkItem *device_items, const FusedHeader &
     if (header.num_items < 1 || header.num_items > kMaxFusedItems || total_blocks < 1) throw std::runtime_error("fused launch: bad item count");
     const dim3 grid((unsigned)total_blocks);
     static_assert(kFusedHeaderItems == 8, "the kernel takes seven first-block arguments");
-    const int *b = header.first_block;
+    int b[kFusedHeaderItems];
+    for (int i = 0; i < kFusedHeaderItems; i++) b[i] = i < header.num_items ? header.first_block[i] : INT_MAX;
     switch (threads) {
         case 256:
             hipLaunchKernelGGL(fused_kernel<256>, grid, dim3(256), smem_bytes, stream, device_items, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7]);

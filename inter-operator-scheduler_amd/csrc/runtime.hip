@@ -682,6 +682,8 @@ void Session::build_fused() {
                         pend.item.variant = d.variant;
                         pend.item.tiles = d.tiles;
                         pend.item.groups = d.groups;
+                        pend.item.div_tiles = make_fast_div((unsigned)d.tiles);
+                        pend.item.div_groups = make_fast_div((unsigned)d.groups);
                         pend.item.num_blocks = d.tiles * d.groups * d.slices;
                         pend.item.conv = d.args;
                         pend.threads = d.threads;
