@@ -55,6 +55,7 @@ struct PNode {
     // holds them (the convolution itself, or the private ReLU in front of it, which is then applied after the sum)
     int sum_front = -1;
     bool sum_relu = false;
+    int combine_front = -1;        // activation that combines the values of this addition / product / sum itself
     int references = 0;            // number of input values that name this node
 };
 
@@ -241,7 +242,10 @@ private:
             n.type = NodeType::Pool;
             n.C = C;
             const std::string pool_type = cfg["pool_type"].as_string();
-            if (pool_type != "max" && pool_type != "avg" && pool_type != "global_max" && pool_type != "global_avg")
+            // the reference only looks for the substrings "max" and "global" and takes everything else for an average
+            // (src/ios/ios_runtime.cu:1047-1051; its AlexNet writes 'max_pool'); a name with neither "max" nor "avg" is
+            // refused here instead of silently averaging
+            if (pool_type.find("max") == std::string::npos && pool_type.find("avg") == std::string::npos)
                 throw std::runtime_error("pool '" + name + "': unknown pool_type '" + pool_type + "'");
             if (pool_type.find("global") != std::string::npos) {
                 n.H = 1;
@@ -309,6 +313,7 @@ private:
             }
         }
         find_depthwise_sums();
+        find_activated_combinations();
         for (PNode &n : nodes_) {
             if (n.type == NodeType::Identity && single_value(n)) {
                 n.parent = n.inputs[0][0].node;
@@ -386,6 +391,24 @@ private:
                     r.parent = -1;
                 }
             }
+        }
+    }
+
+    // An activation whose only input is the whole output of an addition, a product or a sum of values that nobody else
+    // reads (the residual unit "add, then ReLU" of reference python/ios/models/resnet.py:25-26): the activation's launch
+    // combines the values itself, so the combining launch and its tensor disappear (the reference runs both,
+    // src/ios/ios_runtime.cu:854-908,939-1010).
+    void find_activated_combinations() {
+        for (PNode &a : nodes_) {
+            if ((a.type != NodeType::Relu && a.type != NodeType::Activation) || !single_value(a) || a.pre_relu_alias || a.no_storage)
+                continue;
+            const Val &v = a.inputs[0][0];
+            PNode &e = nodes_[v.node];
+            const bool combines = e.type == NodeType::Element || (e.type == NodeType::Identity && e.inputs.size() == 1 && e.inputs[0].size() >= 2);
+            if (!combines || e.inputs.size() != 1 || e.inputs[0].size() > (size_t)kMaxNaryInputs) continue;
+            if (e.references != 1 || e.no_storage || v.begin != 0 || v.end != e.C) continue;
+            a.combine_front = v.node;
+            e.no_storage = true;
         }
     }
 
@@ -633,6 +656,12 @@ private:
     void emit_terms(const PNode &n, int index, int act, bool multiply) {
         const ViewRef out = view_of(index);
         int offset = 0;
+        if (n.combine_front >= 0) {
+            const PNode &front = nodes_[n.combine_front];
+            const bool product = front.type == NodeType::Element && (*front.cfg)["op_type"].as_string() == "mul";
+            materialise_term(n, front.inputs[0], out, act, product);
+            return;
+        }
         for (const auto &term : n.inputs) {
             const int len = term[0].end - term[0].begin;
             bool in_place = false;

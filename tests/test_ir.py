@@ -142,6 +142,44 @@ def test_model_output_shapes():
     assert sum(len(p) for p in nm.blocks[0].parts) == len(nm.blocks[0].inner_nodes) + 1
 
 
+def test_chain_and_residual_networks_of_the_zoo():
+    """
+    AlexNet, VGG and ResNet as the reference builds them (python/ios/models/{alexnet,vgg,resnet}.py): operator counts and
+    exit shapes, and the multiply-accumulate / parameter counts of the convolutions, which are the published figures of
+    these architectures (VGG-16 15.35 GMAC and 14.71 M, VGG-19 19.51 GMAC, ResNet-18 1.81 GMAC and 11.17 M, ResNet-34 3.66
+    GMAC, ResNet-50 with the stride on the first 1x1 convolution 3.86 GMAC and 23.45 M; all without classifier layers).
+    """
+    expect = {   # name: (operators incl. placeholder, blocks, exit shape, GMAC, M parameters)
+        'alexnet': (8, 1, (256, 8, 8), 0.5329, 2.469),
+        'vgg_11': (15, 1, (512, 1, 1), 7.4855, 9.218),
+        'vgg_13': (17, 1, (512, 1, 1), 11.1848, 9.402),
+        'vgg_16': (20, 1, (512, 1, 1), 15.3466, 14.710),
+        'vgg_19': (23, 1, (512, 1, 1), 19.5084, 20.019),
+        'resnet18': (30, 5, (512, 7, 7), 1.8136, 11.167),
+        'resnet34': (54, 5, (512, 7, 7), 3.6632, 21.268),
+        'resnet50': (87, 5, (2048, 7, 7), 3.8559, 23.455),
+    }
+    for name, (count, blocks, exit_shape, gmac, mparam) in expect.items():
+        graph = getattr(ios.models, name)()
+        nodes = list(graph.nodes())
+        assert [n.name for n in nodes] == [str(i) for i in range(count)], name
+        assert len(graph.blocks) == blocks and tuple(graph.exit_node.output_shape) == exit_shape, name
+        macs = sum(np.prod(c.output_shape) * c.fan_in for c in graph.conv_nodes())
+        params = sum(np.prod(c.weight_shape) for c in graph.conv_nodes())
+        assert macs / 1e9 == pytest.approx(gmac, abs=1e-4) and params / 1e6 == pytest.approx(mparam, abs=1e-3), name
+        config = json.loads(json.dumps(graph.export_config()))
+        assert json.loads(json.dumps(Graph.from_config(config).export_config())) == config
+    r50 = {n.name: n for n in ios.models.resnet50().nodes()}
+    # first residual unit: projection of the block input beside 1x1 - 3x3 - 1x1, addition of the two, in-place ReLU
+    assert [r50[str(i)].type for i in range(3, 9)] == ['conv', 'conv', 'conv', 'conv', 'element', 'activation']
+    assert r50['3'].act == 'relu' and r50['6'].act == 'identity' and r50['7'].op_type == 'add' and r50['8'].inplace
+    assert [(v.node.name) for v in r50['7'].inputs[0]] == ['6', '3']
+    # a greedy schedule runs the projection beside the first convolution of the unit
+    graph = ios.models.resnet50()
+    graph.greedy_schedule(8)
+    assert graph.blocks[1].stages[0] == [['3'], ['4']]
+
+
 def test_randwire_graph_generator_is_seeded_and_valid():
     from ios.models.randwire import watts_strogatz_edges, read_graph, write_graph
     e1 = watts_strogatz_edges(32, 4, 0.75, seed=3)

@@ -55,8 +55,8 @@ def test_host_planner_fuses_concats_and_folds_relus():
     kinds = collections.Counter(op['kind'] for op in ops)
     assert kinds['conv_depthwise'] == 96 and kinds['conv_mfma'] == 99
     # a node's depth-wise convolution adds the node's predecessors (and applies the ReLU) in its loader: the only summing
-    # launches left are the stage outputs
-    assert kinds['nary'] == 3 and sum(kinds.values()) == 200
+    # launches left are the stage outputs, the last of them inside the ReLU that follows it
+    assert kinds['nary'] == 3 and kinds['unary'] == 0 and sum(kinds.values()) == 199
     depthwise = [op for op in ops if op['kind'] == 'conv_depthwise']
     assert max(op['inputs'] for op in depthwise) >= 5 and all(op['conv']['pre_relu'] for op in depthwise if op['inputs'] > 1)
     folded = [op for op in depthwise if op['inputs'] == 1 and op['conv']['pre_relu']]
@@ -241,7 +241,8 @@ def _simulate(ops):
 
 @pytest.mark.parametrize('name,batch,schedule', [('squeezenet_1_1', 2, 'sequential'), ('squeezenet_1_1', 1, 'greedy'),
                                                  ('randwire_small', 1, 'greedy'), ('nasnet_mobile', 1, 'greedy'),
-                                                 ('nasnet_mobile', 2, 'sequential'), ('inception_v3', 1, 'greedy')])
+                                                 ('nasnet_mobile', 2, 'sequential'), ('inception_v3', 1, 'greedy'),
+                                                 ('resnet50', 1, 'greedy'), ('resnet18', 2, 'sequential')])
 def test_arena_reuse_never_lets_an_operator_read_what_another_overwrote(name, batch, schedule):
     graph = getattr(ios.models, name)()
     if schedule == 'greedy':
@@ -266,6 +267,29 @@ def test_arena_reuse_never_lets_an_operator_read_what_another_overwrote(name, ba
     for op in shared:
         for begin, stop in op['writes']:
             assert all(e <= begin or stop <= b for b, e in first_reads), op['node']
+
+
+def test_residual_additions_join_the_activation_behind_them_and_pool_names_follow_the_reference():
+    # ResNet-50: 16 residual units end in addition + in-place ReLU (reference python/ios/models/resnet.py:25-26); the plan
+    # holds one launch per unit for both, applying the ReLU, and the addition has no tensor of its own
+    graph = ios.models.resnet50()
+    ops = rt.plan_describe(graph, 1)
+    kinds = [op['kind'] for op in ops]
+    assert kinds.count('conv_mfma') == 53 and kinds.count('nary') == 16 and kinds.count('unary') == 0 and kinds.count('pool') == 1
+    nodes = {n.name: n for n in graph.nodes()}
+    assert all(nodes[op['node']].type == 'activation' and op['act'] == 1 and len(op['reads']) == 2 for op in ops if op['kind'] == 'nary')
+    # ResNet-18 / 34 have no activation behind their additions: the addition itself is the launch
+    ops18 = rt.plan_describe(ios.models.resnet18(), 1)
+    assert sum(op['kind'] == 'nary' for op in ops18) == 8 and all(op['act'] == 0 for op in ops18 if op['kind'] == 'nary')
+    # pooling names: the reference looks for the substrings "max" and "global" (src/ios/ios_runtime.cu:1047-1051) and its
+    # AlexNet writes 'max_pool'
+    config = ios.models.alexnet().export_config()
+    plain = rt.plan_describe(ios.Graph.from_config(config), 1)
+    for node in config['blocks'][0]['inner_nodes']:
+        if node['type'] == 'pool':
+            node['pool_type'] = 'max_pool'
+    renamed = rt.plan_describe(ios.Graph.from_config(config), 1)
+    assert [(op['kind'], op['reads'], op['writes']) for op in renamed] == [(op['kind'], op['reads'], op['writes']) for op in plain]
 
 
 def test_planner_options_need_no_device_and_change_the_plan():
