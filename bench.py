@@ -485,8 +485,10 @@ def main():
             if search or not args.greedy_big:
                 rt.set_option('executor', args.search_executor)
                 t0 = time.time()
-                scheduled = ios.optimize(g, batch_size=1, opt_type='dp_parallel', compute_weight=True, warmup=2, number=6, repeat=3,
-                                         max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
+                # stages that are the same computation on the same shapes (NASNet's repeated cells) are measured once
+                shared = ios.IOSCostModel(share_identical_stages=True)
+                scheduled = ios.optimize(g, batch_size=1, cost_model=shared, opt_type='dp_parallel', compute_weight=True, warmup=2, number=6,
+                                         repeat=3, max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
                 search_c = time.time() - t0
                 label = 'dp_parallel'
                 rt.set_option('executor', args.executor)
@@ -512,10 +514,12 @@ def main():
         result['other_configs_batch1'] = configs
         if not args.no_extras:
             # the model variants the reference's own result table uses (its large RandWire / NASNet and SqueezeNet 1.0 with
-            # bypass), sequential and greedy schedules: points of comparison with that table, not part of the metric
+            # bypass) and the chains / residual networks of its zoo, sequential and greedy schedules: points of comparison
+            # with that table, not part of the metric
             variants = {}
             for name, make in (('squeezenet', ios.models.squeezenet), ('randwire_large', ios.models.randwire_large),
-                               ('nasnet_large', ios.models.nasnet_large)):
+                               ('nasnet_large', ios.models.nasnet_large), ('alexnet', ios.models.alexnet), ('vgg_16', ios.models.vgg_16),
+                               ('resnet18', ios.models.resnet18), ('resnet50', ios.models.resnet50)):
                 g = make(init_seed=0, init_scheme='he_normal')
                 g.sequential_schedule()
                 scheduled = make(init_seed=0, init_scheme='he_normal')

@@ -9,7 +9,7 @@ import pytest
 
 import ios
 from ios.cost_model import AnalyticCostModel, CostModel, RandomCostModel
-from ios.ir import Conv, Graph
+from ios.ir import Conv, Graph, Value
 from ios.optimizer import check_merge, graph_chain_decomposition, build_graph, optimize
 
 
@@ -167,6 +167,47 @@ def test_stage_measurements_are_memoised():
     optimize(graph, 1, cost, 'dp_parallel', debug_dp_info=info)
     assert cost.calls == len(info['stage_latency'])
     assert info['#operators'] == [5] and info['#states'][0] >= 5 and info['#schedules'][0] >= 1
+
+
+def test_identical_stages_share_one_measurement():
+    """
+    IOSCostModel(share_identical_stages=True): stages that are the same computation on the same shapes under different
+    operator names are measured once.  The device call is replaced by the additive model here, so the schedule must not
+    change; the signature must tell apart everything the runtime would see (shapes, kernels, slices, wiring).
+    """
+    from ios.cost_model import stage_signature
+
+    class Counting(ios.IOSCostModel):
+        def __init__(self, share):
+            super().__init__(share)
+            self.model = ios.AnalyticCostModel()
+
+        def _measure_stage(self, stage, batch_size, warmup, number, repeat, profile_stage):
+            return self.model.get_stage_latency(stage, batch_size, warmup, number, repeat)
+
+    found = []
+    for share in (False, True):
+        cost_model = Counting(share)
+        scheduled = ios.optimize(ios.models.inception_v3(), 1, cost_model, 'dp_parallel', max_num_groups=8, max_group_size=1)
+        found.append((cost_model.measured_stages, [block.stages for block in scheduled.blocks]))
+    assert found[0][1] == found[1][1]
+    assert found[1][0] < 0.7 * found[0][0]      # the two 160-wide 17x17 blocks and the last two 8x8 blocks repeat
+
+    graph = ios.models.inception_v3()
+    blocks = graph.blocks
+    # blocks 6 and 7 of the network (17x17, 160 channels inside) are the same cell: their first stages match
+    first = lambda block, count: [[node] for node in block.inner_nodes[:count]]
+    assert stage_signature(first(blocks[6], 3)) == stage_signature(first(blocks[7], 3))
+    assert stage_signature(first(blocks[5], 3)) != stage_signature(first(blocks[6], 3))      # 128 against 160 channels
+    # the order of groups and the wiring count
+    a, b = blocks[6].inner_nodes[0], blocks[6].inner_nodes[1]
+    assert stage_signature([[a], [b]]) != stage_signature([[a, b]])
+    ios.reset_name()
+    v = ios.placeholder((8, 6, 6))
+    block = ios.Block(v.node)
+    left = ios.conv2d(block, [[Value(v.node, 0, 4)]], 4)
+    right = ios.conv2d(block, [[Value(v.node, 4, 8)]], 4)
+    assert stage_signature([[left.node]]) != stage_signature([[right.node]])                # another slice of the input
 
 
 def test_check_merge_rules():
