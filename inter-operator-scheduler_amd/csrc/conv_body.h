@@ -81,7 +81,22 @@ struct ConvKernelArgs {
     int tile_div;        // tiles_n (weights_major) or tiles_m
     FastDiv div_tile;    // by tile_div
     FastDiv div_ohw, div_ow;
+    // residual form: y = res + act(conv + bias), then max(., 0) when post_relu; res is a dense view of the output's
+    // shape (batch stride res_bs elements), null for a plain convolution
+    const float *res;
+    int res_bs, post_relu;
 };
+
+// v = act(conv + bias) of output element (image b, channel, pixel r): adds the residual operand.  The residual form is a
+// compile-time property of a body (RES): the plain form, which every fused stage launch uses, carries no test for it.
+template <bool RES>
+__device__ __forceinline__ float add_residual(const ConvKernelArgs &a, float v, int b, int channel, int r) {
+    if constexpr (RES) {
+        v += a.res[(long long)b * a.res_bs + (long long)channel * a.OHW + r];
+        if (a.post_relu) v = fmaxf(v, 0.0f);
+    }
+    return v;
+}
 
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Tiles are renumbered so that an XCD
 // receives a contiguous range of them, and the range runs along the operand that is cheaper to duplicate: the
@@ -176,6 +191,7 @@ struct ConvTiled {
     static constexpr int SMEM_FLOATS = TILE_FLOATS > RED_FLOATS ? TILE_FLOATS : RED_FLOATS;
 
     // one block: output tile `tile` of group `g`, K slice `z`; smem holds SMEM_FLOATS floats, 16-byte aligned
+    template <bool RES = false>
     __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *smem, int tile, int g, int z) {
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / MT, TN = WTN / MT;
@@ -453,20 +469,23 @@ struct ConvTiled {
 #pragma unroll
                 for (int v = 0; v < M::ACC; v++) {
                     const int m = m0 + wm * WTM + i * MT + M::row(v, lane);
-                    if (m < a.OCg) yb[(long long)m * a.OHW] = apply_act(acc[i][j][v] + a.bias[g * a.OCg + m], a.act);
+                    if (m < a.OCg)
+                        yb[(long long)m * a.OHW] = add_residual<RES>(a, apply_act(acc[i][j][v] + a.bias[g * a.OCg + m], a.act), b, g * a.OCg + m, r);
                 }
         }
     }
     }   // run
 };
 
-// y[b][oc][r] = act(bias[oc] + sum_s ws[s][oc][n]),  n = b * OHW + r; slices are added in index order
+// y[b][oc][r] = act(bias[oc] + sum_s ws[s][oc][n]) (+ residual),  n = b * OHW + r; slices are added in index order
 struct ReduceArgs {
     const float *ws;
     const float *bias;
     float *y;
     int slices, OC, Npix, OHW, act;
     long long slice_floats, y_bs;
+    const float *res;      // residual operand as in ConvKernelArgs, or null
+    int res_bs, post_relu;
 };
 
 __device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int block, int num_blocks) {
@@ -478,7 +497,12 @@ __device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int bloc
         for (int s = 0; s < a.slices; s++) sum += a.ws[s * a.slice_floats + i];
         const int b = n / a.OHW;
         const int r = n - b * a.OHW;
-        a.y[b * a.y_bs + (long long)oc * a.OHW + r] = apply_act(sum + a.bias[oc], a.act);
+        float v = apply_act(sum + a.bias[oc], a.act);
+        if (a.res != nullptr) {
+            v += a.res[(long long)b * a.res_bs + (long long)oc * a.OHW + r];
+            if (a.post_relu) v = fmaxf(v, 0.0f);
+        }
+        a.y[b * a.y_bs + (long long)oc * a.OHW + r] = v;
     }
 }
 
@@ -520,6 +544,7 @@ struct ConvWsplit {
     static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
     static_assert(RP >= 0 && RP <= 2 && (RP == 0 || (QUAD && MT == 16 && U == 4)), "the 16-bit paths are the 16 x 16 x 16 form of the quad layout");
 
+    template <bool RES = false>
     __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *red, int tile, int g, int z) {
 
     const int tid = threadIdx.x;
@@ -824,7 +849,8 @@ struct ConvWsplit {
         if (m < a.OCg && nn < a.Npix) {
             const int b = (int)fast_div((unsigned)nn, a.div_ohw);
             const int r = nn - b * a.OHW;
-            a.y[(long long)b * a.y_bs + ((long long)g * a.OCg + m) * a.OHW + r] = apply_act(sum + bias_pre[t], a.act);
+            a.y[(long long)b * a.y_bs + ((long long)g * a.OCg + m) * a.OHW + r] =
+                add_residual<RES>(a, apply_act(sum + bias_pre[t], a.act), b, g * a.OCg + m, r);
         }
     }
 }   // run

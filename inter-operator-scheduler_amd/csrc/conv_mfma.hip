@@ -9,10 +9,11 @@
 namespace ios {
 
 // stand-alone kernel around a body: grid = (tiles, groups, K slices), dynamic LDS = Body::SMEM_FLOATS floats
-template <typename Body>
+// RES: the residual form of the epilogue (a.res is not null)
+template <typename Body, bool RES = false>
 __global__ __launch_bounds__(Body::THREADS) void conv_kernel(ConvKernelArgs a) {
     extern __shared__ floatx4 conv_smem[];
-    Body::run(a, reinterpret_cast<float *>(conv_smem), blockIdx.x, blockIdx.y, blockIdx.z);
+    Body::template run<RES>(a, reinterpret_cast<float *>(conv_smem), blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
 __global__ void splitk_reduce_kernel(ReduceArgs a) { splitk_reduce_body(a, blockIdx.x, gridDim.x); }
@@ -22,22 +23,25 @@ typedef void (*ConvKernelFn)(ConvKernelArgs);
 
 struct VariantEntry {
     ConvVariant v;
-    ConvKernelFn kernel;
+    ConvKernelFn kernel, kernel_residual;
     int smem_floats;
 };
 
 #define IOS_TILED_ENTRY(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                        \
     {{NAME, BM, BN, BK, WM, WN, WK, MT, false, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::CPAD, false, \
       ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::FUSABLE, false},    \
-     conv_kernel<ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>>, ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::SMEM_FLOATS},
+     conv_kernel<ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>>, conv_kernel<ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>, true>, \
+     ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::SMEM_FLOATS},
 #define IOS_WSPLIT_ENTRY(IDX, NAME, MT, TM, TN, NW, U, QUAD, D, BF16)                                                                  \
     {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::CPAD, QUAD, \
       ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::FUSABLE, BF16},      \
-     conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>>, ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::SMEM_FLOATS},
+     conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>>, conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>, true>,    \
+     ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::SMEM_FLOATS},
 #define IOS_WSPLIT_C4_ENTRY(IDX, NAME, MT, TM, TN, NW, U, QUAD, D, BF16)                                                                  \
     {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::CPAD, QUAD, \
       ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::FUSABLE, BF16},                                                                 \
-     conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>>, ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::SMEM_FLOATS},
+     conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>>, conv_kernel<ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>, true>,    \
+     ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::SMEM_FLOATS},
 
 static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)
                                              IOS_WSPLIT_C4_VARIANTS(IOS_WSPLIT_C4_ENTRY)
@@ -166,7 +170,8 @@ bool conv_matrix_path_supported(const ConvProblem &p) {
 }
 
 ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
-                                const float *bias, const TensorView &y, float *workspace, unsigned *counters) {
+                                const float *bias, const TensorView &y, float *workspace, unsigned *counters,
+                                const TensorView *residual, bool post_relu) {
     if (l.variant < 0 || l.variant >= kNumVariants) throw std::runtime_error("conv: bad variant");
     const VariantEntry &e = kVariants[l.variant];
     if (x.C != p.IC || x.H != p.H || x.W != p.W || y.C != p.OC || y.H != p.OH || y.W != p.OW)
@@ -215,6 +220,18 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     a.div_tile = make_fast_div((unsigned)a.tile_div);
     a.div_ohw = make_fast_div((unsigned)a.OHW);
     a.div_ow = make_fast_div((unsigned)a.OW);
+    a.res = nullptr;
+    a.res_bs = 0;
+    a.post_relu = post_relu ? 1 : 0;
+    if (residual != nullptr) {
+        if (residual->C != p.OC || residual->H != p.OH || residual->W != p.OW) throw std::runtime_error("conv: residual view does not match the output");
+        if ((unsigned long long)(p.B - 1) * residual->bstride + (unsigned long long)p.OC * p.OH * p.OW >= (1ull << 31))
+            throw std::runtime_error("conv: residual view too large");
+        a.res = residual->ptr;
+        a.res_bs = (int)residual->bstride;
+    } else if (post_relu) {
+        throw std::runtime_error("conv: activation after a residual that is not there");
+    }
     if (a.split_k > 1 && workspace == nullptr) throw std::runtime_error("conv: split-K launch without workspace");
     if (p.groups > 65535 || a.split_k > 65535) throw std::runtime_error("conv: grid too large");
     d.variant = l.variant;
@@ -238,17 +255,21 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
         r.act = p.act;
         r.slice_floats = (long long)p.OC * a.Npix;
         r.y_bs = y.bstride;
+        r.res = a.res;
+        r.res_bs = a.res_bs;
+        r.post_relu = a.post_relu;
         d.reduce_blocks = (int)std::min<long long>((r.slice_floats + 255) / 256, 4096);
     }
     return d;
 }
 
 void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
-                      const float *bias, const TensorView &y, float *workspace, unsigned *counters, hipStream_t stream) {
-    const ConvDispatch d = make_conv_dispatch(p, l, x, packed, bias, y, workspace, counters);
+                      const float *bias, const TensorView &y, float *workspace, unsigned *counters, hipStream_t stream,
+                      const TensorView *residual, bool post_relu) {
+    const ConvDispatch d = make_conv_dispatch(p, l, x, packed, bias, y, workspace, counters, residual, post_relu);
     const VariantEntry &e = kVariants[d.variant];
     const dim3 grid((unsigned)d.tiles, (unsigned)d.groups, (unsigned)d.slices);
-    hipLaunchKernelGGL(e.kernel, grid, dim3(d.threads), d.smem_bytes, stream, d.args);
+    hipLaunchKernelGGL(d.args.res != nullptr ? e.kernel_residual : e.kernel, grid, dim3(d.threads), d.smem_bytes, stream, d.args);
     if (d.has_reduce) hipLaunchKernelGGL(splitk_reduce_kernel, dim3(d.reduce_blocks), dim3(256), 0, stream, d.reduce);
 }
 

@@ -20,7 +20,7 @@ struct WorkItem {
     int first_block, num_blocks;   // range of this item inside the fused grid
     int reserved;
     FastDiv div_tiles, div_groups; // convolution: exact quotients by tiles and by groups without an integer division
-    union {
+    union {   // (a work item spans five 64-byte lines: the kernel requests one word of each with its first load)
         ConvKernelArgs conv;
         ReduceArgs reduce;
         PoolArgs pool;
@@ -31,6 +31,7 @@ struct WorkItem {
 
 // Passed by value with the launch: a block finds its item from the kernel-argument segment alone (one scalar load,
 // no walk through the item table), then reads the item's fields from the table.
+static_assert(sizeof(WorkItem) <= 320, "a work item spans at most five 64-byte lines");
 constexpr int kMaxFusedItems = 16;    // = groups per stage
 constexpr int kFusedHeaderItems = 8;  // the schedule search builds stages of up to 8 groups; wider stages walk the table
 struct FusedHeader {

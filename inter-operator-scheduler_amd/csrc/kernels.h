@@ -92,7 +92,8 @@ void launch_pack_filters(const ConvProblem &p, const ConvLaunch &l, const float 
 // finishes a tile last adds the slices inside the kernel; without counters a second kernel adds them on the
 // same stream.  Both forms add in slice order.
 void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
-                      const float *bias, const TensorView &y, float *workspace, unsigned *counters, hipStream_t stream);
+                      const float *bias, const TensorView &y, float *workspace, unsigned *counters, hipStream_t stream,
+                      const TensorView *residual = nullptr, bool post_relu = false);
 
 // Depth-wise convolution (groups == IC == OC), filters in their original [C][1][KH][KW] layout.  With `more`, the input is
 // x + more[0] + ... + more[nmore - 1] (at most kMaxNaryInputs views in all, added left to right before the folded ReLU).

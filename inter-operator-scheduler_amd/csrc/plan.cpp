@@ -56,6 +56,13 @@ struct PNode {
     int sum_front = -1;
     bool sum_relu = false;
     int combine_front = -1;        // activation that combines the values of this addition / product / sum itself
+    // Residual unit: a convolution whose only reader is an addition with one other value adds that value in its epilogue and
+    // writes the addition's tensor (or that of the ReLU absorbing the addition).  On the convolution: the node whose storage
+    // it writes, the other value and the ReLU; on that node: made_by_conv.
+    int residual_into = -1;
+    Val residual_other{-1, 0, 0};
+    bool residual_relu = false;
+    bool made_by_conv = false;
     int references = 0;            // number of input values that name this node
 };
 
@@ -102,6 +109,7 @@ public:
             if (!nodes_.empty() && nodes_[0].type == NodeType::Placeholder) plan_.input_name = nodes_[0].name;
         }
         if (units_.empty()) throw std::runtime_error("document contains no operators");
+        index_schedule(stage_names);
         decide_storage();
         allocate_outputs();
         for (size_t i = 0; i < nodes_.size(); i++) emit(static_cast<int>(i));
@@ -314,6 +322,7 @@ private:
         }
         find_depthwise_sums();
         find_activated_combinations();
+        find_residual_convolutions();
         for (PNode &n : nodes_) {
             if (n.type == NodeType::Identity && single_value(n)) {
                 n.parent = n.inputs[0][0].node;
@@ -412,6 +421,80 @@ private:
         }
     }
 
+    // Where the schedule puts every unit (names the schedule does not know stay at -1; assign_stages reports them).
+    void index_schedule(const std::vector<std::vector<std::vector<std::string>>> &stage_names) {
+        std::map<std::string, int> unit_of;
+        for (size_t u = 0; u < units_.size(); u++) unit_of[units_[u]] = static_cast<int>(u);
+        slots_.assign(units_.size(), Slot{});
+        groups_in_stage_.clear();
+        for (const auto &stage : stage_names) groups_in_stage_.push_back((int)stage.size());
+        for (size_t s = 0; s < stage_names.size(); s++)
+            for (size_t g = 0; g < stage_names[s].size(); g++)
+                for (size_t k = 0; k < stage_names[s][g].size(); k++) {
+                    auto it = unit_of.find(stage_names[s][g][k]);
+                    if (it != unit_of.end()) slots_[it->second] = Slot{(int)s, (int)g, (int)k};
+                }
+    }
+
+    bool alone_in_its_stage(int unit) const { return slots_[unit].stage >= 0 && groups_in_stage_[slots_[unit].stage] == 1; }
+
+    // true when everything `node` writes is complete before the unit `consumer_unit` starts
+    bool complete_before(int node, int consumer_unit) const {
+        const int unit = nodes_[node].unit;
+        if (unit < 0) return true;   // placeholder
+        const Slot &a = slots_[unit], &b = slots_[consumer_unit];
+        if (a.stage < 0 || b.stage < 0) return false;
+        return a.stage < b.stage || (a.stage == b.stage && a.group == b.group && a.pos < b.pos);
+    }
+
+    // "convolution, + skip value (, ReLU)" of a residual unit (reference python/ios/models/resnet.py:10-27): when the
+    // convolution's output is read by the addition only, the skip value is complete before the convolution starts, the
+    // convolution has its stage to itself and takes the matrix path, its epilogue adds the skip value (and applies the ReLU) and the addition's launch
+    // and the convolution's own tensor disappear.  The rounding is that of the separate launches: act(conv + bias) is
+    // rounded to fp32 before the skip value is added.
+    void find_residual_convolutions() {
+        for (size_t i = 0; i < nodes_.size(); i++) {
+            PNode &e = nodes_[i];
+            if (e.type != NodeType::Element || (*e.cfg)["op_type"].as_string() != "add") continue;
+            if (e.inputs.size() != 1 || e.inputs[0].size() != 2 || e.made_by_conv) continue;
+            // the node that holds the result: the addition, or the activation that absorbed it
+            int holder = static_cast<int>(i);
+            bool relu = false;
+            if (e.no_storage) {
+                holder = -1;
+                for (size_t k = 0; k < nodes_.size(); k++)
+                    if (nodes_[k].combine_front == static_cast<int>(i)) holder = static_cast<int>(k);
+                if (holder < 0) continue;
+                const PNode &act = nodes_[holder];
+                const int code = act.type == NodeType::Relu ? ACT_RELU : act_code((*act.cfg)["act_type"].as_string());
+                if (code != ACT_RELU) continue;
+                relu = true;
+            }
+            for (int side = 0; side < 2; side++) {
+                const Val &mine = e.inputs[0][side], &other = e.inputs[0][1 - side];
+                PNode &c = nodes_[mine.node];
+                if (c.type != NodeType::Conv || c.unit < 0 || c.references != 1 || mine.begin != 0 || mine.end != c.C) continue;
+                if (c.residual_into >= 0 || c.sum_front >= 0 || nodes_[other.node].type == NodeType::Sequential) continue;
+                if (unit_result_[c.unit] != mine.node) continue;   // a member of a Sequential
+                const ConvProblem p = problem_of(c);
+                if (p.is_depthwise() || (p.groups > 1 && (p.ICg() < 4 || p.OCg() < 8)) || !conv_matrix_path_supported(p) || conv_thin_applies(p))
+                    continue;
+                if ((unsigned long long)batch_ * p.OC * p.OH * p.OW * 4ull >= (1ull << 30)) continue;
+                // (the residual epilogue exists in the stand-alone kernels only: a stage of several groups is one fused launch)
+                if (!alone_in_its_stage(c.unit) || !complete_before(other.node, c.unit)) continue;
+                c.residual_into = holder;
+                c.parent = holder;   // the convolution writes the holder's tensor
+                c.parent_begin = 0;
+                c.residual_other = other;
+                c.residual_relu = relu;
+                nodes_[holder].made_by_conv = true;
+                if (holder != static_cast<int>(i)) nodes_[holder].combine_front = -1;   // nothing left to combine
+                e.no_storage = holder != static_cast<int>(i);
+                break;
+            }
+        }
+    }
+
     int resolve_sequential(int index) const {
         while (nodes_[index].type == NodeType::Sequential) index = nodes_[index].parent;
         return index;
@@ -471,6 +554,7 @@ private:
             touch(op.in.offset, op.stage);
             touch(op.out.offset, op.stage);
             for (const ViewRef &v : op.srcs) touch(v.offset, op.stage);
+            if (op.has_residual) touch(op.residual.offset, op.stage);
             if (op.conv >= 0 && plan_.convs[op.conv].ws_floats > 0) touch(plan_.convs[op.conv].ws_off, op.stage);
         }
         if (Region *r = region_of(plan_.output.offset)) r->pinned = true;
@@ -521,6 +605,7 @@ private:
             op.in.offset = placed(op.in.offset);
             op.out.offset = placed(op.out.offset);
             for (ViewRef &v : op.srcs) v.offset = placed(v.offset);
+            if (op.has_residual) op.residual.offset = placed(op.residual.offset);
         }
         for (PlanConv &c : plan_.convs)
             if (c.ws_floats > 0) c.ws_off = placed(c.ws_off);
@@ -629,6 +714,7 @@ private:
         PNode &n = nodes_[index];
         if (n.type == NodeType::Placeholder || n.type == NodeType::Sequential) return;
         if (n.no_storage) return;   // ReLU in front of a depth-wise convolution that reads the summed inputs itself
+        if (n.made_by_conv) return;  // addition (and ReLU) of a residual unit: the convolution's epilogue wrote this tensor
         // levels count inside a schedule unit; the members of a Sequential follow each other
         if (n.unit != level_unit_) {
             level_unit_ = n.unit;
@@ -724,6 +810,29 @@ private:
         const double k = sum_srcs.empty() ? 1.0 : (double)sum_srcs.size();
         op.flops = p.flops() + (k - 1.0) * (double)batch_ * C * H * W;
         op.bytes = 4.0 * (k * (double)batch_ * C * H * W + (double)p.OC * p.K() + p.OC + (double)batch_ * p.OC * p.OH * p.OW);
+        if (n.residual_into >= 0) {
+            const double out_elems = (double)batch_ * p.OC * p.OH * p.OW;
+            const ViewRef other = view_of(n.residual_other.node).window(n.residual_other.begin, n.residual_other.end);
+            if (matrix_path && !plan_.convs[conv].thin) {
+                op.has_residual = true;
+                op.residual = other;
+                op.post_relu = n.residual_relu ? 1 : 0;
+                op.flops += out_elems;
+                op.bytes += 4.0 * out_elems;
+            } else {
+                // (an input view beyond the matrix path's offsets: the other kernels have no residual form, the sum follows
+                // in place as a launch of its own)
+                const ViewRef out = op.out;
+                PlanOp &sum = push(OpKind::Nary, n);
+                sum.srcs = {out, other};
+                sum.out = out;
+                sum.act = n.residual_relu ? ACT_RELU : ACT_NONE;
+                sum.flops = out_elems;
+                sum.bytes = 12.0 * out_elems;
+                sum.level = level_base_ + 1;
+                level_top_ = std::max(level_top_, sum.level + 1);
+            }
+        }
     }
 
     void emit_pool(PNode &n, const Json &cfg, int C, int H, int W, int index) {
@@ -764,6 +873,10 @@ private:
                     const int pu = nodes_[v.node].unit;
                     if (pu >= 0 && pu != n.unit) deps[n.unit].insert(pu);
                 }
+            if (n.residual_into >= 0) {   // the convolution's epilogue reads the other value of the addition
+                const int pu = nodes_[n.residual_other.node].unit;
+                if (pu >= 0 && pu != n.unit) deps[n.unit].insert(pu);
+            }
         }
         std::vector<int> state(units_.size(), 0);   // 0 pending, 1 in the running stage, 2 finished
         std::vector<int> group_of(units_.size(), -1);
@@ -807,7 +920,7 @@ private:
     void finish() {
         for (size_t i = 0; i < nodes_.size(); i++) {
             const PNode &n = nodes_[i];
-            if (n.pre_relu_alias || n.no_storage) continue;   // never materialised
+            if (n.pre_relu_alias || n.no_storage || n.residual_into >= 0) continue;   // never materialised
             plan_.tensors[n.name] = view_of(static_cast<int>(i));
         }
         plan_.input = view_of(0);
@@ -860,6 +973,11 @@ private:
     std::map<std::string, int> by_name_;
     std::vector<std::string> units_;
     std::vector<int> unit_result_;
+    struct Slot {
+        int stage = -1, group = -1, pos = -1;
+    };
+    std::vector<Slot> slots_;
+    std::vector<int> groups_in_stage_;
     struct SeqRange { int first, second; };
     std::vector<SeqRange> sequentials_;
     std::vector<Region> regions_;   // ascending virtual offsets
@@ -931,6 +1049,7 @@ std::string describe_plan(const Plan &plan) {
         if (op.kind == OpKind::Nary) os << ",\"inputs\":" << op.srcs.size() << ",\"accumulate\":" << op.accumulate;
         if (op.kind == OpKind::ConvDepthwise) os << ",\"inputs\":" << (op.srcs.empty() ? 1 : op.srcs.size());
         if (op.kind == OpKind::Nary || op.kind == OpKind::Unary) os << ",\"act\":" << op.act;
+        if (op.has_residual) os << ",\"residual\":true,\"post_relu\":" << op.post_relu;
         os << ",\"level\":" << op.level;
         // arena extents in floats, one [begin, end) per image: what the operation writes and what it reads
         auto ranges = [&](const char *key, const std::vector<ViewRef> &views) {
@@ -947,6 +1066,7 @@ std::string describe_plan(const Plan &plan) {
         std::vector<ViewRef> reads = op.srcs;
         if (op.kind != OpKind::Nary && op.srcs.empty()) reads.push_back(op.in);
         if (op.kind == OpKind::Nary && op.accumulate) reads.push_back(op.out);
+        if (op.has_residual) reads.push_back(op.residual);
         ranges("writes", {op.out});
         ranges("reads", reads);
         os << '}';

@@ -67,6 +67,10 @@ struct PlanOp {
     PoolProblem pool{};
     std::vector<ViewRef> srcs;   // Nary: inputs; ConvDepthwise of a sum: the views it adds in its loader (else empty)
     int multiply = 0, accumulate = 0, act = 0;
+    // ConvMfma of a residual unit: out = residual + act(conv + bias), then max(., 0) when post_relu
+    bool has_residual = false;
+    ViewRef residual;
+    int post_relu = 0;
     double flops = 0.0, bytes = 0.0;
 };
 

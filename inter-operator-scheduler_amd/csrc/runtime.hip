@@ -544,8 +544,10 @@ void Session::launch_op(const PlanOp &op, hipStream_t stream) {
     switch (op.kind) {
         case OpKind::ConvMfma: {
             const PlanConv &c = plan_.convs[op.conv];
+            const TensorView residual = op.has_residual ? tv(op.residual) : TensorView{};
             launch_conv_mfma(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off, tv(op.out),
-                             c.ws_floats ? base_ + c.ws_off : nullptr, counters_of(c), stream);
+                             c.ws_floats ? base_ + c.ws_off : nullptr, counters_of(c), stream, op.has_residual ? &residual : nullptr,
+                             op.post_relu != 0);
             break;
         }
         case OpKind::ConvDepthwise: {
@@ -672,12 +674,15 @@ void Session::build_fused() {
                 switch (op.kind) {
                     case OpKind::ConvMfma: {
                         const PlanConv &c = plan_.convs[op.conv];
+                        const TensorView residual = op.has_residual ? tv(op.residual) : TensorView{};
                         const ConvDispatch d = make_conv_dispatch(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off,
-                                                                  tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr, counters_of(c));
-                        pend.fusable = conv_variant(d.variant).fusable();
+                                                                  tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr, counters_of(c),
+                                                                  op.has_residual ? &residual : nullptr, op.post_relu != 0);
+                        pend.fusable = conv_variant(d.variant).fusable() && !op.has_residual;   // (the fused kernel holds the plain epilogue)
                         if (!pend.fusable && !solo)
-                            throw std::runtime_error(std::string("convolution kernel configuration ") + conv_variant(d.variant).name +
-                                                     " cannot run inside a fused stage launch");
+                            throw std::runtime_error(op.has_residual ? std::string("internal: a residual convolution is planned for single-group stages only")
+                                                                     : std::string("convolution kernel configuration ") + conv_variant(d.variant).name +
+                                                                           " cannot run inside a fused stage launch");
                         pend.item.kind = WORK_CONV;
                         pend.item.variant = d.variant;
                         pend.item.tiles = d.tiles;

@@ -270,17 +270,34 @@ def test_arena_reuse_never_lets_an_operator_read_what_another_overwrote(name, ba
 
 
 def test_residual_additions_join_the_activation_behind_them_and_pool_names_follow_the_reference():
-    # ResNet-50: 16 residual units end in addition + in-place ReLU (reference python/ios/models/resnet.py:25-26); the plan
-    # holds one launch per unit for both, applying the ReLU, and the addition has no tensor of its own
+    # ResNet-50: 16 residual units end in convolution, addition of the skip value, in-place ReLU (reference
+    # python/ios/models/resnet.py:19-27).  The convolution's epilogue adds the skip value and applies the ReLU: one launch for
+    # the three operators, no tensor for the convolution and the addition
     graph = ios.models.resnet50()
     ops = rt.plan_describe(graph, 1)
     kinds = [op['kind'] for op in ops]
-    assert kinds.count('conv_mfma') == 53 and kinds.count('nary') == 16 and kinds.count('unary') == 0 and kinds.count('pool') == 1
+    assert kinds.count('conv_mfma') == 53 and kinds.count('pool') == 1 and len(ops) == 54
+    residual = [op for op in ops if op.get('residual')]
     nodes = {n.name: n for n in graph.nodes()}
-    assert all(nodes[op['node']].type == 'activation' and op['act'] == 1 and len(op['reads']) == 2 for op in ops if op['kind'] == 'nary')
-    # ResNet-18 / 34 have no activation behind their additions: the addition itself is the launch
+    assert len(residual) == 16 and all(op['post_relu'] == 1 and len(op['reads']) == 2 and nodes[op['node']].act == 'identity' for op in residual)
+    # ResNet-18 / 34 have no activation behind their additions
     ops18 = rt.plan_describe(ios.models.resnet18(), 1)
-    assert sum(op['kind'] == 'nary' for op in ops18) == 8 and all(op['act'] == 0 for op in ops18 if op['kind'] == 'nary')
+    assert len(ops18) == 21 and sum(1 for op in ops18 if op.get('residual') and op['post_relu'] == 0) == 8
+    # the skip value has to be complete before the convolution starts: with the projection '3' scheduled beside the last
+    # convolution '6' of the first unit, the addition stays a launch of its own (the ReLU behind it still joins it)
+    late = ios.models.resnet50()
+    stages = late.blocks[1].stages
+    assert stages[:5] == [[['3']], [['4']], [['5']], [['6']], [['7']]]
+    late.blocks[1].stages = [[['4']], [['5']], [['6'], ['3']]] + stages[4:]
+    ops_late = rt.plan_describe(late, 1)
+    assert sum(1 for op in ops_late if op.get('residual')) == 15
+    kept = [op for op in ops_late if op['kind'] == 'nary']
+    assert len(kept) == 1 and kept[0]['node'] == '8' and kept[0]['act'] == 1 and len(kept[0]['reads']) == 2
+    # in one group the later of the two convolutions adds the earlier one's output, whichever it is
+    for order, adder in ((['6', '3'], '3'), (['3', '6'], '6')):
+        late.blocks[1].stages = [[['4']], [['5']], [order]] + stages[4:]
+        found = [op['node'] for op in rt.plan_describe(late, 1) if op.get('residual')]
+        assert len(found) == 16 and found[0] == adder
     # pooling names: the reference looks for the substrings "max" and "global" (src/ios/ios_runtime.cu:1047-1051) and its
     # AlexNet writes 'max_pool'
     config = ios.models.alexnet().export_config()
