@@ -125,7 +125,10 @@ int ios_session_run(ios_session *session);                                  /* o
 int ios_session_enqueue(ios_session *session);
 int ios_session_synchronize(ios_session *session);
 int ios_session_get_output(ios_session *session, float *output);
-/* Dense copy of any operator's output (batch x C x H x W) after a run. */
+/* Dense copy of an operator's output (batch x C x H x W) after a run.  Fails, with a message that says which, for an
+ * operator whose output is never written as such (a ReLU applied by the convolution that reads it, a sum added by the
+ * depth-wise convolution or the activation that reads it, the convolution and the addition of a residual unit whose result
+ * the convolution's epilogue writes) and, under "arena_reuse" = "1", for one whose memory a later operator took over. */
 int ios_session_get_tensor(ios_session *session, const char *node_name, float *output);
 /* Same protocol and outputs as graph_latency, on the resident session. */
 int ios_session_measure(ios_session *session, int warmup, int number, int repeat, int profile_stage_latency,
