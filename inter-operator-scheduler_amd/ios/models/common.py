@@ -116,7 +116,10 @@ def _depthwise_conv(inputs, channels, kernel, stride, padding):
 
 
 def _channels_of(inputs):
-    return sum(term[0].node.output_shape[0] for term in inputs)
+    # channels of the concatenated terms; a term's width is that of its values, which may be channel slices (the reference
+    # takes the producer's full width here, python/ios/models/common.py:396,436, and builds an invalid depth-wise convolution
+    # from a sliced input; for whole values the two agree)
+    return sum(term[0].end - term[0].begin for term in inputs)
 
 
 def sep_conv(block: Block, inputs: List[List[Value]], out_channels, kernel, stride, padding, is_exit=False):

@@ -740,6 +740,41 @@ def test_activation_absorbs_the_combination_in_front_of_it():
             assert_close(rt.graph_inference(graph, batch, x), want, f'absorbed combinations, {executor}, batch {batch}')
 
 
+@pytest.mark.parametrize('seed', range(48))
+def test_random_network_matches_oracle(seed):
+    """Seeded random wiring of every operator kind under a random schedule (tests/random_graphs.py): every tensor the plan
+    materialises and the result agree with the oracle, under the stream and the fused executor, with and without arena reuse."""
+    import random_graphs
+    graph, batch = random_graphs.random_graph(seed)
+    x = np.random.default_rng(seed).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
+    want_all = ios_oracle.run(graph, x, keep_all=True)
+    want = want_all[graph.exit_node.name]
+    rt.set_option('arena_reuse', 0)
+    with rt.Session(graph, batch) as session:
+        session.load_weights()
+        session.set_input(x)
+        session.run()
+        compared = 0
+        for node in list(graph.nodes())[1:]:
+            try:
+                tensor = session.tensor(node)
+            except RuntimeError as error:
+                assert 'no materialised output' in str(error)
+                continue
+            assert_close(tensor, want_all[node.name], f'seed {seed}: node {node.name} ({node.type})', scaled=True)
+            compared += 1
+        assert compared >= len(list(graph.nodes())) // 2
+    rt.set_option('arena_reuse', 1)
+    for executor in ('streams', 'fused', 'fused_graph'):
+        rt.set_option('executor', executor)
+        with rt.Session(graph, batch) as session:
+            session.load_weights()
+            session.set_input(x)
+            for _ in range(2):
+                session.run()
+            assert_close(session.output(), want, f'seed {seed}, {executor}', scaled=True)
+
+
 def test_inception_batch_16_under_the_schedule_searched_at_that_batch():
     """
     The middle point of the batch sweep, the way the benchmark runs it: dp_parallel schedule searched with on-device stage

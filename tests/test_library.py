@@ -309,6 +309,24 @@ def test_residual_additions_join_the_activation_behind_them_and_pool_names_follo
     assert [(op['kind'], op['reads'], op['writes']) for op in renamed] == [(op['kind'], op['reads'], op['writes']) for op in plain]
 
 
+@pytest.mark.parametrize('seed', range(0, 120, 3))
+def test_random_networks_plan_and_share_the_arena_safely(seed):
+    """Random wiring of every operator kind under random schedules (tests/random_graphs.py): the planner accepts them, and
+    with arena reuse every operation still reads what the same operations wrote."""
+    import random_graphs
+    graph, batch = random_graphs.random_graph(seed)
+    try:
+        rt.set_option('arena_reuse', 0)
+        plain = rt.plan_describe(graph, batch)
+        rt.set_option('arena_reuse', 1)
+        shared = rt.plan_describe(graph, batch)
+    finally:
+        rt.set_option('arena_reuse', 1)
+    assert [(op['node'], op['kind']) for op in plain] == [(op['node'], op['kind']) for op in shared]
+    assert _simulate(shared) == _simulate(plain)
+    assert rt.plan_arena_bytes(graph, batch) > 0
+
+
 def test_planner_options_need_no_device_and_change_the_plan():
     graph = ios.models.inception_v3()
     graph.sequential_schedule()
