@@ -132,6 +132,10 @@ def check_merge(s: int, idn: Dict[int, Node]) -> bool:
     if not all(isinstance(node, Conv) for node in nodes):
         return False
     first = nodes[0]
+    # (the reference tests groups and inputs from the second operator on, optimizer.py:259-277; a grouped first convolution
+    # would be stacked as if it were dense, so it is refused here; further input terms of the first one are merged correctly)
+    if first.groups != 1:
+        return False
     for node in nodes[1:]:
         if tuple(node.input_shape[1:]) != tuple(first.input_shape[1:]):
             return False
@@ -373,12 +377,26 @@ def construct(stage_list: List[Stage], block: Block, constructed_blocks: List[Bl
         return new
 
     def merge(convs: List[Conv]) -> Node:
+        """
+        One convolution for all of ``convs`` (reference optimizer.py:662-711): its input concatenates the distinct input
+        terms of the merged convolutions, its filters hold every convolution's filters in the rows of its output channels
+        and the columns of its own terms (zeros elsewhere), smaller kernels centred in the common window.  ``check_merge``
+        admits convolutions that read one and the same value; like the reference's it does not look at the inputs of the
+        first one, which may therefore bring further terms along.
+        """
         out_channels, kernel, stride, padding = merged_conv_geometry(convs)
         terms = get_input(convs, block, nid, idn)
-        assert len(terms) == 1 and len(terms[0]) == 1, 'merged convolutions must share one input value'
+
+        def key_of(term):
+            return tuple((id(v.node), v.begin, v.end) for v in term)
+
+        begin_of, at = {}, 0
+        for term in terms:
+            begin_of[key_of(term)] = at
+            at += term[0].length
         new = Conv(convs[0].name, ' '.join(c.hint_name for c in convs), None, out_channels, kernel, stride,
                    padding, 1, convs[0].act, None)
-        new.inputs = relocate(terms)
+        new.inputs = relocate(terms)      # (joins neighbouring slices; the channel order stays)
         new._register_uses()
         new.infer_shape()
         if compute_weight:
@@ -391,7 +409,13 @@ def construct(stage_list: List[Stage], block: Block, constructed_blocks: List[Bl
                 # smaller kernels sit centred inside the common kernel window, zeros around them
                 r0 = (kernel[0] - conv.kernel[0]) // 2
                 c0 = (kernel[1] - conv.kernel[1]) // 2
-                new.weight[first:last, :, r0:r0 + conv.kernel[0], c0:c0 + conv.kernel[1]] = conv.weight
+                own = 0
+                for term in conv.inputs:
+                    width = term[0].length
+                    column = begin_of[key_of(term)]
+                    new.weight[first:last, column:column + width, r0:r0 + conv.kernel[0], c0:c0 + conv.kernel[1]] += \
+                        conv.weight[:, own:own + width]
+                    own += width
                 new.bias[first:last] = conv.bias
             located[conv] = (new, first, last)
             first = last

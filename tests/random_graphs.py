@@ -62,12 +62,20 @@ def random_block(rng, enter, downsample):
             base = ios.conv2d(block, [[enter]], int(rng.integers(4, 17)), (3, 3), (2, 2), (1, 1), 1, _pick(rng, ['relu', 'identity']))
         values = [base]
     for _ in range(int(rng.integers(4, 11))):
-        kind = _pick(rng, ['conv', 'conv', 'conv', 'depthwise', 'grouped', 'pool', 'relu', 'activation', 'element', 'sum', 'concat', 'separable'])
+        kind = _pick(rng, ['conv', 'conv', 'conv', 'sibling', 'depthwise', 'grouped', 'pool', 'relu', 'activation', 'element', 'sum', 'concat', 'separable'])
         if kind == 'conv':
             terms = _terms(rng, values)
             k = _pick(rng, [(1, 1), (1, 1), (3, 3), (3, 3), (1, 3), (3, 1), (5, 5)])
             out = ios.conv2d(block, terms, int(rng.integers(3, 25)), k, (1, 1), (k[0] // 2, k[1] // 2), 1,
                              _pick(rng, ['relu', 'relu', 'identity', 'identity', 'tanh', 'sigmoid']))
+        elif kind == 'sibling':
+            # a second convolution on the inputs of an earlier one, same stride and activation: what the merge search stacks
+            convs = [v.node for v in values if v.node.type == 'conv' and v.node.groups == 1 and v.node.inputs is not None]
+            if not convs:
+                continue
+            twin = _pick(rng, convs)
+            k = _pick(rng, [tuple(twin.kernel), (1, 1), (3, 3), (1, 3), (3, 1)])
+            out = ios.conv2d(block, [list(term) for term in twin.inputs], int(rng.integers(3, 17)), k, tuple(twin.stride), (k[0] // 2, k[1] // 2), 1, twin.act)
         elif kind == 'depthwise':
             terms = _terms(rng, values, max_terms=1, max_summed=4)
             k = _pick(rng, [3, 3, 5, 7])
@@ -115,7 +123,11 @@ def random_block(rng, enter, downsample):
 
 
 def random_graph(seed):
-    """(graph with a schedule, batch size)"""
+    """
+    (graph with a schedule, batch size, the graph as it was built).  A fifth of the graphs went through the merge search,
+    which replaces sibling convolutions by one convolution with stacked filters read through channel slices; the graph as
+    built computes the same function and is what a result is checked against.
+    """
     rng = np.random.default_rng(seed)
     ios.reset_name()
     side = int(rng.integers(5, 14))
@@ -126,14 +138,16 @@ def random_graph(seed):
         blocks.append(block)
     graph = Graph(f'random_{seed}', pv.node, blocks)
     graph.init_weights(seed, 'he_normal_bias')
+    built = graph
     batch = int(rng.integers(1, 4))
-    choice = int(rng.integers(4))
+    choice = int(rng.integers(5))
     if choice == 0:
         graph.sequential_schedule()
     elif choice == 1:
         graph.greedy_schedule(int(rng.integers(2, 9)))
     else:
         graph.sequential_schedule()
+        kind = 'dp_parallel' if choice < 4 else _pick(rng, ['dp_merge', 'dp_parallel_merge'])
         graph = ios.optimize(graph, batch, ios.AnalyticCostModel(launch=1.0, rate=float(10 ** rng.integers(4, 8)), sync=float(rng.random())),
-                             'dp_parallel', max_group_size=int(rng.integers(1, 4)), max_num_groups=int(rng.integers(2, 7)), compute_weight=True)
-    return graph, batch
+                             kind, max_group_size=int(rng.integers(1, 4)), max_num_groups=int(rng.integers(2, 7)), compute_weight=True)
+    return graph, batch, built

@@ -740,15 +740,15 @@ def test_activation_absorbs_the_combination_in_front_of_it():
             assert_close(rt.graph_inference(graph, batch, x), want, f'absorbed combinations, {executor}, batch {batch}')
 
 
-@pytest.mark.parametrize('seed', range(48))
+@pytest.mark.parametrize('seed', range(60))
 def test_random_network_matches_oracle(seed):
     """Seeded random wiring of every operator kind under a random schedule (tests/random_graphs.py): every tensor the plan
     materialises and the result agree with the oracle, under the stream and the fused executor, with and without arena reuse."""
     import random_graphs
-    graph, batch = random_graphs.random_graph(seed)
+    graph, batch, built = random_graphs.random_graph(seed)
     x = np.random.default_rng(seed).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
     want_all = ios_oracle.run(graph, x, keep_all=True)
-    want = want_all[graph.exit_node.name]
+    want = ios_oracle.run(built, x)      # (the graph as built: a merge search must not change the function)
     rt.set_option('arena_reuse', 0)
     with rt.Session(graph, batch) as session:
         session.load_weights()

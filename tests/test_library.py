@@ -314,7 +314,7 @@ def test_random_networks_plan_and_share_the_arena_safely(seed):
     """Random wiring of every operator kind under random schedules (tests/random_graphs.py): the planner accepts them, and
     with arena reuse every operation still reads what the same operations wrote."""
     import random_graphs
-    graph, batch = random_graphs.random_graph(seed)
+    graph, batch, _ = random_graphs.random_graph(seed)
     try:
         rt.set_option('arena_reuse', 0)
         plain = rt.plan_describe(graph, batch)

@@ -228,6 +228,45 @@ def test_check_merge_rules():
     assert check_merge(sum(1 << idx_e[n] for n in ['99', '100']), idn_e)
 
 
+def test_merge_with_further_terms_on_the_first_convolution_and_grouped_convolutions():
+    """
+    The reference's check_merge looks at groups and inputs from the second convolution on (optimizer.py:259-277).  A first
+    convolution that concatenates a further term is merged with its filters in the columns of its own terms; a grouped first
+    convolution is refused.  Both were found by the random networks of tests/random_graphs.py.
+    """
+    from oracle import ios_oracle
+    ios.reset_name()
+    v = ios.placeholder((6, 9, 9))
+    block = ios.Block(v.node)
+    u = ios.pool2d(block, [[Value(v.node, 1, 6)]], 'avg', (3, 3), (1, 1), (1, 1))
+    a = ios.conv2d(block, [[v], [u]], 7, (3, 3), padding=(1, 1), act='relu')       # reads v and u
+    b = ios.conv2d(block, [[v]], 4, (1, 3), padding=(0, 1), act='relu')              # reads v only
+    ios.identity(block, [[a], [b]], is_exit=True)
+    graph = Graph('merge_terms', v.node, [block])
+    graph.init_weights(3, 'he_normal_bias')
+    graph.sequential_schedule()
+    merged = optimize(graph, 1, AnalyticCostModel(launch=1.0, rate=1e12, sync=0.0), 'dp_merge', compute_weight=True)
+    stacked = [n for n in merged.nodes() if ' ' in n.hint_name]
+    assert len(stacked) == 1 and stacked[0].out_channels == 11 and stacked[0].input_shape[0] == 11      # v (6) and u (5)
+    x = np.random.default_rng(0).standard_normal((2, 6, 9, 9)).astype(np.float32)
+    np.testing.assert_allclose(ios_oracle.run(merged, x), ios_oracle.run(graph, x), rtol=1e-5, atol=1e-5)
+
+    ios.reset_name()
+    v = ios.placeholder((6, 9, 9))
+    block = ios.Block(v.node)
+    d = ios.conv2d(block, [[v]], 6, (3, 3), padding=(1, 1), groups=6, act='relu')
+    e = ios.conv2d(block, [[v]], 4, (3, 3), padding=(1, 1), act='relu')
+    ios.identity(block, [[d], [e]], is_exit=True)
+    graph = Graph('merge_grouped', v.node, [block])
+    graph.init_weights(3, 'he_normal_bias')
+    graph.sequential_schedule()
+    idn = {i: n for i, n in enumerate([d.node, e.node])}
+    assert not check_merge(0b11, idn)
+    merged = optimize(graph, 1, AnalyticCostModel(launch=1.0, rate=1e12, sync=0.0), 'dp_merge', compute_weight=True)
+    assert not any(' ' in n.hint_name for n in merged.nodes())
+    np.testing.assert_allclose(ios_oracle.run(merged, x), ios_oracle.run(graph, x), rtol=1e-5, atol=1e-5)
+
+
 def test_merged_graph_weights_reproduce_unmerged_outputs():
     from oracle import ios_oracle
     ios.reset_name()
