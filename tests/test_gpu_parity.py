@@ -775,6 +775,34 @@ def test_random_network_matches_oracle(seed):
             assert_close(session.output(), want, f'seed {seed}, {executor}', scaled=True)
 
 
+@pytest.mark.parametrize('seed', range(100, 124))
+def test_random_network_through_the_other_entry_points(seed):
+    """The same random networks through the entry point that allocates nothing (bit-identical), in the reduced-precision
+    modes (error of the operand rounding) and through graph / block / stage latency under the stream and the fused executor."""
+    import random_graphs
+    graph, batch, built = random_graphs.random_graph(seed)
+    x = np.random.default_rng(seed).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
+    want = ios_oracle.run(built, x)
+    rt.set_option('executor', 'fused')
+    plain = rt.graph_inference(graph, batch, x)
+    assert_close(plain, want, f'seed {seed}', scaled=True)
+    np.testing.assert_array_equal(rt.graph_inference(graph, batch, x, no_alloc=True), plain)
+    for precision in ('bf16', 'fp16'):
+        rt.set_option('precision', precision)
+        assert_close_reduced(rt.graph_inference(graph, batch, x), want, f'seed {seed}, {precision}')
+    rt.set_option('precision', 'fp32')
+    stages = sum(len(block.stages) for block in graph.blocks)
+    for executor in ('streams', 'fused'):
+        rt.set_option('executor', executor)
+        total, per_stage = rt.graph_latency(graph, batch, 0, 1, 2, profile_stage=True)
+        assert len(total) == 2 and len(per_stage) == 2 * stages and min(total) > 0
+        for block in graph.blocks:
+            assert min(rt.block_latency(block, batch, 0, 1, 1)) > 0
+            names = {node.name: node for node in block.inner_nodes + [block.exit_node]}
+            for stage in block.stages:
+                assert min(rt.stage_latency([[names[name] for name in group] for group in stage], batch, 0, 1, 1)) > 0
+
+
 def test_inception_batch_16_under_the_schedule_searched_at_that_batch():
     """
     The middle point of the batch sweep, the way the benchmark runs it: dp_parallel schedule searched with on-device stage
