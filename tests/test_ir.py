@@ -130,6 +130,18 @@ def test_config_round_trip_all_models():
         assert json.loads(json.dumps(again.export_config())) == config
 
 
+def test_random_networks_round_trip_through_the_wire_format():
+    import random_graphs
+    for seed in range(0, 60, 2):
+        graph, _, _ = random_graphs.random_graph(seed)
+        config = json.loads(json.dumps(graph.export_config()))
+        again = Graph.from_config(config)
+        assert json.loads(json.dumps(again.export_config())) == config
+        assert [n.name for n in again.nodes()] == [n.name for n in graph.nodes()]
+        assert [tuple(n.output_shape) for n in again.nodes()] == [tuple(n.output_shape) for n in graph.nodes()]
+        assert again.flops() == graph.flops() and again.kernels() == graph.kernels()
+
+
 def test_model_output_shapes():
     assert tuple(ios.models.squeezenet_1_1().exit_node.output_shape) == (1000, 1, 1)
     sq = ios.models.squeezenet_1_1()

@@ -111,6 +111,25 @@ def test_dp_optimum_equals_brute_force(r, s):
         assert got == pytest.approx(want, rel=1e-12), graph.name
 
 
+@pytest.mark.parametrize('seed', range(16))
+def test_dp_optimum_equals_brute_force_on_random_blocks(seed):
+    """Random wiring (tests/random_graphs.py: sums, slices, separable units, dead-end-free blocks of 5-12 operators)."""
+    import random_graphs
+    _, _, graph = random_graphs.random_graph(seed)
+    r, s = [(1, 4), (2, 3), (3, 8)][seed % 3]
+    cost = TableCost(seed=seed)
+    graph.sequential_schedule()
+    new_graph = optimize(graph, 1, cost, 'dp_parallel', max_group_size=r, max_num_groups=s)
+    check_schedule_invariants(graph, new_graph, r, s)
+    for old, new in zip(graph.blocks, new_graph.blocks):
+        if len(old.inner_nodes) > 11:
+            continue
+        want = brute_force_best(old, cost, r, s)
+        by_name = {n.name: n for n in new.inner_nodes + [new.exit_node]}
+        got = sum(stage_key_cost(cost, [[by_name[n] for n in g] for g in stage]) for stage in new.stages)
+        assert got == pytest.approx(want, rel=1e-12), (seed, old.exit_node.name)
+
+
 def check_schedule_invariants(graph, new_graph, max_group_size, max_num_groups):
     assert len(new_graph.blocks) == len(graph.blocks)
     for old, new in zip(graph.blocks, new_graph.blocks):
