@@ -52,21 +52,21 @@ def _channels(terms):
     return sum(term[0].length for term in terms)
 
 
-def random_block(rng, enter, downsample):
+def random_block(rng, enter, downsample, wide=1):
     block = ios.Block(enter.node)
     values = [enter]
     if downsample:
         if rng.random() < 0.5:
             base = ios.pool2d(block, [[enter]], _pick(rng, ['max', 'avg']), (3, 3), (2, 2), (1, 1))
         else:
-            base = ios.conv2d(block, [[enter]], int(rng.integers(4, 17)), (3, 3), (2, 2), (1, 1), 1, _pick(rng, ['relu', 'identity']))
+            base = ios.conv2d(block, [[enter]], wide * int(rng.integers(4, 17)), (3, 3), (2, 2), (1, 1), 1, _pick(rng, ['relu', 'identity']))
         values = [base]
     for _ in range(int(rng.integers(4, 11))):
         kind = _pick(rng, ['conv', 'conv', 'conv', 'sibling', 'depthwise', 'grouped', 'pool', 'relu', 'activation', 'element', 'sum', 'concat', 'separable'])
         if kind == 'conv':
             terms = _terms(rng, values)
             k = _pick(rng, [(1, 1), (1, 1), (3, 3), (3, 3), (1, 3), (3, 1), (5, 5)])
-            out = ios.conv2d(block, terms, int(rng.integers(3, 25)), k, (1, 1), (k[0] // 2, k[1] // 2), 1,
+            out = ios.conv2d(block, terms, wide * int(rng.integers(3, 25)), k, (1, 1), (k[0] // 2, k[1] // 2), 1,
                              _pick(rng, ['relu', 'relu', 'identity', 'identity', 'tanh', 'sigmoid']))
         elif kind == 'sibling':
             # a second convolution on the inputs of an earlier one, same stride and activation: what the merge search stacks
@@ -75,7 +75,7 @@ def random_block(rng, enter, downsample):
                 continue
             twin = _pick(rng, convs)
             k = _pick(rng, [tuple(twin.kernel), (1, 1), (3, 3), (1, 3), (3, 1)])
-            out = ios.conv2d(block, [list(term) for term in twin.inputs], int(rng.integers(3, 17)), k, tuple(twin.stride), (k[0] // 2, k[1] // 2), 1, twin.act)
+            out = ios.conv2d(block, [list(term) for term in twin.inputs], wide * int(rng.integers(3, 17)), k, tuple(twin.stride), (k[0] // 2, k[1] // 2), 1, twin.act)
         elif kind == 'depthwise':
             terms = _terms(rng, values, max_terms=1, max_summed=4)
             k = _pick(rng, [3, 3, 5, 7])
@@ -85,7 +85,7 @@ def random_block(rng, enter, downsample):
             terms = _terms(rng, values)
             c = _channels(terms)
             groups = 2 if c % 2 == 0 else 1
-            out = ios.conv2d(block, terms, groups * int(rng.integers(2, 9)), (3, 3), (1, 1), (1, 1), groups, _pick(rng, ['relu', 'identity']))
+            out = ios.conv2d(block, terms, groups * wide * int(rng.integers(2, 9)), (3, 3), (1, 1), (1, 1), groups, _pick(rng, ['relu', 'identity']))
         elif kind == 'pool':
             out = ios.pool2d(block, _terms(rng, values, max_terms=1, max_summed=2), _pick(rng, ['max', 'avg']), (3, 3), (1, 1), (1, 1))
         elif kind == 'relu':
@@ -111,7 +111,7 @@ def random_block(rng, enter, downsample):
             terms = _terms(rng, values, max_terms=1, max_summed=4)
             k = _pick(rng, [3, 5])
             make = ios.relu_sep_conv if rng.random() < 0.7 else ios.sep_conv
-            out = make(block, terms, int(rng.integers(4, 17)), (k, k), (1, 1), (k // 2, k // 2))
+            out = make(block, terms, wide * int(rng.integers(4, 17)), (k, k), (1, 1), (k // 2, k // 2))
         values.append(out)
     # the exit concatenates everything nobody has read yet, so that no operator is dead
     loose = [value for value in values[1:] if not value.node.uses] or [values[-1]]
@@ -122,19 +122,23 @@ def random_block(rng, enter, downsample):
     return exit_value, block
 
 
-def random_graph(seed):
+def random_graph(seed, large=False):
     """
+    `large`: eight times the channels on 20-44 pixel sides (several tiles per convolution, long reductions, the wide pooling
+    path) instead of 3-24 channels on 5-13 pixel sides.
+
     (graph with a schedule, batch size, the graph as it was built).  A fifth of the graphs went through the merge search,
     which replaces sibling convolutions by one convolution with stacked filters read through channel slices; the graph as
     built computes the same function and is what a result is checked against.
     """
     rng = np.random.default_rng(seed)
     ios.reset_name()
-    side = int(rng.integers(5, 14))
-    pv = ios.placeholder((int(rng.integers(3, 13)), side, int(rng.integers(5, 14))))
+    wide = 8 if large else 1
+    low, high = (20, 45) if large else (5, 14)
+    pv = ios.placeholder((wide * int(rng.integers(3, 13)), int(rng.integers(low, high)), int(rng.integers(low, high))))
     value, blocks = pv, []
     for index in range(int(rng.integers(1, 4))):
-        value, block = random_block(rng, value, downsample=index > 0 and rng.random() < 0.6)
+        value, block = random_block(rng, value, downsample=index > 0 and rng.random() < 0.6, wide=wide)
         blocks.append(block)
     graph = Graph(f'random_{seed}', pv.node, blocks)
     graph.init_weights(seed, 'he_normal_bias')

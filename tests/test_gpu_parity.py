@@ -740,12 +740,13 @@ def test_activation_absorbs_the_combination_in_front_of_it():
             assert_close(rt.graph_inference(graph, batch, x), want, f'absorbed combinations, {executor}, batch {batch}')
 
 
-@pytest.mark.parametrize('seed', range(60))
-def test_random_network_matches_oracle(seed):
-    """Seeded random wiring of every operator kind under a random schedule (tests/random_graphs.py): every tensor the plan
-    materialises and the result agree with the oracle, under the stream and the fused executor, with and without arena reuse."""
+@pytest.mark.parametrize('seed,large', [(seed, False) for seed in range(60)] + [(seed, True) for seed in range(16)])
+def test_random_network_matches_oracle(seed, large):
+    """Seeded random wiring of every operator kind under a random schedule (tests/random_graphs.py; `large`: 24-190 channels
+    on 20-44 pixel sides): every tensor the plan materialises and the result agree with the oracle, under the stream and the
+    fused executors, with and without arena reuse."""
     import random_graphs
-    graph, batch, built = random_graphs.random_graph(seed)
+    graph, batch, built = random_graphs.random_graph(seed, large)
     x = np.random.default_rng(seed).standard_normal((batch, *graph.enter_node.output_shape)).astype(np.float32)
     want_all = ios_oracle.run(graph, x, keep_all=True)
     want = ios_oracle.run(built, x)      # (the graph as built: a merge search must not change the function)
