@@ -228,12 +228,15 @@ def probe(args, np, ios, rt):
         # measured schedule search (fills the kernel-configuration cache named by IOS_TUNE_CACHE), schedule written to a file
         rt.set_option('executor', args.search_executor)
         t0 = time.time()
+        big = args.model in ('randwire_small', 'nasnet_mobile')      # (minutes at r = 3)
+        group_size = args.big_max_group_size if big else args.max_group_size
         optimized = ios.optimize(graph, batch_size=batch, opt_type='dp_parallel', compute_weight=True, warmup=2,
                                  number=args.search_number, repeat=args.search_repeat,
-                                 max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
+                                 max_group_size=group_size, max_num_groups=args.max_num_groups)
         with open(args.schedule_file, 'w') as f:
             json.dump(optimized.export_config(), f)
         print(json.dumps({'probe': 'search', 'model': args.model, 'batch': batch, 'search_seconds': time.time() - t0,
+                          'pruning': f'r = {group_size}, s = {args.max_num_groups}',
                           'stages': sum(len(b.stages) for b in optimized.blocks), 'schedule_file': args.schedule_file}))
         return
     # --probe pass: N passes of one plan and nothing else that launches kernels of the same names
@@ -285,10 +288,12 @@ def main():
                              "closed-form model (no device probes; keeps profiler traces small)")
     parser.add_argument('--search-number', type=int, default=6, help='passes per stage probe of the schedule search')
     parser.add_argument('--search-repeat', type=int, default=3, help='probes per candidate stage of the schedule search')
-    parser.add_argument('--max-group-size', type=int, default=1,
-                        help='pruning knob r of the schedule search (operators per group).  The fused executor runs the groups of a '
-                             'stage level by level, so groups of one operator (r = 1) let the search place every level freely; the '
-                             'reference default r = 3 is measured beside it')
+    parser.add_argument('--max-group-size', type=int, default=3,
+                        help='pruning knob r of the schedule search (operators per group); 3 is the reference default '
+                             '(python/ios/optimizer.py:42).  The search with r = 1 is measured beside it')
+    parser.add_argument('--big-max-group-size', type=int, default=1,
+                        help='r for the searches of RandWire and NASNet, whose searches take minutes at r = 3 (709 s / 168 s) and half a '
+                             'minute at r = 1; their entries name the r they were searched with')
     parser.add_argument('--max-num-groups', type=int, default=8, help='pruning knob s of the schedule search (groups per stage)')
     parser.add_argument('--search-restarts', type=int, default=2,
                         help='schedule searches to run (stage measurements are noisy: the schedule that measures faster as a whole is kept)')
@@ -296,10 +301,9 @@ def main():
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg and the oracle comparisons')
     parser.add_argument('--no-configs', action='store_true', help='skip the other four configuration networks')
     parser.add_argument('--no-extras', action='store_true',
-                        help='skip the r = 3 and merged-convolution searches, the reduced-precision mode and the reference table variants')
+                        help='skip the r = 1 and merged-convolution searches, the reduced-precision mode and the reference table variants')
     parser.add_argument('--greedy-big', action='store_true',
-                        help='use the greedy schedule for RandWire and NASNet instead of the measured search (half a minute each at r = 1, '
-                             'minutes at r = 3)')
+                        help='use the greedy schedule for RandWire and NASNet instead of the measured search')
     parser.add_argument('--search-variants', action='store_true',
                         help="measured schedule search also for the reference table's large model variants (about two more minutes)")
     parser.add_argument('--option', action='append', default=[], metavar='KEY=VALUE', help='extra runtime option (repeatable)')
@@ -398,18 +402,22 @@ def main():
     rt.set_option('executor', args.executor)
 
     if not args.no_extras:
-        # the same search with the reference's default pruning (r = 3, s = 8), for comparison with the headline's r and s
-        if (args.max_group_size, args.max_num_groups) != (3, 8):
-            rt.set_option('executor', args.search_executor)
-            t0 = time.time()
-            default_knobs = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
-                                         warmup=2, number=args.search_number, repeat=args.search_repeat)
-            default_search_s = time.time() - t0
-            graph.sequential_schedule()
-            rt.set_option('executor', args.executor)
-            r3, _ = timed_latency(rt, np, default_knobs, batch, x, args.steps, args.warmup)
-            result['dp_parallel_r3_s8'] = {'latency_ms': r3, 'images_per_s': batch / (r3['wall'] * 1e-3), 'search_seconds': default_search_s,
-                                           'num_stages': sum(len(b.stages) for b in default_knobs.blocks)}
+        # the same search with the other pruning of interest, for comparison with the headline's r and s: groups of one
+        # operator (r = 1: the fused executor runs the groups of a stage level by level, so the search can cut every level
+        # where it measures best) when the headline uses the reference's defaults, the reference's defaults otherwise
+        other_r, other_s = (1, 8) if (args.max_group_size, args.max_num_groups) == (3, 8) else (3, 8)
+        rt.set_option('executor', args.search_executor)
+        t0 = time.time()
+        other_knobs = ios.optimize(graph, batch_size=batch, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
+                                   warmup=2, number=args.search_number, repeat=args.search_repeat, max_group_size=other_r,
+                                   max_num_groups=other_s)
+        other_search_s = time.time() - t0
+        graph.sequential_schedule()
+        rt.set_option('executor', args.executor)
+        other_ms, _ = timed_latency(rt, np, other_knobs, batch, x, args.steps, args.warmup)
+        result[f'dp_parallel_r{other_r}_s{other_s}'] = {'latency_ms': other_ms, 'images_per_s': batch / (other_ms['wall'] * 1e-3),
+                                                       'search_seconds': other_search_s,
+                                                       'num_stages': sum(len(b.stages) for b in other_knobs.blocks)}
 
         # the reference's best schedule family (parallel groups + merged convolutions, "IOS-Both"); the headline metric
         # is the dp_parallel schedule, this one is reported beside it
@@ -487,8 +495,9 @@ def main():
                 t0 = time.time()
                 # stages that are the same computation on the same shapes (NASNet's repeated cells) are measured once
                 shared = ios.IOSCostModel(share_identical_stages=True)
+                group_size = args.max_group_size if search else args.big_max_group_size
                 scheduled = ios.optimize(g, batch_size=1, cost_model=shared, opt_type='dp_parallel', compute_weight=True, warmup=2, number=6,
-                                         repeat=3, max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
+                                         repeat=3, max_group_size=group_size, max_num_groups=args.max_num_groups)
                 search_c = time.time() - t0
                 label = 'dp_parallel'
                 rt.set_option('executor', args.executor)
@@ -503,6 +512,7 @@ def main():
             ops_c = rt.plan_describe(g, 1)
             _, launches_c, kernels_c = launch_profile(rt, scheduled, 1, xc)
             configs[name] = {'sequential_ms': c_seq['wall'], f'{label}_ms': c_par['wall'], 'search_seconds': search_c,
+                             'search_pruning': None if label == 'greedy' else f'r={group_size}, s={args.max_num_groups}',
                              'initialisation': CONFIG_MODELS[name][1], 'device_operations': len(ops_c), 'launches_per_pass': len(launches_c),
                              'network_roofline_ms': network_roofline_ms(ops_c, parallel=False),
                              'fraction_of_network_roofline': network_roofline_ms(ops_c, parallel=False) / c_par['wall'],
@@ -532,7 +542,7 @@ def main():
                     rt.set_option('executor', args.search_executor)
                     t0 = time.time()
                     searched = ios.optimize(make(init_seed=0, init_scheme='he_normal'), batch_size=1, opt_type='dp_parallel', compute_weight=True,
-                                            warmup=2, number=6, repeat=3, max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
+                                            warmup=2, number=6, repeat=3, max_group_size=args.big_max_group_size, max_num_groups=args.max_num_groups)
                     variants[name]['search_seconds'] = time.time() - t0
                     rt.set_option('executor', args.executor)
                     v_dp, _ = timed_latency(rt, np, searched, 1, xc, 50, 5)
