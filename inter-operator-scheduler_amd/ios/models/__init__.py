@@ -1,5 +1,5 @@
 from .inception_v3 import inception_v3
-from .randwire import randwire_small, randwire_large
+from .randwire import randwire_small, randwire_large, randwire_xlarge
 from .squeezenet import squeezenet, squeezenet_1_1
 from .nasnet import nasnet_mobile, nasnet_large
 from .sample import sample_network

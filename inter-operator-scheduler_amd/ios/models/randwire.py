@@ -10,9 +10,12 @@ generator; here ``watts_strogatz_edges`` generates them from a seed and ``read_g
 file format (line 1: n, line 2: m, then m lines "u v" with u < v).
 
 ``randwire_small`` is the configuration with three stages of 32 nodes (k=4, p=0.75) and 78/156/312
-channels behind the two-convolution small front; ``randwire_large`` mirrors the reference's large
-model (:72-87) with generated graphs.
+channels behind the two-convolution small front, on graphs from the seeded generator.  ``randwire_large``
+(:72-87) and ``randwire_xlarge`` (:89-101) are the reference's models on the reference's own edge lists
+(``randwire_graphs/generated/*.txt``, shipped as data); with ``graph_seeds`` the large model takes generated
+graphs of the same parameters instead.
 """
+import os
 from typing import List, Sequence, Tuple
 
 import numpy as np
@@ -21,6 +24,7 @@ from .common import (Block, Graph, Value, conv2d, identity, placeholder, pool2d,
                      rwconv2d)
 
 Edges = List[Tuple[int, int]]
+graph_dir = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'randwire_graphs', 'generated')
 
 
 def watts_strogatz_edges(n: int, k: int, p: float, seed: int) -> Edges:
@@ -111,13 +115,14 @@ def randwire_stage(r: Value, ch: int, n: int, edges: Sequence[Tuple[int, int]]):
     return identity(block, [sinks], is_exit=True), block
 
 
-def _randwire(name, front, front_ch, stage_specs, init_seed, init_scheme):
+def _randwire(name, front, front_ch, stages, init_seed, init_scheme):
+    """``stages``: (channels, number of nodes, edges) per stage."""
     reset_name()
     pv = placeholder(output_shape=(3, 224, 224))
     v, block = front(pv, front_ch)
     blocks = [block]
-    for ch, n, k, p, seed in stage_specs:
-        v, block = randwire_stage(v, ch, n, watts_strogatz_edges(n, k, p, seed))
+    for ch, n, edges in stages:
+        v, block = randwire_stage(v, ch, n, edges)
         blocks.append(block)
     v, block = randwire_tail(v)
     blocks.append(block)
@@ -128,11 +133,27 @@ def _randwire(name, front, front_ch, stage_specs, init_seed, init_scheme):
 
 def randwire_small(init_seed=None, init_scheme='uniform', graph_seeds=(3, 4, 5)) -> Graph:
     ch = 78
-    specs = [(ch << i, 32, 4, 0.75, graph_seeds[i]) for i in range(3)]
-    return _randwire("randwire_small", randwire_small_front, ch, specs, init_seed, init_scheme)
+    stages = [(ch << i, 32, watts_strogatz_edges(32, 4, 0.75, graph_seeds[i])) for i in range(3)]
+    return _randwire("randwire_small", randwire_small_front, ch, stages, init_seed, init_scheme)
 
 
-def randwire_large(init_seed=None, init_scheme='uniform', graph_seeds=(2, 3, 4, 5)) -> Graph:
+def randwire_large(init_seed=None, init_scheme='uniform', graph_seeds=None) -> Graph:
+    """
+    The reference's large model (154 / 308 / 616 / 1232 channels on graphs of 16, 32, 32, 32 nodes) on its own edge lists;
+    ``graph_seeds`` (four seeds) replaces them by generated graphs with the same parameters.
+    """
     ch = 154
-    specs = [(ch, 16, 4, 0.75, graph_seeds[0])] + [(ch << i, 32, 4, 0.75, graph_seeds[i]) for i in (1, 2, 3)]
-    return _randwire("randwire_large", randwire_regular_front, ch, specs, init_seed, init_scheme)
+    if graph_seeds is None:
+        files = ['ws-16-4-0.75-2.txt', 'ws-32-4-0.75-3.txt', 'ws-32-4-0.75-4.txt', 'ws-32-4-0.75-5.txt']
+        graphs = [read_graph(os.path.join(graph_dir, fname)) for fname in files]
+    else:
+        graphs = [(n, watts_strogatz_edges(n, 4, 0.75, seed)) for n, seed in zip((16, 32, 32, 32), graph_seeds)]
+    stages = [(ch << i, n, edges) for i, (n, edges) in enumerate(graphs)]
+    return _randwire("randwire_large", randwire_regular_front, ch, stages, init_seed, init_scheme)
+
+
+def randwire_xlarge(init_seed=None, init_scheme='uniform') -> Graph:
+    """One stage of 320 nodes (k = 20) at 154 channels: the graph the reference counts schedule-search states on."""
+    ch = 154
+    n, edges = read_graph(os.path.join(graph_dir, 'ws-320-20-0.75-x.txt'))
+    return _randwire("randwire_xlarge", randwire_regular_front, ch, [(ch, n, edges)], init_seed, init_scheme)

@@ -201,6 +201,35 @@ def test_randwire_graph_generator_is_seeded_and_valid():
     assert watts_strogatz_edges(8, 2, 0.0, seed=0) == sorted([(i, i + 1) for i in range(7)] + [(0, 7)])
 
 
+def test_reference_randwire_graphs_and_the_models_built_on_them():
+    """
+    The edge lists the reference ships (python/ios/models/randwire_graphs/generated/, kept as data beside the model code):
+    32-node graphs with 64 edges, largest fan-in 6 / 8 / 5 / 5 over the four stages of the large model (sums of more than five
+    values are what the reference adds with repeated cudnnAddTensor calls, src/ios/ios_runtime.cu:746-751), and the 320-node
+    graph of the extra-large model.
+    """
+    from ios.models.randwire import graph_dir, read_graph
+    fan_in = []
+    for fname, nodes, count in (('ws-16-4-0.75-2.txt', 16, 32), ('ws-32-4-0.75-3.txt', 32, 64), ('ws-32-4-0.75-4.txt', 32, 64),
+                                ('ws-32-4-0.75-5.txt', 32, 64), ('ws-320-20-0.75-x.txt', 320, 3200)):
+        n, edges = read_graph(os.path.join(graph_dir, fname))
+        assert n == nodes and len(edges) == count and all(0 <= u < v < n for u, v in edges) and len(set(edges)) == count
+        degree = [0] * n
+        for _, v in edges:
+            degree[v] += 1
+        fan_in.append(max(degree))
+    assert fan_in[:4] == [6, 8, 5, 5] and fan_in[4] > 8
+    large = ios.models.randwire_large()
+    assert [tuple(b.exit_node.output_shape) for b in large.blocks] == [(77, 112, 112), (154, 56, 56), (308, 28, 28), (616, 14, 14),
+                                                                        (1232, 7, 7), (1280, 1, 1)]
+    assert [len(b.inner_nodes) + 1 for b in large.blocks[1:5]] == [17, 33, 33, 33]      # nodes + the summing exit
+    assert max(len(n.nodes[0].inputs[0]) for b in large.blocks[1:5] for n in b.inner_nodes) == 8
+    seeded = ios.models.randwire_large(graph_seeds=(2, 3, 4, 5))                          # generated graphs, same parameters
+    assert [tuple(b.exit_node.output_shape) for b in seeded.blocks] == [tuple(b.exit_node.output_shape) for b in large.blocks]
+    xlarge = ios.models.randwire_xlarge()
+    assert len(xlarge.blocks) == 3 and len(xlarge.blocks[1].inner_nodes) == 320 and tuple(xlarge.exit_node.output_shape) == (1280, 1, 1)
+
+
 def test_randwire_edge_file_format(tmp_path):
     from ios.models.randwire import watts_strogatz_edges, read_graph, write_graph
     edges = watts_strogatz_edges(16, 4, 0.75, seed=2)
