@@ -10,12 +10,10 @@ generator; here ``watts_strogatz_edges`` generates them from a seed and ``read_g
 file format (line 1: n, line 2: m, then m lines "u v" with u < v).
 
 ``randwire_small`` is the configuration with three stages of 32 nodes (k=4, p=0.75) and 78/156/312
-channels behind the two-convolution small front, on graphs from the seeded generator.  ``randwire_large``
-(:72-87) and ``randwire_xlarge`` (:89-101) are the reference's models on the reference's own edge lists
-(``randwire_graphs/generated/*.txt``, shipped as data); with ``graph_seeds`` the large model takes generated
-graphs of the same parameters instead.
+channels behind the two-convolution small front.  ``randwire_large`` (:72-87) and ``randwire_xlarge``
+(:89-101) are the reference's models; their graphs come from the seeded generator with the reference's
+parameters, or from edge-list files in the reference's format (``graph_files`` / ``graph_file``).
 """
-import os
 from typing import List, Sequence, Tuple
 
 import numpy as np
@@ -24,7 +22,6 @@ from .common import (Block, Graph, Value, conv2d, identity, placeholder, pool2d,
                      rwconv2d)
 
 Edges = List[Tuple[int, int]]
-graph_dir = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'randwire_graphs', 'generated')
 
 
 def watts_strogatz_edges(n: int, k: int, p: float, seed: int) -> Edges:
@@ -137,23 +134,24 @@ def randwire_small(init_seed=None, init_scheme='uniform', graph_seeds=(3, 4, 5))
     return _randwire("randwire_small", randwire_small_front, ch, stages, init_seed, init_scheme)
 
 
-def randwire_large(init_seed=None, init_scheme='uniform', graph_seeds=None) -> Graph:
+def randwire_large(init_seed=None, init_scheme='uniform', graph_seeds=(2, 3, 4, 5), graph_files=None) -> Graph:
     """
-    The reference's large model (154 / 308 / 616 / 1232 channels on graphs of 16, 32, 32, 32 nodes) on its own edge lists;
-    ``graph_seeds`` (four seeds) replaces them by generated graphs with the same parameters.
+    The reference's large model: 154 / 308 / 616 / 1232 channels on graphs of 16, 32, 32, 32 nodes (k = 4, p = 0.75), which
+    are generated from ``graph_seeds`` or read from the four edge-list files ``graph_files``.
     """
     ch = 154
-    if graph_seeds is None:
-        files = ['ws-16-4-0.75-2.txt', 'ws-32-4-0.75-3.txt', 'ws-32-4-0.75-4.txt', 'ws-32-4-0.75-5.txt']
-        graphs = [read_graph(os.path.join(graph_dir, fname)) for fname in files]
+    if graph_files is not None:
+        graphs = [read_graph(fname) for fname in graph_files]
     else:
         graphs = [(n, watts_strogatz_edges(n, 4, 0.75, seed)) for n, seed in zip((16, 32, 32, 32), graph_seeds)]
+    if len(graphs) != 4:
+        raise ValueError('randwire_large has four stages')
     stages = [(ch << i, n, edges) for i, (n, edges) in enumerate(graphs)]
     return _randwire("randwire_large", randwire_regular_front, ch, stages, init_seed, init_scheme)
 
 
-def randwire_xlarge(init_seed=None, init_scheme='uniform') -> Graph:
-    """One stage of 320 nodes (k = 20) at 154 channels: the graph the reference counts schedule-search states on."""
+def randwire_xlarge(init_seed=None, init_scheme='uniform', graph_seed=0, graph_file=None) -> Graph:
+    """One stage of 320 nodes (k = 20, p = 0.75) at 154 channels: the graph the reference counts schedule-search states on."""
     ch = 154
-    n, edges = read_graph(os.path.join(graph_dir, 'ws-320-20-0.75-x.txt'))
+    n, edges = read_graph(graph_file) if graph_file is not None else (320, watts_strogatz_edges(320, 20, 0.75, graph_seed))
     return _randwire("randwire_xlarge", randwire_regular_front, ch, [(ch, n, edges)], init_seed, init_scheme)

@@ -7,6 +7,8 @@ by the tensor's largest magnitude and reports how many elements miss the unscale
 Whole networks run with seeded non-zero biases.  With the kernel configuration pinned, schedule and executor
 changes must not change results at all.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -673,8 +675,9 @@ ZOO = [
     ('resnet18', lambda: ios.models.resnet18(init_seed=0, init_scheme='bn_folded'), 2, 8),
     ('resnet34', lambda: ios.models.resnet34(init_seed=0, init_scheme='bn_folded'), 1, 16),
     ('resnet50', lambda: ios.models.resnet50(init_seed=0, init_scheme='bn_folded'), 1, 32),
-    # one stage of 320 nodes on the reference's own edge list: sums of up to 33 values, in chunks of eight
-    ('randwire_xlarge', lambda: ios.models.randwire_xlarge(init_seed=0, init_scheme='bn_folded'), 1, 1),
+    # one stage of 320 nodes on the reference's own edge list (a fixture): sums of up to 33 values, in chunks of eight
+    ('randwire_xlarge', lambda: ios.models.randwire_xlarge(init_seed=0, init_scheme='bn_folded', graph_file=os.path.join(
+        os.path.dirname(__file__), 'golden', 'randwire_graphs', 'ws-320-20-0.75-x.txt')), 1, 1),
 ]
 
 

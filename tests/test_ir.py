@@ -203,12 +203,13 @@ def test_randwire_graph_generator_is_seeded_and_valid():
 
 def test_reference_randwire_graphs_and_the_models_built_on_them():
     """
-    The edge lists the reference ships (python/ios/models/randwire_graphs/generated/, kept as data beside the model code):
+    The edge lists the reference ships (python/ios/models/randwire_graphs/generated/, kept as fixtures under tests/golden/):
     32-node graphs with 64 edges, largest fan-in 6 / 8 / 5 / 5 over the four stages of the large model (sums of more than five
     values are what the reference adds with repeated cudnnAddTensor calls, src/ios/ios_runtime.cu:746-751), and the 320-node
     graph of the extra-large model.
     """
-    from ios.models.randwire import graph_dir, read_graph
+    from ios.models.randwire import read_graph
+    graph_dir = os.path.join(GOLDEN, 'randwire_graphs')
     fan_in = []
     for fname, nodes, count in (('ws-16-4-0.75-2.txt', 16, 32), ('ws-32-4-0.75-3.txt', 32, 64), ('ws-32-4-0.75-4.txt', 32, 64),
                                 ('ws-32-4-0.75-5.txt', 32, 64), ('ws-320-20-0.75-x.txt', 320, 3200)):
@@ -219,14 +220,17 @@ def test_reference_randwire_graphs_and_the_models_built_on_them():
             degree[v] += 1
         fan_in.append(max(degree))
     assert fan_in[:4] == [6, 8, 5, 5] and fan_in[4] > 8
-    large = ios.models.randwire_large()
+    files = [os.path.join(graph_dir, f) for f in ('ws-16-4-0.75-2.txt', 'ws-32-4-0.75-3.txt', 'ws-32-4-0.75-4.txt', 'ws-32-4-0.75-5.txt')]
+    large = ios.models.randwire_large(graph_files=files)
     assert [tuple(b.exit_node.output_shape) for b in large.blocks] == [(77, 112, 112), (154, 56, 56), (308, 28, 28), (616, 14, 14),
                                                                         (1232, 7, 7), (1280, 1, 1)]
     assert [len(b.inner_nodes) + 1 for b in large.blocks[1:5]] == [17, 33, 33, 33]      # nodes + the summing exit
     assert max(len(n.nodes[0].inputs[0]) for b in large.blocks[1:5] for n in b.inner_nodes) == 8
-    seeded = ios.models.randwire_large(graph_seeds=(2, 3, 4, 5))                          # generated graphs, same parameters
+    seeded = ios.models.randwire_large()                                                   # generated graphs, same parameters
     assert [tuple(b.exit_node.output_shape) for b in seeded.blocks] == [tuple(b.exit_node.output_shape) for b in large.blocks]
-    xlarge = ios.models.randwire_xlarge()
+    xlarge = ios.models.randwire_xlarge(graph_file=os.path.join(graph_dir, 'ws-320-20-0.75-x.txt'))
+    generated = ios.models.randwire_xlarge()
+    assert len(generated.blocks[1].inner_nodes) == 320 and generated.blocks[1].exit_node.output_shape == xlarge.blocks[1].exit_node.output_shape
     assert len(xlarge.blocks) == 3 and len(xlarge.blocks[1].inner_nodes) == 320 and tuple(xlarge.exit_node.output_shape) == (1280, 1, 1)
 
 
