@@ -133,6 +133,6 @@ def nasnet_mobile(init_seed=None, init_scheme='uniform') -> Graph:
     return nasnet("nasnet_mobile", 224, 32, 44, 4, init_seed, init_scheme)
 
 
-def nasnet_large(init_seed=None, init_scheme='uniform') -> Graph:
-    """NASNet-A large, 6 @ 4032, 3x331x331 input."""
-    return nasnet("nasnet_large", 331, 96, 168, 6, init_seed, init_scheme)
+def nasnet_large(stem_filters=96, filters=168, init_seed=None, init_scheme='uniform') -> Graph:
+    """NASNet-A large, 6 @ 4032, 3x331x331 input (parameters of reference python/ios/models/nasnet.py:138)."""
+    return nasnet("nasnet_large", 331, stem_filters, filters, 6, init_seed, init_scheme)
