@@ -98,7 +98,9 @@ def normal_cell(block, x: Value, x_prev: Value, out_channels_left, out_channels_
 def nasnet(name, input_size, stem_filters, filters, cells_per_stack, init_seed=None, init_scheme='uniform') -> Graph:
     """
     NASNet-A with ``cells_per_stack`` cells (one first cell + normal cells) in each of the three stacks
-    and ``filters`` channels per branch in the first stack; the final feature map has 24*filters channels.
+    and ``filters`` channels per branch in the first stack; the final feature map has 20*filters channels (the
+    reference's normal cell concatenates five sums, python/ios/models/nasnet.py:112, where the published cell also
+    passes one of its inputs through: 880 instead of 1056 channels for the mobile model, 3360 instead of 4032 for the large one).
     Every cell output is a split point of ``block.parts``.
     """
     reset_name()
