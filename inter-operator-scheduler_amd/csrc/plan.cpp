@@ -449,9 +449,9 @@ private:
 
     // "convolution, + skip value (, ReLU)" of a residual unit (reference python/ios/models/resnet.py:10-27): when the
     // convolution's output is read by the addition only, the skip value is complete before the convolution starts, the
-    // convolution has its stage to itself and takes the matrix path, its epilogue adds the skip value (and applies the ReLU) and the addition's launch
-    // and the convolution's own tensor disappear.  The rounding is that of the separate launches: act(conv + bias) is
-    // rounded to fp32 before the skip value is added.
+    // convolution has its stage to itself and takes the matrix path, its epilogue adds the skip value (and applies the
+    // ReLU) and the addition's launch and the convolution's own tensor disappear.  The rounding is that of the separate
+    // launches: act(conv + bias) is rounded to fp32 before the skip value is added.
     void find_residual_convolutions() {
         for (size_t i = 0; i < nodes_.size(); i++) {
             PNode &e = nodes_[i];

@@ -62,7 +62,7 @@ def random_block(rng, enter, downsample, wide=1):
             base = ios.conv2d(block, [[enter]], wide * int(rng.integers(4, 17)), (3, 3), (2, 2), (1, 1), 1, _pick(rng, ['relu', 'identity']))
         values = [base]
     for _ in range(int(rng.integers(4, 11))):
-        kind = _pick(rng, ['conv', 'conv', 'conv', 'sibling', 'depthwise', 'grouped', 'pool', 'relu', 'activation', 'element', 'sum', 'concat', 'separable'])
+        kind = _pick(rng, ['conv', 'conv', 'conv', 'sibling', 'residual', 'depthwise', 'grouped', 'pool', 'relu', 'activation', 'element', 'sum', 'concat', 'separable'])
         if kind == 'conv':
             terms = _terms(rng, values)
             k = _pick(rng, [(1, 1), (1, 1), (3, 3), (3, 3), (1, 3), (3, 1), (5, 5)])
@@ -76,6 +76,14 @@ def random_block(rng, enter, downsample, wide=1):
             twin = _pick(rng, convs)
             k = _pick(rng, [tuple(twin.kernel), (1, 1), (3, 3), (1, 3), (3, 1)])
             out = ios.conv2d(block, [list(term) for term in twin.inputs], wide * int(rng.integers(3, 17)), k, tuple(twin.stride), (k[0] // 2, k[1] // 2), 1, twin.act)
+        elif kind == 'residual':
+            # convolution, + an earlier value of the same width (, ReLU): what a convolution's epilogue can take over
+            skip = _pick(rng, values)
+            k = _pick(rng, [(1, 1), (3, 3)])
+            y = ios.conv2d(block, _terms(rng, values), skip.length, k, (1, 1), (k[0] // 2, k[1] // 2), 1, _pick(rng, ['identity', 'identity', 'relu']))
+            out = ios.addition(block, [[y, skip] if rng.random() < 0.5 else [skip, y]])
+            if rng.random() < 0.6:
+                out = ios.activation(block, [[out]], _pick(rng, ['relu', 'relu', 'tanh']), bool(rng.integers(2)))
         elif kind == 'depthwise':
             terms = _terms(rng, values, max_terms=1, max_summed=4)
             k = _pick(rng, [3, 3, 5, 7])
