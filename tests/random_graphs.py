@@ -1,9 +1,9 @@
 """
 Seeded random networks for the planner and parity tests: small blocks that mix every operator kind the runtime knows
 (convolutions with all activations, grouped and depth-wise ones, pools, ReLU / activation nodes, two-operand additions and
-products, sums, concatenations, channel slices, separable units) in random wiring, so that the planner's rewrites (folded
-ReLUs, concatenations written in place, sums in depth-wise loaders, additions absorbed by activations or by a convolution's
-epilogue) meet each other in combinations no hand-written case holds.
+products, sums, concatenations, channel slices, separable units, sibling convolutions, residual units) in random wiring,
+so that the planner's rewrites (folded ReLUs, concatenations written in place, sums in depth-wise loaders, additions
+absorbed by activations or by a convolution's epilogue) meet each other in combinations no hand-written case holds.
 """
 import numpy as np
 
