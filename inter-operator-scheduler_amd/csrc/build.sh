@@ -7,11 +7,12 @@ mkdir -p build
 # starts), which takes one scalar-load round trip out of every fused launch
 FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclang -packed-fp32-ops -mllvm -amdgpu-mfma-vgpr-form=1 -mllvm -amdgpu-kernarg-preload-count=16 -Wno-unused-result"
 # The stand-alone convolution kernels are scheduled for instruction-level parallelism (more of a K step's loads ahead of its
-# MFMAs): 0.3 % of an Inception-v3 pass in same-device A/B runs with identical kernel configurations.  Not for the fused stage
-# kernel: there it spills in the 1024-thread form and slows the memory-bound bodies (NASNet +0.8 %).
-declare -A FILE_FLAGS=([conv_mfma.hip]="-mllvm -amdgpu-sched-strategy=max-ilp")
+# MFMAs): 0.3 % of an Inception-v3 pass in same-device A/B runs with identical kernel configurations.  The same for the
+# 512-thread form of the fused stage kernel, which holds most convolution levels (another 0.4 % there and on NASNet); the other
+# two forms spill or slow the memory-bound bodies down with it (NASNet +0.8 %), so they keep the default.
+declare -A FILE_FLAGS=([conv_mfma.hip]="-mllvm -amdgpu-sched-strategy=max-ilp" [fused_512.hip]="-mllvm -amdgpu-sched-strategy=max-ilp")
 pids=()
-for src in conv_mfma.hip pointwise.hip fused.hip runtime.hip c_api.hip; do
+for src in conv_mfma.hip pointwise.hip fused.hip fused_512.hip runtime.hip c_api.hip; do
     # the resource remarks go to a log: a kernel that spills registers to scratch memory is reported below
     hipcc $FLAGS ${FILE_FLAGS[$src]:-} -Rpass-analysis=kernel-resource-usage -c "$src" -o "build/${src%.hip}.o" 2> "build/${src%.hip}.log" &
     pids+=($!)
@@ -28,5 +29,5 @@ if grep -h "ScratchSize \[bytes/lane\]: [1-9]" build/*.log > /dev/null; then
     echo "warning: kernels spilling to scratch memory:" >&2
     grep -h -B4 "ScratchSize \[bytes/lane\]: [1-9]" build/*.log | grep "Function Name" | sed 's/.*Function Name: /  /; s/ \[-R.*//' >&2
 fi
-hipcc --offload-arch=gfx950 -shared -fPIC -o build/libios_runtime.so build/conv_mfma.o build/pointwise.o build/fused.o build/runtime.o build/c_api.o build/plan.o
+hipcc --offload-arch=gfx950 -shared -fPIC -o build/libios_runtime.so build/conv_mfma.o build/pointwise.o build/fused.o build/fused_512.o build/runtime.o build/c_api.o build/plan.o
 echo "built $(pwd)/build/libios_runtime.so"

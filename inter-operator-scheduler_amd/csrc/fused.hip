@@ -1,113 +1,10 @@
 // The fused stage kernel: see fused.h.
-#include "fused.h"
+#include "fused_kernel.h"
 
 #include <climits>
 #include <stdexcept>
 
 namespace ios {
-
-// The first blocks of the items travel as scalar kernel arguments (b1 ... b7; item 0 starts at block 0): with
-// -amdgpu-kernarg-preload-count the command processor hands them to a wavefront in registers, so a block knows its item
-// without a load and its first load is the item itself.
-template <int T>
-__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fused_kernel(const WorkItem *__restrict__ items, int num_items, int b1, int b2,
-                                                                                            int b3, int b4, int b5, int b6, int b7) {
-    extern __shared__ floatx4 fused_smem[];
-    float *smem = reinterpret_cast<float *>(fused_smem);
-    const int bid = blockIdx.x;
-    FusedHeader header;
-    header.num_items = num_items;
-    header.first_block[0] = 0;
-    header.first_block[1] = b1; header.first_block[2] = b2; header.first_block[3] = b3; header.first_block[4] = b4;
-    header.first_block[5] = b5; header.first_block[6] = b6; header.first_block[7] = b7;
-    int index = 0;   // number of further items that start at or before this block
-    if (header.num_items <= kFusedHeaderItems) {
-#pragma unroll
-        for (int i = 1; i < kFusedHeaderItems; i++) index += bid >= header.first_block[i] ? 1 : 0;   // unused entries are INT_MAX
-    } else {
-        while (index + 1 < header.num_items && bid >= items[index + 1].first_block) index++;
-    }
-    const WorkItem &item = items[index];
-    // An item spans five 64-byte lines of the scalar cache, and the bodies read its fields in two or three dependent steps
-    // (kind, then configuration, then arguments): one word of every line is requested together with the first step, so
-    // that the later steps find their lines in the cache instead of paying a miss each.  The comparison below never
-    // holds (first_block is not negative) and only keeps the compiler from dropping the loads.
-    {
-        const int *words = reinterpret_cast<const int *>(&item);
-        int touched = 0;
-#pragma unroll
-        for (int line = 1; line * 16 < (int)(sizeof(WorkItem) / sizeof(int)); line++) touched |= words[line * 16];
-        if (item.first_block == -1 && touched == 0x5a5a5a5a) return;
-    }
-    const int local = bid - item.first_block;
-    const int num_blocks = item.num_blocks;
-    switch (item.kind) {
-        case WORK_CONV: {
-            if ((int)threadIdx.x >= item.threads) return;   // surplus wavefronts of a narrower body
-            const ConvKernelArgs &a = item.conv;   // fields are fetched with scalar loads where they are used
-            const int rest = (int)fast_div((unsigned)local, item.div_tiles);
-            const int tile = local - rest * item.tiles;
-            const int z = (int)fast_div((unsigned)rest, item.div_groups);
-            const int g = rest - z * item.groups;
-            switch (item.variant) {
-#define IOS_CASE_TILED(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                          \
-    case IDX:                                                                                              \
-        if constexpr (64 * WM * WN * WK <= T && ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::FUSABLE)                   \
-            ConvTiled<BM, BN, BK, WM, WN, WK, MT, PD>::run(a, smem, tile, g, z);                                      \
-        break;
-#define IOS_CASE_WSPLIT(IDX, NAME, MT, TM, TN, NW, U, QUAD, D, BF16)                                        \
-    case IDX:                                                                                      \
-        if constexpr (64 * NW <= T && ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::FUSABLE)              \
-            ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16>::run(a, smem, tile, g, z);                       \
-        break;
-#define IOS_CASE_WSPLIT_C4(IDX, NAME, MT, TM, TN, NW, U, QUAD, D, BF16)                                     \
-    case IDX:                                                                                      \
-        if constexpr (64 * NW <= T && ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::FUSABLE)           \
-            ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::run(a, smem, tile, g, z);                    \
-        break;
-                IOS_TILED_VARIANTS(IOS_CASE_TILED)
-                IOS_WSPLIT_VARIANTS(IOS_CASE_WSPLIT)
-                IOS_WSPLIT_C4_VARIANTS(IOS_CASE_WSPLIT_C4)
-                IOS_WSPLIT_T32_VARIANTS(IOS_CASE_WSPLIT)
-                IOS_WSPLIT_F16_VARIANTS(IOS_CASE_WSPLIT)
-#undef IOS_CASE_WSPLIT_C4
-#undef IOS_CASE_TILED
-#undef IOS_CASE_WSPLIT
-                default: break;
-            }
-            break;
-        }
-        case WORK_REDUCE: {
-            const ReduceArgs a = item.reduce;
-            splitk_reduce_body(a, local, num_blocks);
-            break;
-        }
-        case WORK_POOL: {
-            const PoolArgs a = item.pool;
-            pool_body(a, local, num_blocks);
-            break;
-        }
-        case WORK_GLOBAL_POOL: {
-            const PoolArgs a = item.pool;
-            global_pool_body(a, local, num_blocks);
-            break;
-        }
-        case WORK_DWCONV: {
-            dwconv_dispatch(item.direct, local, num_blocks);   // (the table of summed inputs is read in place)
-            break;
-        }
-        case WORK_CONV_DIRECT: {
-            const DirectConvArgs a = item.direct;
-            conv_direct_body(a, local, num_blocks);
-            break;
-        }
-        case WORK_NARY: {
-            nary_dispatch(item.nary, local, num_blocks);   // read in place: the source table is indexed dynamically
-            break;
-        }
-        default: break;
-    }
-}
 
 void launch_fused(int threads, const WorkItem *device_items, const FusedHeader &header, int total_blocks, int smem_bytes, hipStream_t stream) {
     if (header.num_items < 1 || header.num_items > kMaxFusedItems || total_blocks < 1) throw std::runtime_error("fused launch: bad item count");
@@ -119,9 +16,7 @@ void launch_fused(int threads, const WorkItem *device_items, const FusedHeader &
         case 256:
             hipLaunchKernelGGL(fused_kernel<256>, grid, dim3(256), smem_bytes, stream, device_items, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7]);
             break;
-        case 512:
-            hipLaunchKernelGGL(fused_kernel<512>, grid, dim3(512), smem_bytes, stream, device_items, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7]);
-            break;
+        case 512: launch_fused_512(device_items, header.num_items, b, total_blocks, smem_bytes, stream); break;
         case 1024:
             hipLaunchKernelGGL(fused_kernel<1024>, grid, dim3(1024), smem_bytes, stream, device_items, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7]);
             break;
