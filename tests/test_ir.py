@@ -277,6 +277,27 @@ def test_value_and_uses():
     assert b.node.input_readable_str() == '(1+0)'
 
 
+def test_draw_writes_graphviz_source_without_pydot(tmp_path):
+    from ios.visualizer import to_dot
+    graph = ios.models.sample_network()
+    graph.blocks[0].stages = [[['1'], ['2']], [['4'], ['3']], [['5']]]
+    source = to_dot(graph, label='demo')
+    assert source.startswith('digraph') and source.count('->') == 7 and 'subgraph cluster_0' in source
+    for name, stage in (('1', 0), ('2', 0), ('4', 1), ('3', 1), ('5', 2)):
+        assert f'{name} @ stage {stage}' in source
+    assert source.count('fillcolor=lightblue') == 2      # the two operators of the first stage share a colour
+    target = ios.draw(graph, str(tmp_path / 'demo.gv'), label='demo')
+    assert open(target).read() == source
+    # slices and summed values are marked on their edges; every operator of a large network is drawn once
+    nasnet = ios.models.nasnet_mobile()
+    nasnet.greedy_schedule(8)
+    text = to_dot(nasnet)
+    assert text.count('arrowhead=odot') > 50 and sum(1 for line in text.splitlines() if 'fillcolor=' in line and '->' not in line) == \
+           1 + sum(len(b.inner_nodes) + 1 for b in nasnet.blocks)
+    merged = Graph.from_config(json.load(open(os.path.join(GOLDEN, 'inception_v3_dp_parallel_merge.json'))))
+    assert '[' in to_dot(merged) and ':' in to_dot(merged)      # channel slices of merged convolutions
+
+
 def test_unknown_node_type_raises():
     with pytest.raises(ValueError):
         ios.ir.Node.from_config({'type': 'softmax', 'name': 'x', 'hint_name': 'x', 'inputs': [], 'output_shape': None}, {})
