@@ -506,6 +506,14 @@ def main():
                 scheduled.greedy_schedule(4)
                 label = 'greedy'
                 search_c = 0.0
+            other_ms = None
+            if search and label == 'dp_parallel' and group_size != 1:
+                # the small networks are searched in a fraction of a second: the r = 1 search beside the default one
+                rt.set_option('executor', args.search_executor)
+                single = ios.optimize(g, batch_size=1, cost_model=ios.IOSCostModel(share_identical_stages=True), opt_type='dp_parallel',
+                                      compute_weight=True, warmup=2, number=6, repeat=3, max_group_size=1, max_num_groups=args.max_num_groups)
+                rt.set_option('executor', args.executor)
+                other_ms = timed_latency(rt, np, single, 1, xc, 100, 10)[0]['wall']
             g.sequential_schedule()
             c_seq, _ = timed_latency(rt, np, g, 1, xc, 100, 10)
             c_par, c_out = timed_latency(rt, np, scheduled, 1, xc, 100, 10)
@@ -518,6 +526,8 @@ def main():
                              'fraction_of_network_roofline': network_roofline_ms(ops_c, parallel=False) / c_par['wall'],
                              'roofline': roofline_block(kernels_c, c_par['wall']),
                              'memory_bound_ops_gbs': memory_bound_ops(rt, g, 1, xc)}
+            if other_ms is not None:
+                configs[name]['dp_parallel_r1_ms'] = other_ms
             rt.set_option('executor', args.executor)
             if not args.no_cpu:
                 configs[name]['oracle'] = oracle_check(np, c_out, ios_oracle.run(g, xc))
