@@ -488,9 +488,9 @@ struct ReduceArgs {
     int res_bs, post_relu;
 };
 
-__device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int block, int num_blocks) {
+__device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int block, int num_blocks, unsigned threads) {
     const long long total = (long long)a.OC * a.Npix;
-    for (long long i = block * (long long)blockDim.x + threadIdx.x; i < total; i += (long long)num_blocks * blockDim.x) {
+    for (long long i = block * (long long)threads + threadIdx.x; i < total; i += (long long)num_blocks * threads) {
         const int oc = (int)(i / a.Npix);
         const int n = (int)(i - (long long)oc * a.Npix);
         float sum = 0.f;

@@ -16,7 +16,7 @@ __global__ __launch_bounds__(Body::THREADS) void conv_kernel(ConvKernelArgs a) {
     Body::template run<RES>(a, reinterpret_cast<float *>(conv_smem), blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
-__global__ void splitk_reduce_kernel(ReduceArgs a) { splitk_reduce_body(a, blockIdx.x, gridDim.x); }
+__global__ void splitk_reduce_kernel(ReduceArgs a) { splitk_reduce_body(a, blockIdx.x, gridDim.x, blockDim.x); }
 
 // ---- variant table --------------------------------------------------------------------------------------------
 typedef void (*ConvKernelFn)(ConvKernelArgs);

@@ -44,7 +44,11 @@ struct FusedHeader {
 // wavefronts that have not ended), the memory-bound bodies adapt to any block size.
 constexpr int kFusedThreadClasses[] = {256, 512, 1024};
 
-// Launch `num_items` items (device pointer) as one grid of `total_blocks` blocks of `threads` threads.
-void launch_fused(int threads, const WorkItem *device_items, const FusedHeader &header, int total_blocks, int smem_bytes, hipStream_t stream);
+// Launch `num_items` items as one grid of `total_blocks` blocks of `threads` threads.  `device_items` is the table in device
+// memory; `host_items` (the same items on the host, or null) lets launches that qualify carry their items in the
+// kernel-argument segment instead (fused_kernel.h).
+// Whether a launch of these items (host copies) takes the form with the items in the kernel-argument segment.
+bool fused_items_inline(const WorkItem *host_items, int num_items);
+void launch_fused(int threads, const WorkItem *device_items, const WorkItem *host_items, const FusedHeader &header, int total_blocks, int smem_bytes, hipStream_t stream);
 
 }  // namespace ios

@@ -8,15 +8,15 @@
 
 namespace ios {
 
-__global__ void pool_kernel(PoolArgs a) { pool_body(a, blockIdx.x, gridDim.x); }
-__global__ void global_pool_kernel(PoolArgs a) { global_pool_body(a, blockIdx.x, gridDim.x); }
-__global__ void dwconv_kernel(DirectConvArgs a) { dwconv_dispatch(a, blockIdx.x, gridDim.x); }
-__global__ void conv_direct_kernel(DirectConvArgs a) { conv_direct_body(a, blockIdx.x, gridDim.x); }
+__global__ void pool_kernel(PoolArgs a) { pool_body(a, blockIdx.x, gridDim.x, blockDim.x); }
+__global__ void global_pool_kernel(PoolArgs a) { global_pool_body(a, blockIdx.x, gridDim.x, blockDim.x); }
+__global__ void dwconv_kernel(DirectConvArgs a) { dwconv_dispatch(a, blockIdx.x, gridDim.x, blockDim.x); }
+__global__ void conv_direct_kernel(DirectConvArgs a) { conv_direct_body(a, blockIdx.x, gridDim.x, blockDim.x); }
 __global__ __launch_bounds__(256) void conv_thin_kernel(DirectConvArgs a) {
     __shared__ float filters[kThinConvSmemFloats];
     conv_thin_body(a, filters, blockIdx.x, gridDim.x);
 }
-__global__ void nary_kernel(NaryKernelArgs a) { nary_dispatch(a, blockIdx.x, gridDim.x); }
+__global__ void nary_kernel(NaryKernelArgs a) { nary_dispatch(a, blockIdx.x, gridDim.x, blockDim.x); }
 
 static int blocks_for(long long n, int per_block, int cap) {
     return (int)std::max<long long>(1, std::min<long long>((n + per_block - 1) / per_block, cap));

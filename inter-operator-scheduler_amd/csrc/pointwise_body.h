@@ -28,14 +28,14 @@ struct PoolArgs {
     int vec_columns;  // 3 x 3 windows: output columns per thread, 1 or kPoolVecColumns (see pool3x3_vec_body)
 };
 
-__device__ __forceinline__ void pool_generic_body(const PoolArgs &a, int block, int num_blocks) {
+__device__ __forceinline__ void pool_generic_body(const PoolArgs &a, int block, int num_blocks, unsigned threads) {
     const PoolProblem &p = a.p;
     // 32-bit index arithmetic: the host side rejects tensors with 2^31 or more elements
     const unsigned plane = (unsigned)(p.OH * p.OW);
     const unsigned per_image = (unsigned)p.C * plane;
     const unsigned total = per_image * (unsigned)p.B;
     const float inv = 1.0f / (float)(p.KH * p.KW);
-    for (unsigned i = block * blockDim.x + threadIdx.x; i < total; i += num_blocks * blockDim.x) {
+    for (unsigned i = block * threads + threadIdx.x; i < total; i += num_blocks * threads) {
         const unsigned b = i / per_image;
         const unsigned o = i - b * per_image;
         const unsigned c = o / plane;
@@ -65,7 +65,7 @@ constexpr int kPoolStripRows = 8;
 // 3 x 3 windows, stride 1 or 2 in h (any stride in w).  Consecutive lanes take consecutive output columns, so the
 // three loads of an input row are contiguous (stride 1) or interleaved (stride 2) across a wavefront.  Per output
 // this reads 3 * (1 + 2 / 8) (stride 1) or 3 * (2 + 1 / 8) (stride 2) elements instead of 9.
-__device__ __forceinline__ void pool3x3_body(const PoolArgs &a, int block, int num_blocks) {
+__device__ __forceinline__ void pool3x3_body(const PoolArgs &a, int block, int num_blocks, unsigned threads) {
     const PoolProblem &p = a.p;
     const int R = a.strip_rows;
     const unsigned strips = (unsigned)((p.OH + R - 1) / R);
@@ -73,7 +73,7 @@ __device__ __forceinline__ void pool3x3_body(const PoolArgs &a, int block, int n
     const unsigned total = per_plane * (unsigned)(p.C * p.B);
     const bool is_max = p.is_max != 0;
     const float neutral = is_max ? -INFINITY : 0.f;
-    for (unsigned i = block * blockDim.x + threadIdx.x; i < total; i += num_blocks * blockDim.x) {
+    for (unsigned i = block * threads + threadIdx.x; i < total; i += num_blocks * threads) {
         const unsigned pc = i / per_plane;
         const unsigned rest = i - pc * per_plane;
         const unsigned strip = rest / (unsigned)p.OW;
@@ -131,7 +131,7 @@ typedef float pw_floatx4_u __attribute__((ext_vector_type(4), aligned(4)));
 constexpr int kPoolVecColumns = 4;
 
 template <int SW>
-__device__ __forceinline__ void pool3x3_vec_body(const PoolArgs &a, int block, int num_blocks) {
+__device__ __forceinline__ void pool3x3_vec_body(const PoolArgs &a, int block, int num_blocks, unsigned threads) {
     const PoolProblem &p = a.p;
     const int R = a.strip_rows;
     constexpr int V = kPoolVecColumns;
@@ -142,7 +142,7 @@ __device__ __forceinline__ void pool3x3_vec_body(const PoolArgs &a, int block, i
     const unsigned total = per_plane * (unsigned)(p.C * p.B);
     const bool is_max = p.is_max != 0;
     const float neutral = is_max ? -INFINITY : 0.f;
-    for (unsigned i = block * blockDim.x + threadIdx.x; i < total; i += num_blocks * blockDim.x) {
+    for (unsigned i = block * threads + threadIdx.x; i < total; i += num_blocks * threads) {
         const unsigned pc = i / per_plane;
         const unsigned rest = i - pc * per_plane;
         const unsigned strip = rest / quads;
@@ -216,23 +216,23 @@ __device__ __forceinline__ void pool3x3_vec_body(const PoolArgs &a, int block, i
     }
 }
 
-__device__ __forceinline__ void pool_body(const PoolArgs &a, int block, int num_blocks) {
+__device__ __forceinline__ void pool_body(const PoolArgs &a, int block, int num_blocks, unsigned threads) {
     if (a.strip_rows > 0 && a.vec_columns > 1) {
-        if (a.p.sw == 1) pool3x3_vec_body<1>(a, block, num_blocks);
-        else pool3x3_vec_body<2>(a, block, num_blocks);
+        if (a.p.sw == 1) pool3x3_vec_body<1>(a, block, num_blocks, threads);
+        else pool3x3_vec_body<2>(a, block, num_blocks, threads);
     } else if (a.strip_rows > 0) {
-        pool3x3_body(a, block, num_blocks);
+        pool3x3_body(a, block, num_blocks, threads);
     } else {
-        pool_generic_body(a, block, num_blocks);
+        pool_generic_body(a, block, num_blocks, threads);
     }
 }
 
 // window == whole map: one wavefront reduces one (image, channel) plane
-__device__ __forceinline__ void global_pool_body(const PoolArgs &a, int block, int num_blocks) {
+__device__ __forceinline__ void global_pool_body(const PoolArgs &a, int block, int num_blocks, unsigned threads) {
     const PoolProblem &p = a.p;
     const int planes = p.B * p.C;
     const int HW = p.H * p.W;
-    const int waves_per_block = blockDim.x >> 6;
+    const int waves_per_block = threads >> 6;
     const int lane = threadIdx.x & 63;
     for (int plane = block * waves_per_block + (threadIdx.x >> 6); plane < planes; plane += num_blocks * waves_per_block) {
         const int b = plane / p.C, c = plane - b * p.C;
@@ -275,14 +275,14 @@ __device__ __forceinline__ float pw_buffer_load(__amdgpu_buffer_rsrc_t r, unsign
 
 // SUM: the instantiation that adds further inputs in its loader (kept apart so that the common single-input form stays small)
 template <int KH, int KW, bool SUM = false>
-__device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, int num_blocks) {
+__device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, int num_blocks, unsigned threads) {
     const ConvProblem &p = a.p;
     const int kh_n = KH > 0 ? KH : p.KH, kw_n = KW > 0 ? KW : p.KW;
     const unsigned plane = (unsigned)(p.OH * p.OW);
     const unsigned per_image = (unsigned)p.OC * plane;
     const unsigned total = per_image * (unsigned)p.B;
     const int relu_floor = p.pre_relu ? 0 : (int)0x80000000;   // folded ReLU as an integer max
-    for (unsigned i = block * blockDim.x + threadIdx.x; i < total; i += num_blocks * blockDim.x) {
+    for (unsigned i = block * threads + threadIdx.x; i < total; i += num_blocks * threads) {
         const unsigned b = i / per_image;
         const unsigned o = i - b * per_image;
         const unsigned c = o / plane;
@@ -360,17 +360,17 @@ __device__ __forceinline__ void dwconv_body(const DirectConvArgs &a, int block, 
     }
 }
 
-__device__ __forceinline__ void dwconv_dispatch(const DirectConvArgs &a, int block, int num_blocks) {
+__device__ __forceinline__ void dwconv_dispatch(const DirectConvArgs &a, int block, int num_blocks, unsigned threads) {
     const ConvProblem &p = a.p;
     if (a.nmore > 0) {   // the host only builds such launches for 3 x 3 and 5 x 5 windows
-        if (p.KH == 3) dwconv_body<3, 3, true>(a, block, num_blocks);
-        else dwconv_body<5, 5, true>(a, block, num_blocks);
+        if (p.KH == 3) dwconv_body<3, 3, true>(a, block, num_blocks, threads);
+        else dwconv_body<5, 5, true>(a, block, num_blocks, threads);
         return;
     }
-    if (p.KH == 3 && p.KW == 3) dwconv_body<3, 3>(a, block, num_blocks);
-    else if (p.KH == 5 && p.KW == 5) dwconv_body<5, 5>(a, block, num_blocks);
-    else if (p.KH == 7 && p.KW == 7) dwconv_body<7, 7>(a, block, num_blocks);
-    else dwconv_body<0, 0>(a, block, num_blocks);
+    if (p.KH == 3 && p.KW == 3) dwconv_body<3, 3>(a, block, num_blocks, threads);
+    else if (p.KH == 5 && p.KW == 5) dwconv_body<5, 5>(a, block, num_blocks, threads);
+    else if (p.KH == 7 && p.KW == 7) dwconv_body<7, 7>(a, block, num_blocks, threads);
+    else dwconv_body<0, 0>(a, block, num_blocks, threads);
 }
 
 // 3 x 3 convolution of a 3-channel image (the first layer of an image network) for large batches: K is 27, so the layer is
@@ -455,12 +455,12 @@ __device__ __forceinline__ void conv_thin_body(const DirectConvArgs &a, float *s
     }
 }
 
-__device__ __forceinline__ void conv_direct_body(const DirectConvArgs &a, int block, int num_blocks) {
+__device__ __forceinline__ void conv_direct_body(const DirectConvArgs &a, int block, int num_blocks, unsigned threads) {
     const ConvProblem &p = a.p;
     const int icg = p.IC / p.groups, ocg = p.OC / p.groups;
     const long long per_image = (long long)p.OC * p.OH * p.OW;
     const long long total = per_image * p.B;
-    for (long long i = block * (long long)blockDim.x + threadIdx.x; i < total; i += (long long)num_blocks * blockDim.x) {
+    for (long long i = block * (long long)threads + threadIdx.x; i < total; i += (long long)num_blocks * threads) {
         const int b = (int)(i / per_image);
         const int o = (int)(i - b * per_image);
         const int oc = o / (p.OH * p.OW);
@@ -496,12 +496,12 @@ struct NaryKernelArgs {
 };
 
 template <int VEC>
-__device__ __forceinline__ void nary_body(const NaryKernelArgs &k, int block, int num_blocks) {
+__device__ __forceinline__ void nary_body(const NaryKernelArgs &k, int block, int num_blocks, unsigned threads) {
     // indices count VEC-wide packets; chw and every batch stride are multiples of VEC on this path
     const NaryArgs &a = k.in;
     const unsigned chw_v = (unsigned)(k.chw / VEC);
     const unsigned total = (unsigned)k.total;
-    for (unsigned i = block * blockDim.x + threadIdx.x; i < total; i += num_blocks * blockDim.x) {
+    for (unsigned i = block * threads + threadIdx.x; i < total; i += num_blocks * threads) {
         const unsigned b = i / chw_v;
         const long long o = (long long)(i - b * chw_v) * VEC;
         float r[VEC];
@@ -545,9 +545,9 @@ __device__ __forceinline__ void nary_body(const NaryKernelArgs &k, int block, in
     }
 }
 
-__device__ __forceinline__ void nary_dispatch(const NaryKernelArgs &k, int block, int num_blocks) {
-    if (k.vec == 4) nary_body<4>(k, block, num_blocks);
-    else nary_body<1>(k, block, num_blocks);
+__device__ __forceinline__ void nary_dispatch(const NaryKernelArgs &k, int block, int num_blocks, unsigned threads) {
+    if (k.vec == 4) nary_body<4>(k, block, num_blocks, threads);
+    else nary_body<1>(k, block, num_blocks, threads);
 }
 
 }  // namespace ios

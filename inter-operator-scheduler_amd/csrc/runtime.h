@@ -172,6 +172,7 @@ private:
     };
     std::vector<std::vector<FusedLaunch>> fused_stages_;   // per stage; empty for stages whose operations all follow each other
     void *fused_items_ = nullptr;                          // device copy of all work items
+    std::vector<WorkItem> fused_items_host_;
     bool fused_built_ = false;
     hipGraph_t graph_ = nullptr;
     ExecMode graph_mode_ = ExecMode::Graph;                // mode the captured graph was built for
