@@ -46,9 +46,12 @@ constexpr int kFusedThreadClasses[] = {256, 512, 1024};
 
 // Launch `num_items` items as one grid of `total_blocks` blocks of `threads` threads.  `device_items` is the table in device
 // memory; `host_items` (the same items on the host, or null) lets launches that qualify carry their items in the
-// kernel-argument segment instead (fused_kernel.h).
-// Whether a launch of these items (host copies) takes the form with the items in the kernel-argument segment.
-bool fused_items_inline(const WorkItem *host_items, int num_items);
-void launch_fused(int threads, const WorkItem *device_items, const WorkItem *host_items, const FusedHeader &header, int total_blocks, int smem_bytes, hipStream_t stream);
+// kernel-argument segment instead (fused_kernel.h); `num_cus`: compute units of the device.
+// The form of the fused kernel a launch of these items (host copies) takes: the items in a table in device memory, or in the
+// kernel-argument segment, where one kernel holds the matrix-path convolution bodies and another the depth-wise / direct ones.
+enum class FusedForm { Table, InlineMatrix, InlineDirect };
+FusedForm fused_launch_form(const WorkItem *host_items, int num_items, int threads, int total_blocks, int num_cus);
+const char *fused_kernel_name(FusedForm form);   // without the block size
+void launch_fused(int threads, const WorkItem *device_items, const WorkItem *host_items, const FusedHeader &header, int total_blocks, int smem_bytes, int num_cus, hipStream_t stream);
 
 }  // namespace ios

@@ -6,8 +6,9 @@
 
 namespace ios {
 
-// One block of a fused launch: the body of `item`.  DIRECT: the depth-wise and direct convolution bodies are part of the kernel.
-template <int T, bool DIRECT = true>
+// One block of a fused launch: the body of `item`.  MATRIX / DIRECT: the matrix-path convolution bodies / the depth-wise and
+// direct convolution bodies are part of the kernel.
+template <int T, bool MATRIX = true, bool DIRECT = true>
 __device__ __forceinline__ void fused_item(const WorkItem &item, const int bid, float *smem) {
     // An item spans five 64-byte lines of the scalar cache, and the bodies read its fields in two or three dependent steps
     // (kind, then configuration, then arguments): one word of every line is requested together with the first step, so
@@ -24,6 +25,7 @@ __device__ __forceinline__ void fused_item(const WorkItem &item, const int bid, 
     const int num_blocks = item.num_blocks;
     switch (item.kind) {
         case WORK_CONV: {
+            if constexpr (!MATRIX) return;
             if ((int)threadIdx.x >= item.threads) return;   // surplus wavefronts of a narrower body
             const ConvKernelArgs &a = item.conv;   // fields are fetched with scalar loads where they are used
             const int rest = (int)fast_div((unsigned)local, item.div_tiles);
@@ -123,19 +125,19 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fus
 }
 
 // The same kernel with the items of the launch inside the kernel-argument segment instead of a table in device memory: a
-// block's first load (its item) then hits the segment the command processor has just read the leading arguments from, where
-// the table costs a miss all the way to memory at the start of every launch (the caches do not keep it from one launch to the
-// next): 1.0 % of an Inception-v3 pass, 1.2 % of NASNet-A mobile, 2 % of SqueezeNet 1.1 in same-device A/B runs.  Launches of
-// at most kInlineItems items take this form unless they hold a depth-wise or direct convolution: with the items in the
-// kernel-argument segment the compiler loads all eight source descriptors of the summing depth-wise body ahead of the loop and
-// spills, so that body and its launches stay with the table form.
+// block's first load (its item) then hits, where the table costs a miss all the way to memory at the start of every launch
+// (the caches do not keep it from one launch to the next): 1.0 % of an Inception-v3 pass, 1.2 % of NASNet-A mobile, 2 % of
+// SqueezeNet 1.1 in same-device A/B runs.  With the items there the compiler loads all eight source descriptors of the
+// summing depth-wise body ahead of its loop, which does not fit beside the matrix-path bodies in 80 registers, so the form
+// comes as two kernels: MATRIX = true holds the matrix-path convolution bodies and no depth-wise / direct ones; MATRIX =
+// false the other way round with four wavefronts per SIMD (another 1.9 % of NASNet-A mobile).  fused_launch_form() chooses.
 constexpr int kInlineItems = 8;
 struct alignas(64) InlineItems { WorkItem v[kInlineItems]; };
 constexpr unsigned kInlineItemsOffset = 64;   // eight ints, then the items at the next multiple of their alignment
 static_assert(8 * sizeof(int) <= kInlineItemsOffset && alignof(InlineItems) == kInlineItemsOffset, "layout of the kernel-argument segment");
 
-template <int T>
-__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fused_kernel_inline(int num_items, int b1, int b2, int b3, int b4, int b5, int b6,
+template <int T, bool MATRIX>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(MATRIX ? 6 : 4))) void fused_kernel_inline(int num_items, int b1, int b2, int b3, int b4, int b5, int b6,
                                                                                                    int b7, const InlineItems inl) {
     extern __shared__ floatx4 fused_smem[];
     float *smem = reinterpret_cast<float *>(fused_smem);
@@ -149,7 +151,7 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fus
     unsigned long long address = (unsigned long long)__builtin_amdgcn_kernarg_segment_ptr() + kInlineItemsOffset;
     asm volatile("" : "+s"(address));
     address += (unsigned)__builtin_amdgcn_readfirstlane(index) * (unsigned)sizeof(WorkItem);
-    fused_item<T, false>(*(const WorkItem *)(ConstantItem)address, bid, smem);
+    fused_item<T, MATRIX, !MATRIX>(*(const WorkItem *)(ConstantItem)address, bid, smem);
 }
 
 // fused_512.hip

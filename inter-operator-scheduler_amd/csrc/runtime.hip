@@ -814,7 +814,7 @@ void Session::enqueue_fused(bool stage_events) {
         } else {
             for (const FusedLaunch &l : fused_stages_[s]) {
                 if (l.single_op >= 0) launch_op(plan_.ops[l.single_op], main);
-                else launch_fused(l.threads, items + l.first_item, fused_items_host_.data() + l.first_item, l.header, l.total_blocks, l.smem_bytes, main);
+                else launch_fused(l.threads, items + l.first_item, fused_items_host_.data() + l.first_item, l.header, l.total_blocks, l.smem_bytes, ctx_.num_cus(), main);
             }
         }
         if (stage_events) IOS_HIP(hipEventRecord(stage_events_[s], main));
@@ -978,8 +978,8 @@ std::vector<Session::LaunchRecord> Session::launches() {
                     out.push_back(r);
                     continue;
                 }
-                const bool inline_items = fused_items_inline(fused_items_host_.data() + f.first_item, f.num_items);
-                r.kernel = std::string(inline_items ? "fused_kernel_inline<" : "fused_kernel<") + std::to_string(f.threads) + ">";
+                const FusedForm form = fused_launch_form(fused_items_host_.data() + f.first_item, f.num_items, f.threads, f.total_blocks, ctx_.num_cus());
+                r.kernel = std::string(fused_kernel_name(form)) + "<" + std::to_string(f.threads) + ">";
                 r.ops = f.ops;
                 r.blocks = f.total_blocks;
                 r.threads = f.threads;
@@ -1038,7 +1038,7 @@ void Session::profile_launches(int warmup, int repeat, float *ms_out, int capaci
         auto issue = [&]() {
             if (r.fused_level >= 0) {
                 const FusedLaunch &l = fused_stages_[r.stage][r.fused_level];
-                launch_fused(l.threads, items + l.first_item, fused_items_host_.data() + l.first_item, l.header, l.total_blocks, l.smem_bytes, main);
+                launch_fused(l.threads, items + l.first_item, fused_items_host_.data() + l.first_item, l.header, l.total_blocks, l.smem_bytes, ctx_.num_cus(), main);
             } else {
                 launch_op(plan_.ops[r.ops[0]], main);
             }

@@ -718,6 +718,43 @@ def test_zoo_network_matches_oracle(name, make, batch, absorbed):
                 assert_close(session.output(), want, f'{name} {executor} {label}')
 
 
+def test_every_form_of_the_fused_stage_kernel_runs_and_matches_the_oracle():
+    """Launches of a fused stage carry their work items in the kernel-argument segment when they hold at most eight of them
+    (one kernel for levels with matrix-path convolutions, one for levels of depth-wise convolutions, pools and sums) and read
+    them from a table in device memory otherwise.  NASNet-A mobile under the greedy schedule uses all three forms; a stage of
+    ten parallel 1x1 convolutions takes the table form because of its size."""
+    graph = ios.models.nasnet_mobile(init_seed=0, init_scheme='he_normal_bias')
+    graph.greedy_schedule(8)
+    x = np.random.default_rng(5).standard_normal((1, *graph.enter_node.output_shape)).astype(np.float32)
+    want = ios_oracle.run(graph, x)
+    rt.set_option('executor', 'fused')
+    with rt.Session(graph, 1) as session:
+        session.load_weights()
+        session.set_input(x)
+        kernels = {launch['kernel'].split('<')[0] for launch in session.launches()}
+        assert {'fused_kernel', 'fused_kernel_inline', 'fused_kernel_inline_direct'} <= kernels, kernels
+        session.run()
+        assert_close(session.output(), want, 'nasnet_mobile greedy')
+
+    ios.reset_name()
+    v = ios.placeholder((16, 12, 12))
+    block = ios.Block(v.node)
+    outs = [ios.conv2d(block, [[v]], 8 + i, (1, 1), (1, 1), (0, 0), 1, 'relu') for i in range(10)]
+    out = ios.identity(block, [[o] for o in outs], is_exit=True)
+    wide = Graph('ten_branches', v.node, [block])
+    wide.init_weights(3, 'he_normal_bias')
+    block.stages = [[[o.node.name] for o in outs], [[out.node.name]]]
+    x = np.random.default_rng(6).standard_normal((2, 16, 12, 12)).astype(np.float32)
+    want = ios_oracle.run(wide, x)
+    with rt.Session(wide, 2) as session:
+        session.load_weights()
+        session.set_input(x)
+        first = session.launches()[0]
+        assert first['kernel'].startswith('fused_kernel<') and len(first['ops']) == 10, first
+        session.run()
+        assert_close(session.output(), want, 'ten parallel convolutions')
+
+
 def test_activation_absorbs_the_combination_in_front_of_it():
     """add -> relu, mul -> tanh, three-way sum -> sigmoid become one launch each; a combination that somebody else reads, or
     that the activation reads in part, stays a launch of its own.  Results as in the oracle either way."""
