@@ -36,11 +36,11 @@ void launch_fused(int threads, const WorkItem *device_items, const WorkItem *hos
         InlineItems inl{};
         memcpy(inl.v, host_items, (size_t)header.num_items * sizeof(WorkItem));
         if (form == FusedForm::InlineDirect)
-            hipLaunchKernelGGL((fused_kernel_inline<256, false>), grid, dim3(256), smem_bytes, stream, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7], inl);
+            hipLaunchKernelGGL(fused_kernel_inline_direct<256>, grid, dim3(256), smem_bytes, stream, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7], inl);
         else if (threads == 256)
-            hipLaunchKernelGGL((fused_kernel_inline<256, true>), grid, dim3(256), smem_bytes, stream, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7], inl);
+            hipLaunchKernelGGL(fused_kernel_inline<256>, grid, dim3(256), smem_bytes, stream, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7], inl);
         else if (threads == 1024)
-            hipLaunchKernelGGL((fused_kernel_inline<1024, true>), grid, dim3(1024), smem_bytes, stream, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7], inl);
+            hipLaunchKernelGGL(fused_kernel_inline<1024>, grid, dim3(1024), smem_bytes, stream, header.num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7], inl);
         else
             throw std::runtime_error("fused launch: unsupported block size");
         return;

@@ -10,7 +10,7 @@ void launch_fused_512(const WorkItem *device_items, const WorkItem *host_items, 
     if (host_items) {   // (launch_fused has checked that the items fit the inline form)
         InlineItems inl{};
         memcpy(inl.v, host_items, (size_t)num_items * sizeof(WorkItem));
-        hipLaunchKernelGGL((fused_kernel_inline<512, true>), dim3((unsigned)total_blocks), dim3(512), smem_bytes, stream, num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7], inl);
+        hipLaunchKernelGGL(fused_kernel_inline<512>, dim3((unsigned)total_blocks), dim3(512), smem_bytes, stream, num_items, b[1], b[2], b[3], b[4], b[5], b[6], b[7], inl);
         return;
     }
     hipLaunchKernelGGL(fused_kernel<512>, dim3((unsigned)total_blocks), dim3(512), smem_bytes, stream, device_items, num_items, b[1], b[2], b[3], b[4],

@@ -129,16 +129,16 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fus
 // (the caches do not keep it from one launch to the next): 1.0 % of an Inception-v3 pass, 1.2 % of NASNet-A mobile, 2 % of
 // SqueezeNet 1.1 in same-device A/B runs.  With the items there the compiler loads all eight source descriptors of the
 // summing depth-wise body ahead of its loop, which does not fit beside the matrix-path bodies in 80 registers, so the form
-// comes as two kernels: MATRIX = true holds the matrix-path convolution bodies and no depth-wise / direct ones; MATRIX =
-// false the other way round with four wavefronts per SIMD (another 1.9 % of NASNet-A mobile).  fused_launch_form() chooses.
+// comes as two kernels: fused_kernel_inline holds the matrix-path convolution bodies and no depth-wise / direct ones,
+// fused_kernel_inline_direct the other way round with four wavefronts per SIMD (another 1.9 % of NASNet-A mobile).
+// fused_launch_form() chooses.
 constexpr int kInlineItems = 8;
 struct alignas(64) InlineItems { WorkItem v[kInlineItems]; };
 constexpr unsigned kInlineItemsOffset = 64;   // eight ints, then the items at the next multiple of their alignment
 static_assert(8 * sizeof(int) <= kInlineItemsOffset && alignof(InlineItems) == kInlineItemsOffset, "layout of the kernel-argument segment");
 
 template <int T, bool MATRIX>
-__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(MATRIX ? 6 : 4))) void fused_kernel_inline(int num_items, int b1, int b2, int b3, int b4, int b5, int b6,
-                                                                                                   int b7, const InlineItems inl) {
+__device__ __forceinline__ void fused_inline_block(int b1, int b2, int b3, int b4, int b5, int b6, int b7) {
     extern __shared__ floatx4 fused_smem[];
     float *smem = reinterpret_cast<float *>(fused_smem);
     const int bid = blockIdx.x;
@@ -152,6 +152,18 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(MATRIX ? 6 : 
     asm volatile("" : "+s"(address));
     address += (unsigned)__builtin_amdgcn_readfirstlane(index) * (unsigned)sizeof(WorkItem);
     fused_item<T, MATRIX, !MATRIX>(*(const WorkItem *)(ConstantItem)address, bid, smem);
+}
+
+template <int T>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(6))) void fused_kernel_inline(int num_items, int b1, int b2, int b3, int b4, int b5, int b6,
+                                                                                                   int b7, const InlineItems inl) {
+    fused_inline_block<T, true>(b1, b2, b3, b4, b5, b6, b7);
+}
+
+template <int T>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(4))) void fused_kernel_inline_direct(int num_items, int b1, int b2, int b3, int b4, int b5,
+                                                                                                          int b6, int b7, const InlineItems inl) {
+    fused_inline_block<T, false>(b1, b2, b3, b4, b5, b6, b7);
 }
 
 // fused_512.hip
