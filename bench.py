@@ -13,7 +13,7 @@ figures for every kernel of the pass.  `cpu_baseline`: the CPU oracle on the sam
 the host cores for about ten seconds.  Every configuration network and every batch of the sweep is also compared with
 the oracle under the strict tolerance |d| <= 1e-4 + 1e-3 |want|.
 
-Probe modes for the profiler (`--probe copy | search | pass`) run a fixed small workload and print what the counters
+Probe modes for the profiler (`--probe copy | search | pass | floor`) run a fixed small workload and print what the counters
 should be compared with; they are used by the commands recorded under profiles/.
 """
 import argparse
@@ -222,6 +222,44 @@ def probe(args, np, ios, rt):
                           'write_bytes_per_launch': nbytes, 'ms_per_launch': ms,
                           'gbs': 2 * nbytes / (ms * 1e-3) / 1e9}))
         return
+    if args.probe == 'floor':
+        # what a launch costs when it does next to nothing: a chain of dependent tanh activations on one 8 x 8 x 8 tensor and a
+        # chain of dependent 1x1 convolutions (8 -> 8 channels on 8 x 8 pixels), one launch each, under every executor
+        results = {}
+        for kind in ('activation', 'conv1x1'):
+            ios.reset_name()
+            v = ios.placeholder((8, 8, 8))
+            block = ios.Block(v.node)
+            t = v
+            for i in range(args.floor_length):
+                last = i == args.floor_length - 1
+                if kind == 'activation':
+                    t = ios.activation(block, [[t]], 'tanh', False, is_exit=last)
+                else:
+                    t = ios.conv2d(block, [[t]], 8, (1, 1), (1, 1), (0, 0), 1, 'tanh', is_exit=last)
+            graph = ios.Graph('floor_' + kind, v.node, [block])
+            graph.init_weights(0, 'he_normal_bias')
+            graph.sequential_schedule()
+            x = np.random.default_rng(0).standard_normal((1, 8, 8, 8)).astype(np.float32)
+            for executor in args.floor_executors.split(','):
+                rt.set_option('executor', executor)
+                with rt.Session(graph, 1) as session:
+                    session.load_weights()
+                    session.set_input(x)
+                    for _ in range(10):
+                        session.run()
+                    launches = len(session.launches())
+                    session.synchronize()
+                    t0 = time.perf_counter()
+                    for _ in range(args.passes):
+                        session.enqueue()
+                    session.synchronize()
+                    wall = (time.perf_counter() - t0) / args.passes * 1e3
+                    events = float(np.min(session.measure(warmup=2, number=20, repeat=5)))
+                results[f'{kind}/{executor}'] = {'launches_per_pass': launches, 'us_per_launch_queued_back_to_back': wall * 1e3 / launches,
+                                                 'us_per_launch_event_timed': events * 1e3 / launches}
+        print(json.dumps({'probe': 'floor', 'chain_length': args.floor_length, 'passes': args.passes, 'results': results}))
+        return
     graph = make_graph(ios, args.model)
     batch = args.batch
     if args.probe == 'search':
@@ -307,10 +345,13 @@ def main():
     parser.add_argument('--search-variants', action='store_true',
                         help="measured schedule search also for the reference table's large model variants (about two more minutes)")
     parser.add_argument('--option', action='append', default=[], metavar='KEY=VALUE', help='extra runtime option (repeatable)')
-    parser.add_argument('--probe', choices=['copy', 'search', 'pass'], help='run a profiler probe instead of the benchmark')
+    parser.add_argument('--probe', choices=['copy', 'search', 'pass', 'floor'], help='run a profiler probe instead of the benchmark')
     parser.add_argument('--model', default='inception_v3', choices=sorted(CONFIG_MODELS), help='network of the search / pass probes')
     parser.add_argument('--schedule-file', help='probe search: where to write the schedule; probe pass: schedule to run (default: sequential)')
     parser.add_argument('--passes', type=int, default=3, help='forward passes of the pass probe')
+    parser.add_argument('--floor-length', type=int, default=50, help='floor probe: dependent operators in the chain')
+    parser.add_argument('--floor-executors', default='streams,graph,fused,fused_graph',
+                        help='floor probe: executors to time (graph replays are not traced by rocprofv3: give it streams,fused)')
     args = parser.parse_args()
     if args.gpus != 1:
         print('bench.py: this runtime is a single-GPU path; run with --gpus 1', file=sys.stderr)
