@@ -2,9 +2,13 @@
 Benchmark of the north-star path: Inception-v3 at batch 1 under the dp_parallel schedule found by the
 dynamic-programming search with on-device stage measurements, on one MI355X.
 
-A step is one forward pass over one synthetic batch (weights and input already resident in HBM); the K timed steps are
-queued back to back between two synchronisations, so `ms_per_step` is the time the device needs per pass (the figure with the
-host waiting for every pass is reported beside it as `wall_host_waits_for_every_pass`).  Prints one JSON line.
+A step is one forward pass over one synthetic batch (weights and input already resident in HBM).  `ms_per_step` is the
+latency of a pass under the reference's own timing protocol (`measure_latency`, src/ios/ios_runtime.cu:1419-1441): after W
+warm-up passes, each of the K timed passes starts on an idle device (device synchronised first) and is bracketed by its own
+pair of events; `ms_per_step` is their mean and `value` the images per second that latency allows.  The same K passes
+queued back to back between two synchronisations (a throughput figure: the host's launch work overlaps the previous pass)
+and with the host waiting for every pass are reported beside it as `throughput_ms_per_pass` and
+`wall_host_waits_for_every_pass`.  Prints one JSON line.
 
 `roofline` describes the kernel that takes the largest share of the timed pass: every launch of that pass (under the
 executor that is timed) is issued back to back on the launch stream between two HIP events, launches are grouped by
@@ -60,28 +64,31 @@ def network_roofline_ms(ops, parallel):
 
 def timed_latency(rt, np, graph, batch, x, steps, warmup):
     """
-    Wall-clock ms per forward pass over `steps` passes queued back to back between two synchronisations (the device runs
-    them one after the other; what the host spends on a launch overlaps the previous pass), the same with the host
-    waiting for every pass, event-timed latencies (reference protocol) and the output.
+    Latency of a forward pass, three ways over `steps` passes after `warmup` passes, and the output:
+    `latency` - the reference protocol (device synchronised before every pass, an event pair around each, mean);
+    `throughput_ms_per_pass` - wall clock over the passes queued back to back between two synchronisations (the device runs
+    them one after the other, the host's launch work overlaps the previous pass);
+    `wall_host_waits_for_every_pass` - wall clock with the host waiting for every pass.
+    `events_*` repeat the reference protocol with the reference's default counts (warmup 2, number 6, repeat 6).
     """
     with rt.Session(graph, batch) as session:
         session.load_weights()
         session.set_input(x)
-        for _ in range(warmup):
-            session.run()
+        latency = float(session.measure(warmup=warmup, number=steps, repeat=1)[0])
         session.synchronize()
         t = time.perf_counter()
         for _ in range(steps):
             session.enqueue()
         session.synchronize()
-        wall = (time.perf_counter() - t) / steps * 1e3
+        queued = (time.perf_counter() - t) / steps * 1e3
         t = time.perf_counter()
         for _ in range(steps):
             session.run()
         wall_waiting = (time.perf_counter() - t) / steps * 1e3
         events = session.measure(warmup=2, number=6, repeat=6)
-        return {'wall': wall, 'wall_host_waits_for_every_pass': wall_waiting, 'events_mean': float(np.mean(events)),
-                'events_min': float(np.min(events)), 'events_std': float(np.std(events))}, session.output()
+        return {'latency': latency, 'throughput_ms_per_pass': queued, 'wall_host_waits_for_every_pass': wall_waiting,
+                'events_mean': float(np.mean(events)), 'events_min': float(np.min(events)),
+                'events_std': float(np.std(events))}, session.output()
 
 
 def oracle_check(np, got, want):
@@ -131,17 +138,21 @@ def launch_profile(rt, graph, batch, x, stages=False):
 
 
 def committed_traffic(kernel):
-    """HBM bytes per launch of `kernel` from the committed counter summary (None when the summary has no such row)."""
-    try:
-        with open(TRAFFIC_PROFILE) as f:
-            for line in f:
-                match = re.match(r'\|\s*`([^`]+)`\s*\|(.*)\|\s*$', line)
-                if match and match.group(1) == kernel:
-                    cells = [c.strip() for c in match.group(2).split('|')]
-                    return float(cells[-1]) * 1e6    # last column: traffic per launch, MB
-    except (OSError, ValueError):
-        pass
-    return None
+    """
+    HBM bytes per launch of `kernel` and the provenance line of the committed counter summary they come from (an offline
+    figure: FETCH_SIZE and WRITE_SIZE need a profiler run of their own).  A kernel the summary does not list is an error:
+    the summary then describes another build and has to be collected again.
+    """
+    provenance = None
+    with open(TRAFFIC_PROFILE) as f:
+        for line in f:
+            if line.startswith('Collected'):
+                provenance = line.strip()
+            match = re.match(r'\|\s*`([^`]+)`\s*\|(.*)\|\s*$', line)
+            if match and match.group(1) == kernel:
+                cells = [c.strip() for c in match.group(2).split('|')]
+                return float(cells[-1]) * 1e6, provenance    # last column: traffic per launch, MB
+    raise RuntimeError(f'{os.path.relpath(TRAFFIC_PROFILE, ROOT)} has no row for kernel {kernel}: collect the counters again')
 
 
 def roofline_block(kernels, ms_per_step, headline=False):
@@ -152,15 +163,16 @@ def roofline_block(kernels, ms_per_step, headline=False):
     else:
         bound, achieved, peak, unit = 'hbm', k['gbs'], PEAK_HBM_GBS, 'GB/s'
     block = {'bound': bound, 'kernel': name, 'achieved': achieved, 'peak': peak, 'unit': unit, 'frac': achieved / peak,
-             'traffic': committed_traffic(name) if headline else None,
+             'traffic': None,
              'launches_per_pass': k['launches'], 'avg_launch_us': k['avg_launch_us'],
              'algorithmic_flops_per_launch': k['matrix_flops'] / k['launches'],
              'algorithmic_bytes_per_launch': k['bytes'] / k['launches'],
              'kernel_ms_per_pass': k['ms'], 'share_of_launch_time': k['ms'] / sum(v['ms'] for v in kernels.values()),
              'all_launches_ms_per_pass': sum(v['ms'] for v in kernels.values())}
     if headline:
-        block['traffic_source'] = ('bytes per launch, FETCH_SIZE + WRITE_SIZE counter runs of the same pass, read from '
-                                   + os.path.relpath(TRAFFIC_PROFILE, ROOT))
+        block['traffic'], provenance = committed_traffic(name)
+        block['traffic_offline_counter_run'] = ('bytes per launch from FETCH_SIZE + WRITE_SIZE counter runs of a pass of this network, '
+                                                'not of this run: ' + os.path.relpath(TRAFFIC_PROFILE, ROOT) + (' (' + provenance + ')' if provenance else ''))
     assert block['kernel_ms_per_pass'] <= ms_per_step, (block['kernel_ms_per_pass'], ms_per_step)
     return block
 
@@ -343,7 +355,9 @@ def main():
     parser.add_argument('--greedy-big', action='store_true',
                         help='use the greedy schedule for RandWire and NASNet instead of the measured search')
     parser.add_argument('--search-variants', action='store_true',
-                        help="measured schedule search also for the reference table's large model variants (about two more minutes)")
+                        help="also time the model variants of the reference's own result table (its large RandWire / NASNet, SqueezeNet 1.0 "
+                             "with bypass, the chains and residual networks of its zoo) under sequential, greedy and searched schedules "
+                             "(about three more minutes; not part of the metric)")
     parser.add_argument('--option', action='append', default=[], metavar='KEY=VALUE', help='extra runtime option (repeatable)')
     parser.add_argument('--probe', choices=['copy', 'search', 'pass', 'floor'], help='run a profiler probe instead of the benchmark')
     parser.add_argument('--model', default='inception_v3', choices=sorted(CONFIG_MODELS), help='network of the search / pass probes')
@@ -408,12 +422,13 @@ def main():
 
     result = {
         'metric': 'batch-1 latency (ms) + images/s, Inception-v3 IOS dp_parallel schedule',
-        'value': batch / (opt['wall'] * 1e-3),
+        'value': batch / (opt['latency'] * 1e-3),
         'unit': 'images/s',
         'n_gpus': 1,
         'steps': args.steps,
         'warmup': args.warmup,
-        'ms_per_step': opt['wall'],
+        'ms_per_step': opt['latency'],
+        'throughput_ms_per_pass': opt['throughput_ms_per_pass'],
         'higher_is_better': True,
         'scaling': 'weak',
         'vs_baseline': None,
@@ -422,18 +437,18 @@ def main():
         'config': {'workload': f'inception_v3 3x299x299 batch {batch}, dp_parallel schedule (r={args.max_group_size}, s={args.max_num_groups}), {args.executor} executor',
                    'global_batch': batch},
         'latency_ms': {'dp_parallel': opt, 'sequential': seq},
-        'speedup_vs_own_sequential': seq['wall'] / opt['wall'],
+        'speedup_vs_own_sequential': seq['latency'] / opt['latency'],
         'max_abs_diff_between_schedules': float(np.abs(seq_out - opt_out).max()),
         'search_seconds': search_s,
         'num_stages': sum(len(b.stages) for b in optimized.blocks),
         'launches_per_pass': len(launches),
         'network_roofline_ms': {'sequential': roof_seq, 'critical_path': roof_par,
-                                'fraction_of_critical_path_roofline': roof_par / opt['wall'],
-                                'fraction_of_sequential_roofline': roof_seq / opt['wall']},
-        'whole_pass': {'matrix_tflops': conv_flops / (opt['wall'] * 1e-3) / 1e12,
-                       'frac_of_fp32_matrix_peak': conv_flops / (opt['wall'] * 1e-3) / 1e12 / PEAK_FP32_MATRIX_TFLOPS,
-                       'algorithmic_gbs': total_bytes / (opt['wall'] * 1e-3) / 1e9},
-        'roofline': roofline_block(kernels, opt['wall'], headline=True),
+                                'fraction_of_critical_path_roofline': roof_par / opt['latency'],
+                                'fraction_of_sequential_roofline': roof_seq / opt['latency']},
+        'whole_pass': {'matrix_tflops': conv_flops / (opt['latency'] * 1e-3) / 1e12,
+                       'frac_of_fp32_matrix_peak': conv_flops / (opt['latency'] * 1e-3) / 1e12 / PEAK_FP32_MATRIX_TFLOPS,
+                       'algorithmic_gbs': total_bytes / (opt['latency'] * 1e-3) / 1e9},
+        'roofline': roofline_block(kernels, opt['latency'], headline=True),
         'kernels': kernels,
         'kernels_sequential_pass': seq_kernels,
         'stage_overlap': stage_overlap(ops, launches, stage_ms),
@@ -456,7 +471,7 @@ def main():
         graph.sequential_schedule()
         rt.set_option('executor', args.executor)
         other_ms, _ = timed_latency(rt, np, other_knobs, batch, x, args.steps, args.warmup)
-        result[f'dp_parallel_r{other_r}_s{other_s}'] = {'latency_ms': other_ms, 'images_per_s': batch / (other_ms['wall'] * 1e-3),
+        result[f'dp_parallel_r{other_r}_s{other_s}'] = {'latency_ms': other_ms, 'images_per_s': batch / (other_ms['latency'] * 1e-3),
                                                        'search_seconds': other_search_s,
                                                        'num_stages': sum(len(b.stages) for b in other_knobs.blocks)}
 
@@ -470,7 +485,7 @@ def main():
         graph.sequential_schedule()
         rt.set_option('executor', args.executor)
         both, both_out = timed_latency(rt, np, merged, batch, x, args.steps, args.warmup)
-        result['dp_parallel_merge'] = {'latency_ms': both, 'images_per_s': batch / (both['wall'] * 1e-3), 'search_seconds': merge_search_s,
+        result['dp_parallel_merge'] = {'latency_ms': both, 'images_per_s': batch / (both['latency'] * 1e-3), 'search_seconds': merge_search_s,
                                        'num_stages': sum(len(b.stages) for b in merged.blocks),
                                        'max_abs_diff_to_sequential': float(np.abs(seq_out - both_out).max())}
 
@@ -491,13 +506,13 @@ def main():
             graph.sequential_schedule()
             rt.set_option('executor', args.executor)
             s_own, out_own = timed_latency(rt, np, optimized_b, b, xb, steps, 3)
-            _, _, kernels_b = launch_profile(rt, graph if s_seq['wall'] < s_own['wall'] else optimized_b, b, xb)
+            _, _, kernels_b = launch_profile(rt, graph if s_seq['latency'] < s_own['latency'] else optimized_b, b, xb)
             ops_b = rt.plan_describe(graph, b)
-            best = min(s_seq['wall'], s_opt['wall'], s_own['wall'])
+            best = min(s_seq['latency'], s_opt['latency'], s_own['latency'])
             matrix_ms = sum(k['ms'] for k in kernels_b.values() if k['matrix_flops'] > 0)
             matrix_flops = sum(k['matrix_flops'] for k in kernels_b.values())
-            sweep[str(b)] = {'sequential_ms': s_seq['wall'], 'dp_parallel_batch1_schedule_ms': s_opt['wall'],
-                             'dp_parallel_ms': s_own['wall'], 'search_seconds': search_b,
+            sweep[str(b)] = {'sequential_ms': s_seq['latency'], 'dp_parallel_batch1_schedule_ms': s_opt['latency'],
+                             'dp_parallel_ms': s_own['latency'], 'search_seconds': search_b,
                              'max_abs_diff_between_schedules': float(np.abs(out_seq - out_own).max()),
                              'images_per_s': b / (best * 1e-3),
                              'network_roofline_ms': network_roofline_ms(ops_b, parallel=False),
@@ -519,7 +534,7 @@ def main():
                 for b in (1, 64):
                     xb = np.random.default_rng(1).standard_normal((b, 3, 299, 299)).astype(np.float32)
                     r_seq, out_b = timed_latency(rt, np, graph, b, xb, max(10, args.steps // (b * 2)), 3)
-                    reduced[str(b)] = {'sequential_ms': r_seq['wall'], 'images_per_s': b / (r_seq['wall'] * 1e-3)}
+                    reduced[str(b)] = {'sequential_ms': r_seq['latency'], 'images_per_s': b / (r_seq['latency'] * 1e-3)}
                     if b == 1:
                         reduced[str(b)]['max_abs_diff_to_fp32'] = float(np.abs(out_b - seq_out).max())
                         reduced[str(b)]['fp32_output_scale'] = float(np.abs(seq_out).max())
@@ -554,18 +569,18 @@ def main():
                 single = ios.optimize(g, batch_size=1, cost_model=ios.IOSCostModel(share_identical_stages=True), opt_type='dp_parallel',
                                       compute_weight=True, warmup=2, number=6, repeat=3, max_group_size=1, max_num_groups=args.max_num_groups)
                 rt.set_option('executor', args.executor)
-                other_ms = timed_latency(rt, np, single, 1, xc, 100, 10)[0]['wall']
+                other_ms = timed_latency(rt, np, single, 1, xc, 100, 10)[0]['latency']
             g.sequential_schedule()
             c_seq, _ = timed_latency(rt, np, g, 1, xc, 100, 10)
             c_par, c_out = timed_latency(rt, np, scheduled, 1, xc, 100, 10)
             ops_c = rt.plan_describe(g, 1)
             _, launches_c, kernels_c = launch_profile(rt, scheduled, 1, xc)
-            configs[name] = {'sequential_ms': c_seq['wall'], f'{label}_ms': c_par['wall'], 'search_seconds': search_c,
+            configs[name] = {'sequential_ms': c_seq['latency'], f'{label}_ms': c_par['latency'], 'search_seconds': search_c,
                              'search_pruning': None if label == 'greedy' else f'r={group_size}, s={args.max_num_groups}',
                              'initialisation': CONFIG_MODELS[name][1], 'device_operations': len(ops_c), 'launches_per_pass': len(launches_c),
                              'network_roofline_ms': network_roofline_ms(ops_c, parallel=False),
-                             'fraction_of_network_roofline': network_roofline_ms(ops_c, parallel=False) / c_par['wall'],
-                             'roofline': roofline_block(kernels_c, c_par['wall']),
+                             'fraction_of_network_roofline': network_roofline_ms(ops_c, parallel=False) / c_par['latency'],
+                             'roofline': roofline_block(kernels_c, c_par['latency']),
                              'memory_bound_ops_gbs': memory_bound_ops(rt, g, 1, xc)}
             if other_ms is not None:
                 configs[name]['dp_parallel_r1_ms'] = other_ms
@@ -573,7 +588,7 @@ def main():
             if not args.no_cpu:
                 configs[name]['oracle'] = oracle_check(np, c_out, ios_oracle.run(g, xc))
         result['other_configs_batch1'] = configs
-        if not args.no_extras:
+        if args.search_variants:
             # the model variants the reference's own result table uses (its large RandWire / NASNet and SqueezeNet 1.0 with
             # bypass) and the chains / residual networks of its zoo, sequential and greedy schedules: points of comparison
             # with that table, not part of the metric
@@ -588,16 +603,15 @@ def main():
                 xc = np.random.default_rng(1).standard_normal((1, *g.enter_node.output_shape)).astype(np.float32)
                 v_seq, _ = timed_latency(rt, np, g, 1, xc, 50, 5)
                 v_par, _ = timed_latency(rt, np, scheduled, 1, xc, 50, 5)
-                variants[name] = {'sequential_ms': v_seq['wall'], 'greedy_ms': v_par['wall']}
-                if args.search_variants:
-                    rt.set_option('executor', args.search_executor)
-                    t0 = time.time()
-                    searched = ios.optimize(make(init_seed=0, init_scheme='he_normal'), batch_size=1, opt_type='dp_parallel', compute_weight=True,
-                                            warmup=2, number=6, repeat=3, max_group_size=args.big_max_group_size, max_num_groups=args.max_num_groups)
-                    variants[name]['search_seconds'] = time.time() - t0
-                    rt.set_option('executor', args.executor)
-                    v_dp, _ = timed_latency(rt, np, searched, 1, xc, 50, 5)
-                    variants[name]['dp_parallel_ms'] = v_dp['wall']
+                variants[name] = {'sequential_ms': v_seq['latency'], 'greedy_ms': v_par['latency']}
+                rt.set_option('executor', args.search_executor)
+                t0 = time.time()
+                searched = ios.optimize(make(init_seed=0, init_scheme='he_normal'), batch_size=1, opt_type='dp_parallel', compute_weight=True,
+                                        warmup=2, number=6, repeat=3, max_group_size=args.big_max_group_size, max_num_groups=args.max_num_groups)
+                variants[name]['search_seconds'] = time.time() - t0
+                rt.set_option('executor', args.executor)
+                v_dp, _ = timed_latency(rt, np, searched, 1, xc, 50, 5)
+                variants[name]['dp_parallel_ms'] = v_dp['latency']
             result['reference_table_variants_batch1'] = variants
 
     if not args.no_cpu:

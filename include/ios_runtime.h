@@ -59,7 +59,9 @@ int graph_inference(const char *graph_json, int batch_size, float *input, int nu
 /*
  * graph_inference for callers that cannot allocate device memory (harnesses that forbid hipMalloc, tight serving
  * loops).  No counterpart in the reference.  Same arguments and results as graph_inference, but the call makes no
- * hipMalloc / hipFree and creates no events or streams: every device buffer of the pass (operator outputs, filters,
+ * hipMalloc / hipFree and creates no events or streams (the library's per-device context - its streams and the address
+ * of the static array - is created by the first call into the library that touches the device, whichever it is, and is
+ * not part of this promise: call ios_device_info once beforehand where that matters): every device buffer of the pass (operator outputs, filters,
  * packed filters, split-K partial tiles and their ticket counters) is laid out in a static device array of
  * IOS_NO_ALLOC_SCRATCH_BYTES that device 0 holds from library load to process end.  A graph whose plan needs more
  * at the given batch size is refused with an error that names both figures.  Kernel configurations come from the
@@ -71,6 +73,9 @@ int graph_inference(const char *graph_json, int batch_size, float *input, int nu
 #define IOS_NO_ALLOC_SCRATCH_BYTES (256u << 20)
 int graph_inference_no_alloc(const char *graph_json, int batch_size, float *input, int num_convs, char **conv_names,
                              float **filter_data, float **bias_data, float *output);
+
+/* Free device memory in bytes as hipMemGetInfo reports it (creates the device context if there is none yet), or -1. */
+long long ios_device_free_bytes(void);
 
 /* Message of the most recent failure (valid until the next failing call). */
 const char *ios_last_error(void);
@@ -120,8 +125,9 @@ int ios_session_set_conv_weights(ios_session *session, int num_convs, char **con
 int ios_session_set_input(ios_session *session, const float *input);
 int ios_session_run(ios_session *session);                                  /* one forward pass, waits for it */
 /* One forward pass queued behind the earlier ones without waiting, and the wait for everything queued: K passes
- * between two synchronisations run back to back on the device, as the reference's timers see them
- * (src/ios/ios_runtime.cu:1423-1440 takes its events around the device work of a pass). */
+ * between two synchronisations run back to back on the device while the host's launch work overlaps the pass before.
+ * That is a throughput figure.  The reference's timers do something else (src/ios/ios_runtime.cu:1419-1441: the device
+ * is synchronised before every pass and every pass has its own pair of events): ios_session_measure follows them. */
 int ios_session_enqueue(ios_session *session);
 int ios_session_synchronize(ios_session *session);
 int ios_session_get_output(ios_session *session, float *output);

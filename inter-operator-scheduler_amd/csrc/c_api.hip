@@ -140,6 +140,17 @@ int ios_device_info(char *buf, int cap) {
     });
 }
 
+long long ios_device_free_bytes(void) {
+    long long bytes = -1;
+    guarded([&]() {
+        ios::DeviceContext::get();
+        size_t free_bytes = 0, total = 0;
+        if (hipMemGetInfo(&free_bytes, &total) != hipSuccess) throw std::runtime_error("hipMemGetInfo failed");
+        bytes = (long long)free_bytes;
+    });
+    return bytes;
+}
+
 int ios_conv_variant_names(char *buf, int cap) {
     std::string text = "[";
     for (int i = 0; i < ios::conv_num_variants(); i++) text += std::string(i ? "," : "") + '"' + ios::conv_variant(i).name + '"';
@@ -148,13 +159,22 @@ int ios_conv_variant_names(char *buf, int cap) {
     return (int)text.size();
 }
 
+// Kernel configurations of plans made without a device: the closed-form model for a 256-CU part.
+static ios::LaunchChooser host_chooser() {
+    return [](const ios::ConvProblem &p, int share) {
+        ios::ConvLaunch launch = ios::conv_pick_launch(p, 256 / (share > 0 ? share : 1), share > 1);
+        if (ios::planner_host_split_k() > 0) launch.split_k = ios::planner_host_split_k();
+        return launch;
+    };
+}
+
 int ios_plan_describe(const char *graph_json, int batch_size, char *buf, int cap) {
     int needed = -1;
     guarded([&]() {
         const ios::Json doc = ios::Json::parse(graph_json);
         // host-only: the closed-form configuration model for a 256-CU device, no device is touched
         ios::Plan plan = ios::build_plan(ios::PlanMode::Graph, doc, nullptr, batch_size,
-                                         [](const ios::ConvProblem &p, int share) { return ios::conv_pick_launch(p, 256 / (share > 0 ? share : 1), share > 1); });
+                                         host_chooser());
         const std::string text = ios::describe_plan(plan);
         needed = (int)text.size();
         if (buf != nullptr && cap > needed) memcpy(buf, text.c_str(), text.size() + 1);
@@ -167,7 +187,7 @@ long long ios_plan_arena_bytes(const char *graph_json, int batch_size) {
     guarded([&]() {
         const ios::Json doc = ios::Json::parse(graph_json);
         ios::Plan plan = ios::build_plan(ios::PlanMode::Graph, doc, nullptr, batch_size,
-                                         [](const ios::ConvProblem &p, int share) { return ios::conv_pick_launch(p, 256 / (share > 0 ? share : 1), share > 1); });
+                                         host_chooser());
         bytes = (long long)(plan.arena_floats * sizeof(float));
     });
     return bytes;

@@ -539,7 +539,7 @@ struct ConvWsplit {
     static constexpr bool KQUAD = QUAD;                    // packed filters are [k / 4][m][4] instead of [k][m]
     // accumulators + staged operands per lane decide whether the body fits the register budget of a fused launch
     // (the channel-padding-4 forms serve first layers, which are stages of their own: kept out of the fused launches)
-    static constexpr bool FUSABLE = CP == 0 && E + D * U * (TM + TN) <= (QUAD ? 56 : 48);   // per-step addressing of the plain layout needs more registers
+    static constexpr bool FUSABLE = CP == 0 && E + D * U * (TM + TN) <= (QUAD ? (MT == 32 ? 48 : 56) : 48);   // per-step addressing of the plain layout needs more registers, and so do the 16-register accumulator tuples of the 32 x 32 tiles
     static constexpr int KREDUCED = RP;                    // 0: fp32 filters; 1: packed filters hold bfloat16; 2: IEEE half
     static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
     static_assert(RP >= 0 && RP <= 2 && (RP == 0 || (QUAD && MT == 16 && U == 4)), "the 16-bit paths are the 16 x 16 x 16 form of the quad layout");
@@ -632,6 +632,7 @@ struct ConvWsplit {
     // QUAD: scalar state of the next batch to request (batches are requested in K order starting at s_begin)
     int q_cb = 0, q_kh = 0, q_kw = 0;
     unsigned q_w = 0;
+    const int c_lane_last = a.ICg - 1 - U * lk;   // QUAD: the lane's first channel of a batch starting at channel cb is real while cb <= c_lane_last
     if constexpr (QUAD) {
         const int kb = s_begin * M::KSTEP;
         const int tap = (int)__umulhi((unsigned)kb, a.magic_icgp);
@@ -640,13 +641,22 @@ struct ConvWsplit {
         q_kw = tap - q_kh * a.KW;
         q_w = (unsigned)((kb / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
     }
-    auto load_batch = [&](int s0, FilterStage &A, float(&B)[U][TN]) {
+    // `live` (wavefront-uniform) is false for a batch beyond the wavefront's K range: its loads are still issued, against
+    // descriptors of extent zero, and return zeros without touching memory.  Loads are never skipped by a branch inside
+    // the K loop: where a path with and a path without newly issued loads join, the compiler can only wait for *all*
+    // outstanding loads before the next use of an older one, which serialises load latency and matrix work.
+    // `ragged` (a std::bool_constant, QUAD only): the group's channel count is not a multiple of U, so the U channels of a lane
+    // can straddle the end of the real channels and every k-step needs its own test; otherwise a lane's channels are real or
+    // padding together and one test per batch, folded into the lane's offsets, covers them.
+    auto load_batch = [&](int s0, FilterStage &A, float(&B)[U][TN], bool live, auto ragged) {
         if constexpr (QUAD) {
             // The whole batch lies inside one tap (channels are padded to the batch).  Batches are requested in K
             // order, so (first channel, kh, kw) and the filter offset advance incrementally on the SALU.  Lane-constant
             // offsets go into the vector operand of the buffer loads, the per-batch / per-step parts into the scalar
             // operand: a filter load costs no VALU instruction, an input load one add + one or per batch and tile.
             (void)s0;
+            const __amdgpu_buffer_rsrc_t xr = buffer_of(a.x, live ? a.x_bytes : 0u);
+            const __amdgpu_buffer_rsrc_t wr = buffer_of(a.wp, live ? a.w_bytes : 0u);
             if constexpr (RP != 0) {
 #pragma unroll
                 for (int i = 0; i < TM; i++) {   // four 16-bit values = the lane's four k of this batch
@@ -673,8 +683,8 @@ struct ConvWsplit {
                 const unsigned in_w = (unsigned)(iw0[j] + q_kw) < (unsigned)a.W ? 1u : 0u;
                 voff[j] = (x_lane[j] + x_tap) | (((in_h & in_w) ^ 1u) << 31);
             }
-            if (q_cb + U * M::KSTEP > a.ICg) {   // wavefront-uniform: the last batch of a tap when channels are padded
-                const int c_left = a.ICg - 1 - q_cb - U * lk;   // channels of this lane beyond c_left are padding
+            const int c_left = c_lane_last - q_cb;   // channels of this lane beyond c_left are padding (the tap's last batch)
+            if constexpr (decltype(ragged)::value) {
 #pragma unroll
                 for (int u = 0; u < U; u++) {
                     const unsigned c_kill = (unsigned)(c_left - u) & kOutOfRange;   // sign bit
@@ -682,24 +692,26 @@ struct ConvWsplit {
                     for (int j = 0; j < TN; j++) B[u][j] = buffer_load_f32(xr, voff[j] | c_kill, x_chan + (unsigned)(u * a.HW) * 4u);
                 }
             } else {
+                const unsigned c_kill = (unsigned)c_left & kOutOfRange;   // all U channels of the lane at once
+#pragma unroll
+                for (int j = 0; j < TN; j++) voff[j] |= c_kill;
 #pragma unroll
                 for (int u = 0; u < U; u++)
 #pragma unroll
                     for (int j = 0; j < TN; j++) B[u][j] = buffer_load_f32(xr, voff[j], x_chan + (unsigned)(u * a.HW) * 4u);
             }
-            // next batch
+            // next batch (selects, not branches: the loop body stays one basic block)
             q_w += (unsigned)((U * M::KSTEP / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
             q_cb += U * M::KSTEP;
-            if (q_cb >= a.ICgP) {
-                q_cb = 0;
-                q_kw++;
-                if (q_kw == a.KW) {
-                    q_kw = 0;
-                    q_kh++;
-                }
-            }
+            const bool next_tap = q_cb >= a.ICgP;
+            q_cb = next_tap ? 0 : q_cb;
+            q_kw += next_tap ? 1 : 0;
+            const bool next_row = q_kw == a.KW;
+            q_kw = next_row ? 0 : q_kw;
+            q_kh += next_row ? 1 : 0;
             return;
         }
+        (void)live;   // steps at or beyond s_end are dead by their index
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const bool s_ok = (s0 + u) < s_end;
@@ -757,29 +769,67 @@ struct ConvWsplit {
     };
 
     const int batches = (s_end - s_begin + U - 1) / U;   // <= 0 for wavefronts beyond the end of K
-    if constexpr (D == 2) {
-        if (batches > 0) load_batch(s_begin, av[0], bv[0]);
-        for (int b = 0; b < batches; b += 2) {
-            if (b + 1 < batches) load_batch(s_begin + (b + 1) * U, av[1], bv[1]);
-            compute(av[0], bv[0]);
-            if (b + 1 < batches) {
-                if (b + 2 < batches) load_batch(s_begin + (b + 2) * U, av[0], bv[0]);
-                compute(av[1], bv[1]);
+    auto k_loop = [&](auto ragged) {
+        if (batches <= 0) return;
+        if constexpr (decltype(ragged)::value) {
+            // channel counts that are no multiple of U (a few tiny layers): one batch at a time
+            for (int b = 0; b < batches; b++) {
+                load_batch(s_begin + b * U, av[0], bv[0], true, ragged);
+                compute(av[0], bv[0]);
             }
-        }
-    } else {
-        // deeper pipeline: D batches requested before the first one is consumed (wavefront-uniform guards only)
+        } else if constexpr (D == 2) {
+            // Two stages, peeled so that every load sits in straight-line code: the steady state requests batch b + 1,
+            // consumes batch b, requests b + 2, consumes b + 1 with both requests known to be in range; the last one or two
+            // batches are consumed behind the loop.  The waits in front of the matrix instructions then count exactly the
+            // loads issued since, and the next batch's latency overlaps this batch's matrix work.  (The scheduling fences
+            // keep a stage's requests behind the matrix work that still reads the stage: moved ahead of it they need a
+            // second set of registers.)
+            load_batch(s_begin, av[0], bv[0], true, ragged);
+            int b = 0;
+            for (; b + 2 < batches; b += 2) {
+                load_batch(s_begin + (b + 1) * U, av[1], bv[1], true, ragged);
+                __builtin_amdgcn_sched_barrier(0);
+                compute(av[0], bv[0]);
+                __builtin_amdgcn_sched_barrier(0);
+                load_batch(s_begin + (b + 2) * U, av[0], bv[0], true, ragged);
+                __builtin_amdgcn_sched_barrier(0);
+                compute(av[1], bv[1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (b + 1 < batches) {
+                load_batch(s_begin + (b + 1) * U, av[1], bv[1], true, ragged);
+                __builtin_amdgcn_sched_barrier(0);
+                compute(av[0], bv[0]);
+                compute(av[1], bv[1]);
+            } else {
+                compute(av[0], bv[0]);
+            }
+        } else {
+            // deeper pipeline: D batches requested before the first one is consumed.  The loop body is straight-line
+            // (requests beyond the range are issued dead, see load_batch: at most D - 1 of them in the last round that
+            // requests anything); the last D batches are consumed behind the loop, where nothing is requested any more.
 #pragma unroll
-        for (int st = 0; st < D; st++)
-            if (st < batches) load_batch(s_begin + st * U, av[st], bv[st]);
-        for (int b = 0; b < batches; b += D) {
+            for (int st = 0; st < D; st++) load_batch(s_begin + st * U, av[st], bv[st], st < batches, ragged);
+            int b = 0;
+            for (; b + D < batches; b += D) {
+#pragma unroll
+                for (int st = 0; st < D; st++) {
+                    compute(av[st], bv[st]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_batch(s_begin + (b + st + D) * U, av[st], bv[st], b + st + D < batches, ragged);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
 #pragma unroll
             for (int st = 0; st < D; st++)
-                if (b + st < batches) {
-                    compute(av[st], bv[st]);
-                    if (b + st + D < batches) load_batch(s_begin + (b + st + D) * U, av[st], bv[st]);
-                }
+                if (b + st < batches) compute(av[st], bv[st]);
         }
+    };
+    if constexpr (QUAD) {
+        if ((a.ICg & (U - 1)) == 0) k_loop(std::false_type{});
+        else k_loop(std::true_type{});
+    } else {
+        k_loop(std::false_type{});
     }
 
     // partial tiles meet in LDS: element e of lane l of wavefront w lives at red[(w * E + e) * 64 + l]

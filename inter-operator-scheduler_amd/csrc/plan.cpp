@@ -374,6 +374,11 @@ private:
     // nobody else: the depth-wise kernel adds the k values (and applies the ReLU) in its loader, so the summing launch and its
     // output tensor disappear (the reference adds them with a kernel of its own, src/ios/ios_runtime.cu:1047-1057).
     void find_depthwise_sums() {
+        // The summing loader addresses every source with 31-bit byte offsets.  Where the sources will live is decided later
+        // (a source may become a window of a wider concatenation buffer), so the test assumes the widest tensor of the graph
+        // as the batch stride; a sum that could exceed the range keeps its own launch and the generic depth-wise path.
+        unsigned long long widest = 0;
+        for (const PNode &n : nodes_) widest = std::max(widest, (unsigned long long)n.C * n.H * n.W);
         for (const auto &seq : sequentials_) {
             for (int i = seq.first; i <= seq.second; i++) {
                 PNode &dw = nodes_[i];
@@ -392,6 +397,7 @@ private:
                 }
                 const PNode &f = nodes_[front];
                 if (f.inputs.size() != 1 || f.inputs[0].size() < 2 || f.inputs[0].size() > (size_t)kMaxNaryInputs) continue;
+                if (((unsigned long long)(batch_ - 1) * widest + (unsigned long long)pd.IC * pd.H * pd.W) * 4ull >= (1ull << 31)) continue;
                 dw.sum_front = front;
                 dw.sum_relu = relu;
                 if (front != i) {
@@ -999,6 +1005,7 @@ void json_escape(std::ostringstream &os, const std::string &s) {
 namespace {
 bool g_arena_reuse = true;
 long long g_thin_conv_min_pixels = 1LL << 18;
+int g_host_split_k = 0;
 }
 
 bool set_planner_option(const std::string &key, const std::string &value) {
@@ -1010,11 +1017,18 @@ bool set_planner_option(const std::string &key, const std::string &value) {
         g_thin_conv_min_pixels = atoll(value.c_str());
         return true;
     }
+    if (key == "host_plan_split_k") {   // K slices of every matrix-path convolution in plans made without a device (0: the model's choice)
+        const int v = atoi(value.c_str());
+        if (v < 0 || v > 64) throw std::runtime_error("option host_plan_split_k: expected 0..64");
+        g_host_split_k = v;
+        return true;
+    }
     return false;
 }
 
 bool planner_arena_reuse() { return g_arena_reuse; }
 long long planner_thin_conv_min_pixels() { return g_thin_conv_min_pixels; }
+int planner_host_split_k() { return g_host_split_k; }
 
 Plan build_plan(PlanMode mode, const Json &doc, const Json *extra, int batch, const LaunchChooser &chooser) {
     Planner planner(batch, chooser);
@@ -1069,6 +1083,12 @@ std::string describe_plan(const Plan &plan) {
         if (op.has_residual) reads.push_back(op.residual);
         ranges("writes", {op.out});
         ranges("reads", reads);
+        // a split-K convolution first writes, then reads its partial tiles: a region that shares addresses with other tensors
+        // like any other
+        if (op.conv >= 0 && plan.convs[op.conv].ws_floats > 0) {
+            const PlanConv &c = plan.convs[op.conv];
+            os << ",\"scratch\":[[" << c.ws_off << ',' << c.ws_off + c.ws_floats << "]]";
+        }
         os << '}';
     }
     os << ']';

@@ -115,5 +115,6 @@ std::string describe_plan(const Plan &plan);   // JSON array, one object per op
 bool set_planner_option(const std::string &key, const std::string &value);
 bool planner_arena_reuse();
 long long planner_thin_conv_min_pixels();
+int planner_host_split_k();   // option host_plan_split_k
 
 }  // namespace ios

@@ -385,6 +385,7 @@ std::string DeviceContext::info_json() const {
        << ",\"executor\":\"" << (exec_mode_ == ExecMode::Graph ? "graph" : exec_mode_ == ExecMode::Fused ? "fused" : exec_mode_ == ExecMode::FusedGraph ? "fused_graph" : "streams") << "\",\"autotune\":" << (autotune_ ? "true" : "false")
        << ",\"split_k_reduce\":\"" << (inline_reduce_ ? "inline" : "kernel") << "\""
        << ",\"precision\":\"" << (precision_ == PREC_BF16 ? "bf16" : precision_ == PREC_FP16 ? "fp16" : "fp32") << "\""
+       << ",\"conv_variant\":" << forced_variant_ << ",\"conv_split_k\":" << forced_split_k_
        << ",\"arena_reuse\":" << (planner_arena_reuse() ? "true" : "false")
        << ",\"max_groups\":" << kMaxGroups << ",\"conv_variants\":[";
     for (int i = 0; i < conv_num_variants(); i++) os << (i ? "," : "") << '"' << conv_variant(i).name << '"';

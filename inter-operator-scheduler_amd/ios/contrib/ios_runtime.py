@@ -61,6 +61,8 @@ def _declare(handle):
     handle.ios_plan_describe.restype = i
     handle.ios_plan_arena_bytes.argtypes = [s, i]
     handle.ios_plan_arena_bytes.restype = ctypes.c_longlong
+    handle.ios_device_free_bytes.argtypes = []
+    handle.ios_device_free_bytes.restype = ctypes.c_longlong
     handle.ios_session_create.argtypes = [s, i]
     handle.ios_session_create.restype = vp
     handle.ios_session_destroy.argtypes = [vp]
@@ -120,6 +122,14 @@ def device_info() -> dict:
     buf = ctypes.create_string_buffer(4096)
     _check(get_lib().ios_device_info(buf, len(buf)), 'ios_device_info')
     return json.loads(buf.value.decode())
+
+
+def device_free_bytes() -> int:
+    """Free device memory in bytes (hipMemGetInfo)."""
+    free = get_lib().ios_device_free_bytes()
+    if free < 0:
+        _check(1, 'ios_device_free_bytes')
+    return int(free)
 
 
 def conv_variant_names() -> List[str]:

@@ -207,6 +207,8 @@ def test_bench_refuses_more_than_one_gpu():
 def _simulate(ops):
     """Runs a plan symbolically: every float of the arena remembers the operation that wrote it last.  Returns, per
     operation, the writers it sees in what it reads; fails when two groups of one stage touch each other's memory."""
+    # (`scratch`: the partial tiles of a split-K convolution, written and then read by that operation alone)
+    ops = [dict(op, writes=op['writes'] + op.get('scratch', [])) for op in ops]
     end = max(r[1] for op in ops for key in ('writes', 'reads') for r in op[key])
     writer = np.full(end, -1, dtype=np.int32)
     seen = []
@@ -267,6 +269,28 @@ def test_arena_reuse_never_lets_an_operator_read_what_another_overwrote(name, ba
     for op in shared:
         for begin, stop in op['writes']:
             assert all(e <= begin or stop <= b for b, e in first_reads), op['node']
+
+
+def test_split_k_partial_tiles_share_the_arena_like_any_other_region():
+    # every convolution forced to four K slices: their partial tiles are regions with a lifetime of one stage, so they share
+    # addresses with tensors that are dead by then, and must never land on one that a later operation still reads
+    graph = ios.models.inception_v3()
+    graph.greedy_schedule(8)
+    try:
+        rt.set_option('host_plan_split_k', 4)
+        rt.set_option('arena_reuse', 0)
+        plain = rt.plan_describe(graph, 2)
+        rt.set_option('arena_reuse', 1)
+        shared = rt.plan_describe(graph, 2)
+    finally:
+        rt.set_option('host_plan_split_k', 0)
+        rt.set_option('arena_reuse', 1)
+    with_scratch = [op for op in shared if op.get('scratch')]
+    assert len(with_scratch) > 50 and all(op['split_k'] == 4 for op in with_scratch)
+    assert _simulate(shared) == _simulate(plain)
+    # the partial tiles do share addresses with operator outputs in the reusing plan (the test above would be vacuous otherwise)
+    outputs = [r for op in shared for r in op['writes']]
+    assert any(b < e2 and b2 < e for op in with_scratch for b, e in op['scratch'] for b2, e2 in outputs)
 
 
 def test_residual_additions_join_the_activation_behind_them_and_pool_names_follow_the_reference():

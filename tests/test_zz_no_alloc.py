@@ -14,8 +14,12 @@ from oracle import ios_oracle
 pytestmark = pytest.mark.gpu
 
 
+OPTIONS = ('conv_variant', 'conv_split_k', 'autotune', 'executor', 'precision', 'split_k_reduce')
+
+
 @pytest.fixture(autouse=True)
 def closed_form_configurations():
+    before = rt.device_info()      # the options in force, put back afterwards whatever the order of the tests
     rt.set_option('conv_variant', -1)
     rt.set_option('conv_split_k', 0)
     rt.set_option('autotune', 0)
@@ -23,8 +27,9 @@ def closed_form_configurations():
     rt.set_option('precision', 'fp32')
     rt.set_option('split_k_reduce', 'inline')
     yield
-    rt.set_option('conv_split_k', 0)
-    rt.set_option('executor', 'streams')
+    for key in OPTIONS:
+        value = before[key]
+        rt.set_option(key, int(value) if isinstance(value, bool) else value)
 
 
 def both(graph, batch, seed):
@@ -33,6 +38,22 @@ def both(graph, batch, seed):
     static = rt.graph_inference(graph, batch, x, no_alloc=True)
     np.testing.assert_array_equal(static, plain)
     return x, static
+
+
+def test_the_call_allocates_no_device_memory():
+    graph = ios.models.squeezenet_1_1(init_seed=0, init_scheme='he_normal_bias')
+    graph.greedy_schedule(4)
+    x = np.random.default_rng(0).standard_normal((2, 3, 224, 224)).astype(np.float32)
+    rt.device_info()                                   # the device context (streams, address of the static array) exists from here on
+    rt.graph_inference(graph, 2, x, no_alloc=True)     # (and whatever the HIP runtime sets up on a first launch)
+    free = rt.device_free_bytes()
+    for batch in (2, 1, 2):
+        got = rt.graph_inference(graph, batch, x[:batch], no_alloc=True)
+        assert rt.device_free_bytes() == free          # nothing allocated, nothing freed
+    np.testing.assert_array_equal(got, rt.graph_inference(graph, 2, x))
+    # a session, which owns an allocation, does move the figure (the check above is not vacuous)
+    with rt.Session(graph, 2):
+        assert rt.device_free_bytes() < free
 
 
 def test_two_calls_in_a_row_the_second_smaller_equal_graph_inference():
