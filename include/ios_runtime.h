@@ -74,6 +74,13 @@ int graph_inference(const char *graph_json, int batch_size, float *input, int nu
 int graph_inference_no_alloc(const char *graph_json, int batch_size, float *input, int num_convs, char **conv_names,
                              float **filter_data, float **bias_data, float *output);
 
+/* Numbering of the blocks of a split-K convolution whose K slices meet inside one XCD (host only, for tests): for a
+ * launch over `tiles` output tiles and `split` K slices, writes for every block of the grid the tile it works on (-1:
+ * the block has none and ends at once) and its slice, and returns the number of blocks; with null arrays or a capacity
+ * below that number only the number is returned.  Blocks whose indices are equal modulo 8 run on one XCD, and all
+ * slices of a tile have such indices. */
+int ios_xcd_numbering(int tiles, int split, int *tile_of_block, int *slice_of_block, int capacity);
+
 /* Free device memory in bytes as hipMemGetInfo reports it (creates the device context if there is none yet), or -1. */
 long long ios_device_free_bytes(void);
 
@@ -86,8 +93,13 @@ const char *ios_last_error(void);
  *       captured into a hipGraph and replayed);
  *   "autotune" = "1" (default) | "0": measure convolution kernel configurations on first use, like the reference's
  *       cudnnFind-based selection (src/ios/ios_runtime.cu:150-205); "clear_tuning" = anything forgets them;
- *   "split_k_reduce" = "inline" (the last block of a tile adds the split-K slices inside the convolution kernel)
- *       | "kernel" (a second kernel adds them); same results bit for bit;
+ *   "split_k_reduce" = "xcd" (default: the last block of a tile adds the split-K slices inside the convolution kernel,
+ *       and the grid is numbered so that the slices of a tile run on one XCD and meet in its L2; used where a probe at
+ *       start-up finds the dispatcher's round-robin placement, every block checks its own placement, and a mismatch
+ *       makes the next synchronising call fail and switches the form off) | "inline" (the same with the slices anywhere
+ *       on the device, exchanged through memory) | "kernel" (a second kernel adds them); same results bit for bit;
+ *   "host_plan_split_k" = N: K slices of every matrix-path convolution in plans made without a device
+ *       (ios_plan_describe, ios_plan_arena_bytes; 0 = the closed-form model's choice);
  *   "precision" = "fp32" | "bf16" | "fp16": reduced-precision modes of the matrix-path convolutions (bfloat16 or IEEE half
  *       operands, fp32 accumulation and outputs); "fp16" is the counterpart of the reference's USE_FLOAT16 build option
  *       (src/ios/ios_runtime.cu:19-43), with its range (operands beyond 65504 become infinite);

@@ -10,6 +10,7 @@
 #include "../../include/ios_runtime.h"
 #include "plan.h"
 #include "runtime.h"
+#include "conv_body.h"
 
 namespace {
 
@@ -149,6 +150,24 @@ long long ios_device_free_bytes(void) {
         bytes = (long long)free_bytes;
     });
     return bytes;
+}
+
+int ios_xcd_numbering(int tiles, int split, int *tile_of_block, int *slice_of_block, int capacity) {
+    int blocks = -1;
+    guarded([&]() {
+        if (tiles < 1 || split < 1) throw std::runtime_error("xcd numbering: tiles >= 1 and split >= 1 required");
+        blocks = ios::xcd_grid_blocks(tiles, split);
+        if (tile_of_block == nullptr || slice_of_block == nullptr || capacity < blocks) return;
+        const int q = tiles >> 3, r = tiles & 7;
+        for (int b = 0; b < blocks; b++) {
+            const ios::XcdSlot slot = ios::xcd_slot(b, (b >> 3) / split, q, r, split);
+            // the tile a block works on, as the kernels derive it from the slot (xcd_tile)
+            const int c = slot.tile & 7, in_class = slot.tile >> 3;
+            tile_of_block[b] = slot.idle ? -1 : in_class + c * q + (c < r ? c : r);
+            slice_of_block[b] = slot.slice;
+        }
+    });
+    return blocks;
 }
 
 int ios_conv_variant_names(char *buf, int cap) {

@@ -66,7 +66,8 @@ struct ConvKernelArgs {
     float *ws;
     unsigned *counters;               // split-K tickets, one per (group, tile), zero between launches; null: two-kernel split-K
     int H, W, OH, OW, sh, sw, ph, pw;
-    int KW, taps;                     // taps = KH * KW
+    int KW;
+    int xcd_local;                    // split-K inside one XCD, see below
     unsigned magic_icgp, magic_kw;    // floor(2^32 / d) + 1: exact quotients for dividends < 2^16
     int ICg, ICgP, OCg, OCgP, Kq, HW, OHW, groups;   // Kq = taps * ICgP rows of the packed filter matrix
     long long x_bs, y_bs;
@@ -81,11 +82,89 @@ struct ConvKernelArgs {
     int tile_div;        // tiles_n (weights_major) or tiles_m
     FastDiv div_tile;    // by tile_div
     FastDiv div_ohw, div_ow;
-    // residual form: y = res + act(conv + bias), then max(., 0) when post_relu; res is a dense view of the output's
-    // shape (batch stride res_bs elements), null for a plain convolution
-    const float *res;
-    int res_bs, post_relu;
+    // Either the residual form (stand-alone kernels only): y = res + act(conv + bias), then max(., 0) when post_relu; res is a
+    // dense view of the output's shape (batch stride res_bs elements), null for a plain convolution.
+    // Or split-K inside one XCD (xcd_local != 0; plain convolutions without groups, counters set): the grid is numbered so
+    // that all K slices of an output tile run on the same XCD and meet in that XCD's L2 (see XcdSlot).  xcd_map: the XCC id
+    // that blocks with index % 8 == c run on, four bits per c, as measured when the device context was created; fault: a
+    // word in host memory that a block finding itself elsewhere sets to 1 (the host then stops using this form);
+    // magic_split = floor(2^32 / split_k) + 1: exact quotients by split_k for dividends below 2^26.
+    union {
+        struct {
+            const float *res;
+            int res_bs, post_relu;
+        };
+        struct {
+            unsigned *fault;
+            unsigned xcd_map, magic_split;
+        };
+    };
 };
+
+// Numbering of the blocks of a launch whose K slices meet inside one XCD.  The dispatcher deals workgroups to the XCDs
+// round-robin, so the blocks with index % 8 == c share an XCD.  Class c owns the tiles [c * q + min(c, r), ...) (q + 1 of
+// them for c < r, q for the others, where tiles = 8 q + r, the same ranges xcd_tile() uses) and its blocks, in index order,
+// are (first tile, slice 0), (first tile, slice 1), ... : a launch has 8 * split * (q + (r > 0)) blocks, of which the last
+// ones of the classes c >= r (when r > 0) have no tile and end at once.  `tile` is the value xcd_tile() takes
+// (slot-in-class * 8 + c), which also numbers the tile's partial sums and its ticket: those arrays have
+// 8 * (q + (r > 0)) entries.
+struct XcdSlot {
+    int tile, slice;
+    bool idle;
+};
+__host__ __device__ inline int xcd_padded_tiles(int tiles) { return 8 * ((tiles + 7) / 8); }
+__host__ __device__ inline int xcd_grid_blocks(int tiles, int split) { return xcd_padded_tiles(tiles) * split; }
+__host__ __device__ inline XcdSlot xcd_slot(int local, int tile_in_class, int xcd_q, int xcd_r, int split) {
+    // local: index of the block inside the launch (or inside its item of a fused launch); tile_in_class = (local / 8) / split
+    const int c = local & 7;
+    XcdSlot s;
+    s.slice = (local >> 3) - tile_in_class * split;
+    s.tile = tile_in_class * 8 + c;
+    s.idle = tile_in_class >= xcd_q + (c < xcd_r ? 1 : 0);
+    return s;
+}
+
+// XCC id of the executing wavefront (bits 3:0 of the hardware register XCC_ID)
+__device__ __forceinline__ unsigned xcc_id() { return __builtin_amdgcn_s_getreg(20 | (3 << 11)); }
+
+// One block of an XCD-local split-K launch: its slot, and the check that the dispatcher put it where the numbering assumes.
+// `block` is the block's index in the whole launch (the XCD follows from it), `local` its index inside the convolution.
+__device__ __forceinline__ XcdSlot xcd_enter(const ConvKernelArgs &a, int block, int local) {
+    const XcdSlot s = xcd_slot(local, (int)__umulhi((unsigned)local >> 3, a.magic_split), a.xcd_q, a.xcd_r, a.split_k);
+    const unsigned expected = (a.xcd_map >> (4 * (block & 7))) & 15u;
+    if (xcc_id() != expected && threadIdx.x == 0) __hip_atomic_store(a.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    return s;
+}
+
+// Partial sums and tickets of the one-kernel split-K.  Device-wide form: the slices of a tile run on different XCDs, whose
+// L2s are not coherent with each other, so partial sums travel with agent-scope stores and loads (written through to and
+// read from memory) and the ticket is an agent-scope atomic.  XCD-local form: all slices share one L2; plain stores are
+// written through the L1 to that L2, the ticket is a workgroup-scope atomic (executed in the L2), and the sums are read
+// with workgroup-scope loads, which do not use a line the L1 might hold.  In both forms a block waits for its stores to
+// be acknowledged before it takes its ticket.
+template <bool LOCAL>
+__device__ __forceinline__ void partial_store(float *p, float v) {
+    if constexpr (LOCAL) *p = v;
+    else __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <bool LOCAL>
+__device__ __forceinline__ float partial_load(const float *p) {
+    if constexpr (LOCAL) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    else return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// thread 0 of the block: draws the tile's ticket; the block that draws the last one puts the counter back to zero
+template <bool LOCAL>
+__device__ __forceinline__ int draw_ticket(unsigned *counter, int split_k) {
+    unsigned ticket;
+    if constexpr (LOCAL) ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    else ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int last = ticket == (unsigned)split_k - 1u ? 1 : 0;
+    if (last) {
+        if constexpr (LOCAL) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        else __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return last;
+}
 
 // v = act(conv + bias) of output element (image b, channel, pixel r): adds the residual operand.  The residual form is a
 // compile-time property of a body (RES): the plain form, which every fused stage launch uses, carries no test for it.
@@ -409,50 +488,47 @@ struct ConvTiled {
         constexpr int T0 = 64 * WM * WN;
         constexpr int E = TM * TN * M::ACC;
         static_assert(T0 * E == BM * BN, "accumulator layout covers the tile");
-        const size_t tiles = (size_t)a.tiles_m * a.tiles_n;
+        const size_t tiles = (size_t)xcd_padded_tiles(a.tiles_m * a.tiles_n);   // (both forms size their arrays for the padded count)
         float *slices = a.ws + (((size_t)g * tiles + tile) * a.split_k) * (size_t)(BM * BN);
-        if (wk == 0) {
-            float *mine = slices + (size_t)z * (BM * BN) + tid;
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-#pragma unroll
-                    for (int v = 0; v < M::ACC; v++)
-                        __hip_atomic_store(mine + ((i * TN + j) * M::ACC + v) * T0, acc[i][j][v], __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        unsigned *counter = a.counters + (size_t)g * tiles + tile;
         int *last_flag = reinterpret_cast<int *>(smem);
-        if (tid == 0) {
-            unsigned *counter = a.counters + (size_t)g * tiles + tile;
-            const unsigned ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const int last = ticket == (unsigned)a.split_k - 1u ? 1 : 0;
-            if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
-            *last_flag = last;
-        }
-        __syncthreads();
-        if (*last_flag == 0) return;
-        if (wk == 0) {
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-#pragma unroll
-                    for (int v = 0; v < M::ACC; v++) acc[i][j][v] = 0.f;
-            for (int s = 0; s < a.split_k; s++) {
-                const float *theirs = slices + (size_t)s * (BM * BN) + tid;
+        auto exchange = [&](auto local) -> bool {   // true: this block drew the last ticket and holds the sum of all slices
+            constexpr bool LOCAL = decltype(local)::value;
+            if (wk == 0) {
+                float *mine = slices + (size_t)z * (BM * BN) + tid;
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
                     for (int j = 0; j < TN; j++)
 #pragma unroll
-                        for (int v = 0; v < M::ACC; v++)
-                            acc[i][j][v] += __hip_atomic_load(theirs + ((i * TN + j) * M::ACC + v) * T0, __ATOMIC_RELAXED,
-                                                              __HIP_MEMORY_SCOPE_AGENT);
+                        for (int v = 0; v < M::ACC; v++) partial_store<LOCAL>(mine + ((i * TN + j) * M::ACC + v) * T0, acc[i][j][v]);
             }
-        }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (tid == 0) *last_flag = draw_ticket<LOCAL>(counter, a.split_k);
+            __syncthreads();
+            if (*last_flag == 0) return false;
+            if (wk == 0) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+#pragma unroll
+                        for (int v = 0; v < M::ACC; v++) acc[i][j][v] = 0.f;
+                for (int s = 0; s < a.split_k; s++) {
+                    const float *theirs = slices + (size_t)s * (BM * BN) + tid;
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++)
+#pragma unroll
+                            for (int v = 0; v < M::ACC; v++) acc[i][j][v] += partial_load<LOCAL>(theirs + ((i * TN + j) * M::ACC + v) * T0);
+                }
+            }
+            return true;
+        };
+        const bool last = a.xcd_local ? exchange(std::true_type{}) : exchange(std::false_type{});
+        if (!last) return;
     }
 
     // ---- epilogue -------------------------------------------------------------------------------------------
@@ -857,36 +933,40 @@ struct ConvWsplit {
     if (a.split_k > 1) {
         // one-kernel split-K, as in the LDS-tiled kernel: partial tiles in [element][lane] order, a ticket per
         // tile, the block drawing the last ticket adds the slices in slice order
-        const size_t tiles = (size_t)a.tiles_m * a.tiles_n;
+        const size_t tiles = (size_t)xcd_padded_tiles(a.tiles_m * a.tiles_n);
         slices = a.ws + (((size_t)g * tiles + tile) * a.split_k) * (size_t)(BM * BN);
-        float *mine = slices + (size_t)z * (BM * BN) + lane;
-        for (int e = wave; e < E; e += NW) {
-            float sum = 0.f;
-#pragma unroll
-            for (int w = 0; w < NW; w++) sum += red[(w * E + e) * 64 + lane];
-            __hip_atomic_store(mine + e * 64, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        unsigned *counter = a.counters + (size_t)g * tiles + tile;
         int *last_flag = reinterpret_cast<int *>(red);
-        if (tid == 0) {
-            unsigned *counter = a.counters + (size_t)g * tiles + tile;
-            const unsigned ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const int last = ticket == (unsigned)a.split_k - 1u ? 1 : 0;
-            if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            *last_flag = last;
-        }
+        auto hand_in = [&](auto local) {
+            constexpr bool LOCAL = decltype(local)::value;
+            float *mine = slices + (size_t)z * (BM * BN) + lane;
+            for (int e = wave; e < E; e += NW) {
+                float sum = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; w++) sum += red[(w * E + e) * 64 + lane];
+                partial_store<LOCAL>(mine + e * 64, sum);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (tid == 0) *last_flag = draw_ticket<LOCAL>(counter, a.split_k);
+        };
+        if (a.xcd_local) hand_in(std::true_type{});
+        else hand_in(std::false_type{});
         __syncthreads();
         if (*last_flag == 0) return;
     }
+    const bool xcd_local = a.xcd_local != 0;
 #pragma unroll
     for (int t = 0; t < EPW; t++) {
         const int e = wave + t * NW;
         if (e >= E) break;
         float sum = 0.f;
         if (a.split_k > 1) {
-            for (int s2 = 0; s2 < a.split_k; s2++)
-                sum += __hip_atomic_load(slices + (size_t)s2 * (BM * BN) + e * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float *theirs = slices + e * 64 + lane;
+            if (xcd_local)
+                for (int s2 = 0; s2 < a.split_k; s2++) sum += partial_load<true>(theirs + (size_t)s2 * (BM * BN));
+            else
+                for (int s2 = 0; s2 < a.split_k; s2++) sum += partial_load<false>(theirs + (size_t)s2 * (BM * BN));
         } else {
 #pragma unroll
             for (int w = 0; w < NW; w++) sum += red[(w * E + e) * 64 + lane];
@@ -999,6 +1079,20 @@ struct ConvWsplit {
     X(76, "wh_m64n32_w8", 16, 4, 2, 8, 4, true, 2, 2)       \
     X(77, "wh_m64n32_w4_d4", 16, 4, 2, 4, 4, true, 4, 2)    \
     X(78, "wh_m64n64_w4", 16, 4, 4, 4, 4, true, 2, 2)
-constexpr int kNumConvVariants = 79;
+// X(index, name, MT, TM, TN, NW, U, QUAD, D, RP): quad-load configurations with one or two wavefronts per output tile, for
+// layers with many pixels and a short K (the first layers of an image network at batch 1, everything at large batches):
+// a wavefront walks (half of) K by itself, its next batch's loads in flight under this batch's matrix instructions
+#define IOS_WSPLIT_LONGK_VARIANTS(X)                                  \
+    X(79, "wq_m32n32_w1_t32", 32, 1, 1, 1, 8, true, 2, 0)             \
+    X(80, "wq_m32n32_w2_t32", 32, 1, 1, 2, 8, true, 2, 0)             \
+    X(81, "wq_m64n32_w2_t32", 32, 2, 1, 2, 8, true, 2, 0)             \
+    X(82, "wq_m64n32_w1_t32", 32, 2, 1, 1, 8, true, 2, 0)             \
+    X(83, "wq_m32n64_w2_t32", 32, 1, 2, 2, 8, true, 2, 0)             \
+    X(84, "wq_m32n32_w2_t32_d4", 32, 1, 1, 2, 8, true, 4, 0)          \
+    X(85, "wq_m64n32_w2_t32_u4_d4", 32, 2, 1, 2, 4, true, 4, 0)       \
+    X(86, "wq_m32n32_w1_t16_d4", 16, 2, 2, 1, 4, true, 4, 0)          \
+    X(87, "wq_m64n32_w1_t16", 16, 4, 2, 1, 4, true, 2, 0)             \
+    X(88, "wq_m64n64_w2_t32", 32, 2, 2, 2, 8, true, 2, 0)
+constexpr int kNumConvVariants = 89;
 
 }  // namespace ios

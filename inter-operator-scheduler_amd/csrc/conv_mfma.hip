@@ -13,6 +13,12 @@ namespace ios {
 template <typename Body, bool RES = false>
 __global__ __launch_bounds__(Body::THREADS) void conv_kernel(ConvKernelArgs a) {
     extern __shared__ floatx4 conv_smem[];
+    if (a.xcd_local) {   // one-dimensional grid numbered for split-K inside an XCD
+        const XcdSlot slot = xcd_enter(a, blockIdx.x, blockIdx.x);
+        if (slot.idle) return;
+        Body::template run<RES>(a, reinterpret_cast<float *>(conv_smem), slot.tile, 0, slot.slice);
+        return;
+    }
     Body::template run<RES>(a, reinterpret_cast<float *>(conv_smem), blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
@@ -45,7 +51,8 @@ struct VariantEntry {
 
 static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)
                                              IOS_WSPLIT_C4_VARIANTS(IOS_WSPLIT_C4_ENTRY)
-                                             IOS_WSPLIT_T32_VARIANTS(IOS_WSPLIT_ENTRY) IOS_WSPLIT_F16_VARIANTS(IOS_WSPLIT_ENTRY)};
+                                             IOS_WSPLIT_T32_VARIANTS(IOS_WSPLIT_ENTRY) IOS_WSPLIT_F16_VARIANTS(IOS_WSPLIT_ENTRY)
+                                             IOS_WSPLIT_LONGK_VARIANTS(IOS_WSPLIT_ENTRY)};
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 static_assert(kNumVariants == kNumConvVariants, "variant lists and count disagree");
 
@@ -76,16 +83,18 @@ int conv_effective_split(const ConvProblem &p, const ConvLaunch &l) { return eff
 size_t conv_workspace_floats(const ConvProblem &p, const ConvLaunch &l) {
     const int s = effective_split(p, l);
     if (s <= 1) return 0;
-    // two-kernel form: [slice][OC][pixels]; one-kernel form: [group][tile][slice][BM * BN]
+    // two-kernel form: [slice][OC][pixels]; one-kernel forms: [group][tile][slice][BM * BN] with the tile count rounded up
+    // to a multiple of 8 (the numbering of the XCD-local form, see XcdSlot)
     const ConvVariant &v = kVariants[l.variant].v;
-    const size_t padded = (size_t)p.groups * ceil_div(p.OCg(), v.BM) * (size_t)ceil_div(p.Npix(), v.BN) * v.BM * v.BN;
+    const size_t tiles = (size_t)xcd_padded_tiles(ceil_div(p.OCg(), v.BM) * ceil_div(p.Npix(), v.BN));
+    const size_t padded = (size_t)p.groups * tiles * v.BM * v.BN;
     return (size_t)s * std::max((size_t)p.OC * (size_t)p.Npix(), padded);
 }
 
 size_t conv_counter_count(const ConvProblem &p, const ConvLaunch &l) {
     if (effective_split(p, l) <= 1) return 0;
     const ConvVariant &v = kVariants[l.variant].v;
-    return (size_t)p.groups * ceil_div(p.OCg(), v.BM) * (size_t)ceil_div(p.Npix(), v.BN);
+    return (size_t)p.groups * (size_t)xcd_padded_tiles(ceil_div(p.OCg(), v.BM) * ceil_div(p.Npix(), v.BN));
 }
 
 static int variant_by_name(const char *name) {
@@ -170,7 +179,7 @@ bool conv_matrix_path_supported(const ConvProblem &p) {
 }
 
 ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
-                                const float *bias, const TensorView &y, float *workspace, unsigned *counters,
+                                const float *bias, const TensorView &y, float *workspace, const SplitKReduce &reduce,
                                 const TensorView *residual, bool post_relu) {
     if (l.variant < 0 || l.variant >= kNumVariants) throw std::runtime_error("conv: bad variant");
     const VariantEntry &e = kVariants[l.variant];
@@ -185,10 +194,10 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     a.bias = bias;
     a.y = y.ptr;
     a.ws = workspace;
-    a.counters = counters;
+    a.counters = reduce.counters;
     a.H = p.H; a.W = p.W; a.OH = p.OH; a.OW = p.OW;
     a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw;
-    a.KW = p.KW; a.taps = p.KH * p.KW;
+    a.KW = p.KW;
     a.ICg = p.ICg(); a.ICgP = p.ICgP(e.v.cpad); a.OCg = p.OCg(); a.OCgP = p.OCgP(); a.Kq = p.Kq(e.v.cpad);
     a.magic_icgp = (unsigned)((1ULL << 32) / (unsigned)a.ICgP + 1);   // ICgP >= 8
     a.magic_kw = (unsigned)((1ULL << 32) / (unsigned)a.KW + 1);       // unused when KW == 1
@@ -241,6 +250,18 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     d.groups = p.groups;
     d.slices = a.split_k;
     if (a.split_k <= 1) a.counters = nullptr;
+    // K slices that meet inside an XCD: a one-dimensional grid in the numbering of XcdSlot (plain convolutions without
+    // groups; the fields share their place with those of the residual form)
+    a.xcd_local = a.counters != nullptr && reduce.xcd_local && reduce.fault != nullptr && p.groups == 1 && residual == nullptr &&
+                          a.split_k <= 64 && xcd_grid_blocks(d.tiles, a.split_k) / 8 < (1 << 26)
+                      ? 1 : 0;
+    d.xcd_blocks = 0;
+    if (a.xcd_local) {
+        a.fault = reduce.fault;
+        a.xcd_map = reduce.xcd_map;
+        a.magic_split = (unsigned)((1ULL << 32) / (unsigned)a.split_k + 1);
+        d.xcd_blocks = xcd_grid_blocks(d.tiles, a.split_k);
+    }
     d.has_reduce = a.split_k > 1 && a.counters == nullptr;
     d.reduce_blocks = 0;
     if (d.has_reduce) {
@@ -264,12 +285,12 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
 }
 
 void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
-                      const float *bias, const TensorView &y, float *workspace, unsigned *counters, hipStream_t stream,
+                      const float *bias, const TensorView &y, float *workspace, const SplitKReduce &reduce, hipStream_t stream,
                       const TensorView *residual, bool post_relu) {
-    const ConvDispatch d = make_conv_dispatch(p, l, x, packed, bias, y, workspace, counters, residual, post_relu);
+    const ConvDispatch d = make_conv_dispatch(p, l, x, packed, bias, y, workspace, reduce, residual, post_relu);
     const VariantEntry &e = kVariants[d.variant];
-    const dim3 grid((unsigned)d.tiles, (unsigned)d.groups, (unsigned)d.slices);
-    hipLaunchKernelGGL(d.args.res != nullptr ? e.kernel_residual : e.kernel, grid, dim3(d.threads), d.smem_bytes, stream, d.args);
+    const dim3 grid = d.xcd_blocks > 0 ? dim3((unsigned)d.xcd_blocks) : dim3((unsigned)d.tiles, (unsigned)d.groups, (unsigned)d.slices);
+    hipLaunchKernelGGL(!d.args.xcd_local && d.args.res != nullptr ? e.kernel_residual : e.kernel, grid, dim3(d.threads), d.smem_bytes, stream, d.args);
     if (d.has_reduce) hipLaunchKernelGGL(splitk_reduce_kernel, dim3(d.reduce_blocks), dim3(256), 0, stream, d.reduce);
 }
 

@@ -28,10 +28,19 @@ __device__ __forceinline__ void fused_item(const WorkItem &item, const int bid, 
             if constexpr (!MATRIX) return;
             if ((int)threadIdx.x >= item.threads) return;   // surplus wavefronts of a narrower body
             const ConvKernelArgs &a = item.conv;   // fields are fetched with scalar loads where they are used
-            const int rest = (int)fast_div((unsigned)local, item.div_tiles);
-            const int tile = local - rest * item.tiles;
-            const int z = (int)fast_div((unsigned)rest, item.div_groups);
-            const int g = rest - z * item.groups;
+            int tile, z, g;
+            if (a.xcd_local) {   // blocks numbered so that the K slices of a tile share an XCD (the XCD follows from bid)
+                const XcdSlot slot = xcd_enter(a, bid, local);
+                if (slot.idle) return;
+                tile = slot.tile;
+                z = slot.slice;
+                g = 0;
+            } else {
+                const int rest = (int)fast_div((unsigned)local, item.div_tiles);
+                tile = local - rest * item.tiles;
+                z = (int)fast_div((unsigned)rest, item.div_groups);
+                g = rest - z * item.groups;
+            }
             switch (item.variant) {
 #define IOS_CASE_TILED(IDX, NAME, BM, BN, BK, WM, WN, WK, MT, PD)                                          \
     case IDX:                                                                                              \
@@ -53,6 +62,7 @@ __device__ __forceinline__ void fused_item(const WorkItem &item, const int bid, 
                 IOS_WSPLIT_C4_VARIANTS(IOS_CASE_WSPLIT_C4)
                 IOS_WSPLIT_T32_VARIANTS(IOS_CASE_WSPLIT)
                 IOS_WSPLIT_F16_VARIANTS(IOS_CASE_WSPLIT)
+                IOS_WSPLIT_LONGK_VARIANTS(IOS_CASE_WSPLIT)
 #undef IOS_CASE_WSPLIT_C4
 #undef IOS_CASE_TILED
 #undef IOS_CASE_WSPLIT

@@ -87,12 +87,21 @@ size_t conv_packed_floats(const ConvProblem &p, const ConvLaunch &l);
 size_t conv_packed_floats_max(const ConvProblem &p);   // over all configurations
 void launch_pack_filters(const ConvProblem &p, const ConvLaunch &l, const float *w, float *packed, hipStream_t stream);
 
+// How the K slices of a split-K launch meet.  Without `counters` a second kernel adds them on the same stream.  With
+// counters (conv_counter_count of them, zero before the first launch) the block that finishes a tile last adds the slices
+// inside the kernel; `xcd_local` additionally numbers the grid so that the slices of a tile share an XCD and meet in its L2
+// (only for convolutions without groups; others silently use the device-wide form).  All forms add in slice order.
+struct SplitKReduce {
+    unsigned *counters = nullptr;
+    bool xcd_local = false;
+    unsigned xcd_map = 0;        // XCC id of the blocks with index % 8 == c, four bits per c (DeviceContext measures it)
+    unsigned *fault = nullptr;   // device-visible word in host memory, set to 1 by a block that runs on an unexpected XCC
+};
+
 // y = act(conv(x, w) + bias).  `packed` comes from launch_pack_filters.  `workspace` holds the split_k
-// partial outputs (conv_workspace_floats).  With split_k > 1 and `counters` (conv_counter_count) the block that
-// finishes a tile last adds the slices inside the kernel; without counters a second kernel adds them on the
-// same stream.  Both forms add in slice order.
+// partial outputs (conv_workspace_floats).
 void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
-                      const float *bias, const TensorView &y, float *workspace, unsigned *counters, hipStream_t stream,
+                      const float *bias, const TensorView &y, float *workspace, const SplitKReduce &reduce, hipStream_t stream,
                       const TensorView *residual = nullptr, bool post_relu = false);
 
 // Depth-wise convolution (groups == IC == OC), filters in their original [C][1][KH][KW] layout.  With `more`, the input is

@@ -38,9 +38,23 @@ public:
     void set_option(const std::string &key, const std::string &value);
     ExecMode exec_mode() const { return exec_mode_; }
     bool autotune() const { return autotune_; }
-    // split-K partial sums are added by the last block of a tile inside the convolution kernel (true) or by a
-    // second kernel (false)
-    bool inline_reduce() const { return inline_reduce_; }
+    // split-K partial sums are added by a second kernel (Kernel), by the last block of a tile inside the convolution
+    // kernel with the slices of a tile anywhere on the device (Inline), or the same with the slices of a tile numbered
+    // onto one XCD, where they meet in that XCD's L2 (Xcd; the default when the placement probe at start-up found the
+    // dispatcher's round-robin rule, and until a kernel reports a block somewhere else)
+    enum class ReduceMode { Kernel, Inline, Xcd };
+    ReduceMode reduce_mode() const { return reduce_mode_ == ReduceMode::Xcd && !xcd_usable_ ? ReduceMode::Inline : reduce_mode_; }
+    bool inline_reduce() const { return reduce_mode_ != ReduceMode::Kernel; }
+    // What the launchers take, for the mode in force and a launch on stream `group` of the pool.  The XCD a block lands
+    // on depends on the stream (every stream starts its round-robin at an XCC of its own), so the XCD-local form needs
+    // to know the stream; placement_known = false (kernels captured into a graph that forks: the replay runs them on
+    // streams of its own) gives the device-wide form.
+    SplitKReduce split_reduce(unsigned *counters, int group = 0, bool placement_known = true) const;
+    // Throws when a kernel of the XCD-local form has reported a block on another XCC than the numbering assumes (results
+    // of passes since the last check may be wrong); the form is switched off for the rest of the process first, so the
+    // caller's next plan uses the device-wide form.
+    void check_xcd_fault();
+    bool xcd_usable() const { return xcd_usable_; }
     // testing aid: force one kernel configuration for every matrix-path convolution (-1 / 0 = off)
     int forced_variant() const { return forced_variant_; }
     int forced_split_k() const { return forced_split_k_; }
@@ -72,7 +86,11 @@ private:
     float *static_scratch_ = nullptr;
     unsigned *tune_counters_ = nullptr;
     size_t tune_counter_count_ = 0;
-    bool inline_reduce_ = true;
+    ReduceMode reduce_mode_ = ReduceMode::Xcd;
+    bool xcd_usable_ = false;       // the start-up probe found blocks with equal index % 8 on one XCC, launch after launch
+    unsigned xcd_map_[kMaxGroups] = {};   // per stream of the pool: that XCC per index % 8, four bits each
+    unsigned *xcd_fault_ = nullptr; // one word of pinned host memory the kernels can write
+    void probe_xcd_placement();
     int precision_ = PREC_FP32;   // operand type of the matrix-path convolutions (reduced-precision modes: PREC_BF16, PREC_FP16)
     bool share_cost_rule_ = true;   // share classes weigh time by the held share of the device (false: hard footprint budgets)
     int share_threads_per_cu_ = 1024;   // resident threads per compute unit the share-class budgets assume (four wavefronts per SIMD)
@@ -144,7 +162,7 @@ public:
 private:
     void setup();
     void tune_convs();
-    void launch_op(const PlanOp &op, hipStream_t stream);
+    void launch_op(const PlanOp &op, int group);   // on stream `group` of the pool
     unsigned *counters_of(const PlanConv &c) const;
     void enqueue(bool stage_events);   // issue one forward pass according to the execution mode
     void enqueue_streams(bool stage_events);
@@ -174,6 +192,7 @@ private:
     void *fused_items_ = nullptr;                          // device copy of all work items
     std::vector<WorkItem> fused_items_host_;
     bool fused_built_ = false;
+    bool capturing_forks_ = false;   // a graph capture of the stream executor is under way (the replay chooses the streams)
     hipGraph_t graph_ = nullptr;
     ExecMode graph_mode_ = ExecMode::Graph;                // mode the captured graph was built for
     hipGraphExec_t graph_exec_ = nullptr;

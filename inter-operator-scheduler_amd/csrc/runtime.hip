@@ -58,6 +58,7 @@ DeviceContext::DeviceContext() {
     for (int i = 0; i < kMaxGroups; i++) IOS_HIP(hipStreamCreateWithFlags(&streams_[i], hipStreamNonBlocking));
     // the library runs on device 0 only, which is current here: its copy of the array is the one ever used
     IOS_HIP(hipGetSymbolAddress(reinterpret_cast<void **>(&static_scratch_), HIP_SYMBOL(scratch)));
+    probe_xcd_placement();
     const char *mode = getenv("IOS_EXECUTOR");
     if (mode != nullptr) set_option("executor", mode);
     const char *tune = getenv("IOS_AUTOTUNE");
@@ -67,6 +68,68 @@ DeviceContext::DeviceContext() {
         tune_cache_path_ = cache;
         load_tune_cache();
     }
+}
+
+// ---- placement of workgroups on XCDs --------------------------------------------------------------------------------
+// The XCD-local split-K relies on blocks with equal index % 8 running on one XCD (the dispatcher deals the workgroups of
+// a launch round-robin).  The rule is checked here, on launches of several sizes, before anything uses it, and every block
+// of such a launch checks its own XCC id again (xcd_enter).
+__global__ void xcc_probe_kernel(unsigned *out) {
+    if (threadIdx.x == 0) out[blockIdx.x] = xcc_id();
+}
+
+void DeviceContext::probe_xcd_placement() {
+    xcd_usable_ = false;
+    if (hipHostMalloc(reinterpret_cast<void **>(&xcd_fault_), 64, hipHostMallocMapped) != hipSuccess || xcd_fault_ == nullptr) {
+        xcd_fault_ = nullptr;
+        (void)hipGetLastError();
+        return;
+    }
+    *xcd_fault_ = 0;
+    constexpr int kMost = 1031;
+    unsigned *device = nullptr;
+    IOS_HIP(hipMalloc(reinterpret_cast<void **>(&device), kMost * sizeof(unsigned)));
+    std::vector<unsigned> host(kMost);
+    bool consistent = true;
+    // Measured on MI355X: inside a launch, block b runs on XCC (first + b) % 8, and `first` is a constant of the stream
+    // the launch goes to (launch after launch, alone or beside launches of other streams, also for the nodes that a
+    // captured graph runs on the stream it is launched on).
+    for (int g = 0; g < kMaxGroups; g++) {
+        int seen[8] = {-1, -1, -1, -1, -1, -1, -1, -1};
+        for (int blocks : {kMost, 8, 250}) {
+            for (int threads : {64, 512}) {
+                hipLaunchKernelGGL(xcc_probe_kernel, dim3(blocks), dim3(threads), 0, streams_[g], device);
+                IOS_HIP(hipMemcpyAsync(host.data(), device, blocks * sizeof(unsigned), hipMemcpyDeviceToHost, streams_[g]));
+                IOS_HIP(hipStreamSynchronize(streams_[g]));
+                for (int b = 0; b < blocks; b++) {
+                    if (seen[b & 7] < 0) seen[b & 7] = (int)host[b];
+                    consistent = consistent && seen[b & 7] == (int)host[b] && host[b] < 16;
+                }
+            }
+        }
+        xcd_map_[g] = 0;
+        for (int c = 0; c < 8; c++) xcd_map_[g] |= (unsigned)(seen[c] & 15) << (4 * c);
+    }
+    IOS_HIP(hipFree(device));
+    xcd_usable_ = consistent;
+}
+
+SplitKReduce DeviceContext::split_reduce(unsigned *counters, int group, bool placement_known) const {
+    SplitKReduce r;
+    r.counters = inline_reduce() ? counters : nullptr;
+    r.xcd_local = reduce_mode() == ReduceMode::Xcd && placement_known && group >= 0 && group < kMaxGroups;
+    r.xcd_map = r.xcd_local ? xcd_map_[group] : 0;
+    r.fault = xcd_fault_;
+    return r;
+}
+
+void DeviceContext::check_xcd_fault() {
+    if (xcd_fault_ == nullptr || *reinterpret_cast<volatile unsigned *>(xcd_fault_) == 0) return;
+    *xcd_fault_ = 0;
+    xcd_usable_ = false;
+    tuned.clear();
+    throw std::runtime_error("a split-K convolution found a workgroup on another XCD than the round-robin placement it relies on: results since the "
+                             "last synchronisation may be wrong.  The XCD-local form is switched off for the rest of this process; create the session again");
 }
 
 // ---- kernel configuration choice ----------------------------------------------------------------------------------
@@ -80,7 +143,8 @@ static std::string conv_signature(const ConvProblem &p) {
 // the measured winners of the share classes depend on these settings: they are part of every cache key
 std::string DeviceContext::settings_token() const {
     std::ostringstream os;
-    os << (share_cost_rule_ ? "cost" : "budget") << '/' << share_threads_per_cu_ << '/' << (inline_reduce_ ? "inline" : "kernel");
+    os << (share_cost_rule_ ? "cost" : "budget") << '/' << share_threads_per_cu_ << '/'
+       << (reduce_mode() == ReduceMode::Xcd ? "xcd" : reduce_mode() == ReduceMode::Inline ? "inline" : "kernel");
     return os.str();
 }
 
@@ -187,7 +251,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     auto measure = [&](const ConvLaunch &l, int reps) {
         const size_t ws = conv_workspace_floats(p, l);
         float *workspace = ws ? tuning_buffer(3, ws) : nullptr;
-        unsigned *counters = inline_reduce_ ? tuning_counters(conv_counter_count(p, l)) : nullptr;
+        const SplitKReduce counters = split_reduce(tuning_counters(conv_counter_count(p, l)));
         launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream);   // warm-up
         IOS_HIP(hipEventRecord(start, stream));
         for (int r = 0; r < reps; r++) launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream);
@@ -369,9 +433,10 @@ void DeviceContext::set_option(const std::string &key, const std::string &value)
         else if (value == "fp16") precision_ = PREC_FP16;
         else throw std::runtime_error("option precision: expected fp32, bf16 or fp16, got '" + value + "'");
     } else if (key == "split_k_reduce") {
-        if (value == "inline") inline_reduce_ = true;
-        else if (value == "kernel") inline_reduce_ = false;
-        else throw std::runtime_error("option split_k_reduce: expected inline or kernel, got '" + value + "'");
+        if (value == "xcd") reduce_mode_ = ReduceMode::Xcd;   // (falls back to inline where the placement probe failed)
+        else if (value == "inline") reduce_mode_ = ReduceMode::Inline;
+        else if (value == "kernel") reduce_mode_ = ReduceMode::Kernel;
+        else throw std::runtime_error("option split_k_reduce: expected xcd, inline or kernel, got '" + value + "'");
     } else if (key == "clear_tuning") {
         tuned.clear();
     } else {
@@ -383,7 +448,8 @@ std::string DeviceContext::info_json() const {
     std::ostringstream os;
     os << "{\"name\":\"" << name_ << "\",\"arch\":\"" << arch_ << "\",\"compute_units\":" << num_cus_
        << ",\"executor\":\"" << (exec_mode_ == ExecMode::Graph ? "graph" : exec_mode_ == ExecMode::Fused ? "fused" : exec_mode_ == ExecMode::FusedGraph ? "fused_graph" : "streams") << "\",\"autotune\":" << (autotune_ ? "true" : "false")
-       << ",\"split_k_reduce\":\"" << (inline_reduce_ ? "inline" : "kernel") << "\""
+       << ",\"split_k_reduce\":\"" << (reduce_mode_ == ReduceMode::Xcd ? "xcd" : reduce_mode_ == ReduceMode::Inline ? "inline" : "kernel") << "\""
+       << ",\"xcd_placement_probe\":" << (xcd_usable_ ? "true" : "false") << ",\"xcd_map\":" << xcd_map_[0]
        << ",\"precision\":\"" << (precision_ == PREC_BF16 ? "bf16" : precision_ == PREC_FP16 ? "fp16" : "fp32") << "\""
        << ",\"conv_variant\":" << forced_variant_ << ",\"conv_split_k\":" << forced_split_k_
        << ",\"arena_reuse\":" << (planner_arena_reuse() ? "true" : "false")
@@ -541,13 +607,15 @@ unsigned *Session::counters_of(const PlanConv &c) const {
     return reinterpret_cast<unsigned *>(base_ + c.ctr_off);
 }
 
-void Session::launch_op(const PlanOp &op, hipStream_t stream) {
+void Session::launch_op(const PlanOp &op, int group) {
+    hipStream_t stream = ctx_.stream(group);
     switch (op.kind) {
         case OpKind::ConvMfma: {
             const PlanConv &c = plan_.convs[op.conv];
             const TensorView residual = op.has_residual ? tv(op.residual) : TensorView{};
             launch_conv_mfma(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off, tv(op.out),
-                             c.ws_floats ? base_ + c.ws_off : nullptr, counters_of(c), stream, op.has_residual ? &residual : nullptr,
+                             c.ws_floats ? base_ + c.ws_off : nullptr, ctx_.split_reduce(counters_of(c), group, !capturing_forks_), stream,
+                             op.has_residual ? &residual : nullptr,
                              op.post_relu != 0);
             break;
         }
@@ -590,7 +658,7 @@ void Session::enqueue_streams(bool stage_events) {
             for (size_t g = 1; g < groups.size(); g++) IOS_HIP(hipStreamWaitEvent(ctx_.stream((int)g), fork_events_[s], 0));
         }
         for (size_t g = 0; g < groups.size(); g++)
-            for (int op : groups[g]) launch_op(plan_.ops[op], ctx_.stream((int)g));
+            for (int op : groups[g]) launch_op(plan_.ops[op], (int)g);
         if (fork) {
             for (size_t g = 1; g < groups.size(); g++) {
                 IOS_HIP(hipEventRecord(join_events_[s][g - 1], ctx_.stream((int)g)));
@@ -605,7 +673,7 @@ void Session::enqueue_serial() {
     hipStream_t main = ctx_.stream(0);
     for (const auto &groups : plan_.stages)
         for (const auto &group : groups)
-            for (int op : group) launch_op(plan_.ops[op], main);
+            for (int op : group) launch_op(plan_.ops[op], 0);
 }
 
 void Session::enqueue(bool stage_events) {
@@ -677,7 +745,7 @@ void Session::build_fused() {
                         const PlanConv &c = plan_.convs[op.conv];
                         const TensorView residual = op.has_residual ? tv(op.residual) : TensorView{};
                         const ConvDispatch d = make_conv_dispatch(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off,
-                                                                  tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr, counters_of(c),
+                                                                  tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr, ctx_.split_reduce(counters_of(c)),
                                                                   op.has_residual ? &residual : nullptr, op.post_relu != 0);
                         pend.fusable = conv_variant(d.variant).fusable() && !op.has_residual;   // (the fused kernel holds the plain epilogue)
                         if (!pend.fusable && !solo)
@@ -690,7 +758,7 @@ void Session::build_fused() {
                         pend.item.groups = d.groups;
                         pend.item.div_tiles = make_fast_div((unsigned)d.tiles);
                         pend.item.div_groups = make_fast_div((unsigned)d.groups);
-                        pend.item.num_blocks = d.tiles * d.groups * d.slices;
+                        pend.item.num_blocks = d.grid_blocks();
                         pend.item.conv = d.args;
                         pend.threads = d.threads;
                         pend.smem_bytes = d.smem_bytes;
@@ -811,10 +879,10 @@ void Session::enqueue_fused(bool stage_events) {
     for (size_t s = 0; s < plan_.stages.size(); s++) {
         if (fused_stages_[s].empty()) {
             for (const auto &group : plan_.stages[s])
-                for (int op : group) launch_op(plan_.ops[op], main);
+                for (int op : group) launch_op(plan_.ops[op], 0);
         } else {
             for (const FusedLaunch &l : fused_stages_[s]) {
-                if (l.single_op >= 0) launch_op(plan_.ops[l.single_op], main);
+                if (l.single_op >= 0) launch_op(plan_.ops[l.single_op], 0);
                 else launch_fused(l.threads, items + l.first_item, fused_items_host_.data() + l.first_item, l.header, l.total_blocks, l.smem_bytes, ctx_.num_cus(), main);
             }
         }
@@ -825,9 +893,13 @@ void Session::enqueue_fused(bool stage_events) {
 void Session::build_graph() {
     hipStream_t main = ctx_.stream(0);
     IOS_HIP(hipStreamBeginCapture(main, hipStreamCaptureModeRelaxed));
+    // the stream executor forks inside the capture, and the replay runs the branches on streams of its own choice
+    capturing_forks_ = ctx_.exec_mode() == ExecMode::Graph;
     try {
         enqueue(false);
+        capturing_forks_ = false;
     } catch (...) {
+        capturing_forks_ = false;
         hipGraph_t broken = nullptr;
         (void)hipStreamEndCapture(main, &broken);
         if (broken != nullptr) (void)hipGraphDestroy(broken);
@@ -866,7 +938,10 @@ void Session::run() {
     synchronize();
 }
 
-void Session::synchronize() { IOS_HIP(hipStreamSynchronize(ctx_.stream(0))); }
+void Session::synchronize() {
+    IOS_HIP(hipStreamSynchronize(ctx_.stream(0)));
+    ctx_.check_xcd_fault();
+}
 
 void Session::measure(int warmup, int number, int repeat, bool profile_stage, float *results, float *stage_results) {
     if (static_) throw std::runtime_error("a session in the static scratch has no timers");
@@ -908,6 +983,7 @@ void Session::measure(int warmup, int number, int repeat, bool profile_stage, fl
             for (size_t s = 0; s < num_stages; s++) stage_results[i * num_stages + s] = (float)(per_stage[s] / number);
     }
     IOS_HIP(hipDeviceSynchronize());
+    ctx_.check_xcd_fault();
 }
 
 void Session::measure_back_to_back(int warmup, int number, int repeat, float *results) {
@@ -926,6 +1002,7 @@ void Session::measure_back_to_back(int warmup, int number, int repeat, float *re
         results[i] = ms / (float)number;
     }
     IOS_HIP(hipDeviceSynchronize());
+    ctx_.check_xcd_fault();
 }
 
 void Session::profile_ops(int warmup, int repeat, float *ms_out) {
@@ -935,10 +1012,10 @@ void Session::profile_ops(int warmup, int repeat, float *ms_out) {
     run();   // every operator sees the inputs it has in a real pass
     for (size_t i = 0; i < plan_.ops.size(); i++) {
         const PlanOp &op = plan_.ops[i];
-        for (int w = 0; w < warmup; w++) launch_op(op, main);
+        for (int w = 0; w < warmup; w++) launch_op(op, 0);
         IOS_HIP(hipStreamSynchronize(main));
         IOS_HIP(hipEventRecord(start_, main));
-        for (int r = 0; r < repeat; r++) launch_op(op, main);
+        for (int r = 0; r < repeat; r++) launch_op(op, 0);
         IOS_HIP(hipEventRecord(stop_, main));
         IOS_HIP(hipEventSynchronize(stop_));
         float ms = 0.f;
@@ -1041,7 +1118,7 @@ void Session::profile_launches(int warmup, int repeat, float *ms_out, int capaci
                 const FusedLaunch &l = fused_stages_[r.stage][r.fused_level];
                 launch_fused(l.threads, items + l.first_item, fused_items_host_.data() + l.first_item, l.header, l.total_blocks, l.smem_bytes, ctx_.num_cus(), main);
             } else {
-                launch_op(plan_.ops[r.ops[0]], main);
+                launch_op(plan_.ops[r.ops[0]], 0);
             }
         };
         for (int w = 0; w < warmup; w++) issue();

@@ -38,7 +38,7 @@ def default_options():
     rt.set_option('conv_split_k', 0)
     rt.set_option('executor', 'streams')
     rt.set_option('autotune', 0)            # closed-form kernel configurations keep the suite short and repeatable
-    rt.set_option('split_k_reduce', 'inline')
+    rt.set_option('split_k_reduce', 'xcd')   # the library's default: K slices of a tile meet inside one XCD
     rt.set_option('precision', 'fp32')
     rt.set_option('arena_reuse', 1)
     rt.set_option('thin_conv_min_pixels', 1 << 18)
@@ -50,7 +50,7 @@ def default_options():
     rt.set_option('conv_variant', -1)
     rt.set_option('conv_split_k', 0)
     rt.set_option('executor', 'streams')
-    rt.set_option('split_k_reduce', 'inline')
+    rt.set_option('split_k_reduce', 'xcd')
 
 
 def single_op_graph(in_shape, build):
@@ -179,7 +179,7 @@ def test_residual_epilogue_of_every_conv_kernel_variant(variant_name, split_k):
         assert [op['kind'] for op in ops] == ['conv_mfma', 'conv_mfma'] and ops[1]['residual'] and ops[1]['post_relu'] == int(relu)
         x = np.random.default_rng(3).standard_normal((batch, *in_shape)).astype(np.float32)
         want = ios_oracle.run(graph, x)
-        for reduce in ('inline', 'kernel'):
+        for reduce in ('xcd', 'inline', 'kernel'):       # (a residual convolution under 'xcd' takes the device-wide form)
             rt.set_option('split_k_reduce', reduce)
             got = rt.graph_inference(graph, batch, x)
             assert_close(got, want, f'variant {variant_name} split {split_k} ({reduce}) residual unit {in_shape}->{oc} {k}')
@@ -236,8 +236,11 @@ def test_first_layer_configurations_on_three_and_five_channel_inputs(variant_nam
                                           'm32n16k64_w2x1x2_t16', 'm128n64k16_w2x2x1_t32', 'ws_m32n16_w8_t16',
                                           'wq_m16n16_w16_t16', 'wq_m32n32_w16_t16', 'ws_m32n32_w16_t32'])
 def test_split_k_reduction_inside_the_kernel_equals_the_reduction_kernel(variant_name):
-    """Both forms add the same partial tiles in slice order, so they must agree bit for bit, launch after launch."""
-    names = rt.device_info()['conv_variants']
+    """All three forms (second kernel, last block with the slices anywhere on the device, last block with the slices of a tile
+    on one XCD) add the same partial tiles in slice order, so they must agree bit for bit, launch after launch."""
+    info = rt.device_info()
+    assert info['xcd_placement_probe'], 'blocks with equal index % 8 did not share an XCC: the XCD-local form is not exercised'
+    names = info['conv_variants']
     rt.set_option('conv_variant', names.index(variant_name))
     for in_shape, oc, k, p, batch, split in [((200, 8, 8), 136, (1, 1), (0, 0), 1, 6), ((72, 19, 19), 88, (3, 3), (1, 1), 2, 3),
                                              ((96, 17, 17), 40, (1, 7), (0, 3), 1, 4)]:
@@ -246,7 +249,7 @@ def test_split_k_reduction_inside_the_kernel_equals_the_reduction_kernel(variant
         x = np.random.default_rng(5).standard_normal((batch, *in_shape)).astype(np.float32)
         want = ios_oracle.run(graph, x)
         results = {}
-        for form in ('kernel', 'inline'):
+        for form in ('kernel', 'inline', 'xcd'):
             rt.set_option('split_k_reduce', form)
             with rt.Session(graph, batch) as session:
                 session.load_weights()
@@ -260,6 +263,7 @@ def test_split_k_reduction_inside_the_kernel_equals_the_reduction_kernel(variant
                 results[form] = outs[0]
         assert_close(results['inline'], want, f'{variant_name} split {split} {in_shape}')
         np.testing.assert_array_equal(results['inline'], results['kernel'])
+        np.testing.assert_array_equal(results['xcd'], results['kernel'])
 
 
 def test_split_k_is_repeatable_in_a_session():

@@ -271,6 +271,39 @@ def test_arena_reuse_never_lets_an_operator_read_what_another_overwrote(name, ba
             assert all(e <= begin or stop <= b for b, e in first_reads), op['node']
 
 
+@pytest.mark.parametrize('tiles,split', [(1, 2), (5, 3), (8, 4), (9, 2), (48, 4), (190, 2), (231, 5), (1000, 16), (7, 64)])
+def test_xcd_local_split_k_numbering(tiles, split):
+    """The grid of a split-K convolution whose slices meet inside one XCD: every (tile, slice) exactly once, all slices of a
+    tile on blocks with the same index modulo 8 (the dispatcher deals workgroups to the 8 XCDs round-robin), every residue
+    class owning a contiguous range of tiles of nearly equal length, idle blocks only where a class has one tile less."""
+    lib = rt.get_lib()
+    blocks = lib.ios_xcd_numbering(tiles, split, None, None, 0)
+    assert blocks == 8 * ((tiles + 7) // 8) * split
+    tile = (ctypes.c_int * blocks)()
+    piece = (ctypes.c_int * blocks)()
+    assert lib.ios_xcd_numbering(tiles, split, tile, piece, blocks) == blocks
+    seen = {}
+    for block in range(blocks):
+        if tile[block] < 0:
+            continue
+        assert 0 <= tile[block] < tiles and 0 <= piece[block] < split
+        assert (tile[block], piece[block]) not in seen
+        seen[(tile[block], piece[block])] = block
+    assert len(seen) == tiles * split
+    per_class = {}
+    for (t, _), block in seen.items():
+        per_class.setdefault(block % 8, set()).add(t)
+    for t in range(tiles):
+        assert len({seen[(t, z)] % 8 for z in range(split)}) == 1       # one XCD per tile
+        order = [seen[(t, z)] for z in range(split)]
+        assert order == sorted(order) and order[-1] - order[0] == 8 * (split - 1)   # dispatched together, slice 0 first
+    sizes = [len(per_class.get(c, ())) for c in range(8)]
+    assert max(sizes) - min(sizes) <= 1 and sum(sizes) == tiles
+    for c, owned in per_class.items():
+        assert sorted(owned) == list(range(min(owned), max(owned) + 1))  # contiguous: an XCD's L2 sees neighbouring tiles
+    assert blocks - len(seen) == (8 * ((tiles + 7) // 8) - tiles) * split
+
+
 def test_split_k_partial_tiles_share_the_arena_like_any_other_region():
     # every convolution forced to four K slices: their partial tiles are regions with a lifetime of one stage, so they share
     # addresses with tensors that are dead by then, and must never land on one that a later operation still reads

@@ -25,7 +25,7 @@ def closed_form_configurations():
     rt.set_option('autotune', 0)
     rt.set_option('executor', 'fused')
     rt.set_option('precision', 'fp32')
-    rt.set_option('split_k_reduce', 'inline')
+    rt.set_option('split_k_reduce', 'xcd')
     yield
     for key in OPTIONS:
         value = before[key]
@@ -80,7 +80,7 @@ def test_split_k_tickets_and_partial_tiles_live_in_the_static_array():
     graph.init_weights(seed=5, scheme='he_normal_bias')
     graph.sequential_schedule()
     rt.set_option('conv_split_k', 4)
-    for form in ('inline', 'kernel'):
+    for form in ('xcd', 'inline', 'kernel'):
         rt.set_option('split_k_reduce', form)
         for batch in (3, 1, 2, 1):                     # shrinking and growing: tickets must be back at zero every time
             x, got = both(graph, batch, seed=batch)
