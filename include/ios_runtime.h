@@ -81,6 +81,10 @@ int graph_inference_no_alloc(const char *graph_json, int batch_size, float *inpu
  * slices of a tile have such indices. */
 int ios_xcd_numbering(int tiles, int split, int *tile_of_block, int *slice_of_block, int capacity);
 
+/* The three bfloat16 terms into which the "x3_*" convolution kernels split an fp32 operand, each as the upper half of a
+ * 32-bit word (host only, for tests): terms[0] + terms[1] + terms[2], read as floats, equal x exactly for every normal x. */
+void ios_split_bf16x3(float x, unsigned *terms);
+
 /* Free device memory in bytes as hipMemGetInfo reports it (creates the device context if there is none yet), or -1. */
 long long ios_device_free_bytes(void);
 

@@ -170,6 +170,10 @@ int ios_xcd_numbering(int tiles, int split, int *tile_of_block, int *slice_of_bl
     return blocks;
 }
 
+void ios_split_bf16x3(float x, unsigned *terms) {
+    if (terms != nullptr) ios::split3(x, terms[0], terms[1], terms[2]);
+}
+
 int ios_conv_variant_names(char *buf, int cap) {
     std::string text = "[";
     for (int i = 0; i < ios::conv_num_variants(); i++) text += std::string(i ? "," : "") + '"' + ios::conv_variant(i).name + '"';

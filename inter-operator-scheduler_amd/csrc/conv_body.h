@@ -253,6 +253,110 @@ struct Mfma<16> {
     __device__ static __forceinline__ int row(int v, int lane) { return 4 * (lane >> 4) + v; }
 };
 
+// Tail of the LDS-tiled kernels once a block holds its accumulators (wavefronts with wk == 0; the others only take part in the
+// barriers): the split-K exchange in its three forms, then bias, activation and the store through the output view.
+template <int MT, int BM, int BN, int TM, int TN, int WM, int WN, bool RES>
+__device__ __forceinline__ void tiled_tail(const ConvKernelArgs &a, float *smem, typename Mfma<MT>::acc_t (&acc)[TM][TN], int tile, int g, int z,
+                                           int m0, int n0, int wm, int wn, int wk) {
+    using M = Mfma<MT>;
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int lc = lane % MT;
+    // ---- split-K ----------------------------------------------------------------------------------------------
+    if (a.split_k > 1) {
+        if (a.counters == nullptr) {
+            // two-kernel form: store this slice's partial tile; splitk_reduce_kernel adds the slices, bias and activation
+            float *wsz = a.ws + ((size_t)z * a.groups + g) * a.OCg * (size_t)a.Npix;
+            if (wk == 0) {
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const int nn = n0 + wn * WTN + j * MT + lc;
+                    if (nn >= a.Npix) continue;
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int v = 0; v < M::ACC; v++) {
+                            const int m = m0 + wm * WTM + i * MT + M::row(v, lane);
+                            if (m < a.OCg) wsz[(size_t)m * a.Npix + nn] = acc[i][j][v];
+                        }
+                }
+            }
+            return;
+        }
+        // one-kernel form: every slice stores its partial tile in accumulator layout ([element][thread], so a
+        // wavefront writes 256 contiguous bytes), then takes a ticket on the tile's counter; the block that
+        // draws the last ticket adds all slices in slice order (its own included, so the sum does not depend
+        // on which block came last) and runs the epilogue.  Partials and tickets move with device-scope
+        // atomics, which are coherent across the per-XCD L2s without cache-wide write-backs or invalidations;
+        // the wait on the outstanding stores before the barrier orders a block's partials before its ticket.
+        constexpr int T0 = 64 * WM * WN;
+        constexpr int E = TM * TN * M::ACC;
+        static_assert(T0 * E == BM * BN, "accumulator layout covers the tile");
+        const size_t tiles = (size_t)xcd_padded_tiles(a.tiles_m * a.tiles_n);   // (both forms size their arrays for the padded count)
+        float *slices = a.ws + (((size_t)g * tiles + tile) * a.split_k) * (size_t)(BM * BN);
+        unsigned *counter = a.counters + (size_t)g * tiles + tile;
+        int *last_flag = reinterpret_cast<int *>(smem);
+        auto exchange = [&](auto local) -> bool {   // true: this block drew the last ticket and holds the sum of all slices
+            constexpr bool LOCAL = decltype(local)::value;
+            if (wk == 0) {
+                float *mine = slices + (size_t)z * (BM * BN) + tid;
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+#pragma unroll
+                        for (int v = 0; v < M::ACC; v++) partial_store<LOCAL>(mine + ((i * TN + j) * M::ACC + v) * T0, acc[i][j][v]);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (tid == 0) *last_flag = draw_ticket<LOCAL>(counter, a.split_k);
+            __syncthreads();
+            if (*last_flag == 0) return false;
+            if (wk == 0) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+#pragma unroll
+                        for (int v = 0; v < M::ACC; v++) acc[i][j][v] = 0.f;
+                for (int s = 0; s < a.split_k; s++) {
+                    const float *theirs = slices + (size_t)s * (BM * BN) + tid;
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++)
+#pragma unroll
+                            for (int v = 0; v < M::ACC; v++) acc[i][j][v] += partial_load<LOCAL>(theirs + ((i * TN + j) * M::ACC + v) * T0);
+                }
+            }
+            return true;
+        };
+        const bool last = a.xcd_local ? exchange(std::true_type{}) : exchange(std::false_type{});
+        if (!last) return;
+    }
+
+    // ---- epilogue -------------------------------------------------------------------------------------------
+    if (wk == 0) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int nn = n0 + wn * WTN + j * MT + lc;
+            if (nn >= a.Npix) continue;
+            const int b = (int)fast_div((unsigned)nn, a.div_ohw);
+            const int r = nn - b * a.OHW;
+            float *yb = a.y + (long long)b * a.y_bs + (long long)g * a.OCg * a.OHW + r;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int v = 0; v < M::ACC; v++) {
+                    const int m = m0 + wm * WTM + i * MT + M::row(v, lane);
+                    if (m < a.OCg)
+                        yb[(long long)m * a.OHW] = add_residual<RES>(a, apply_act(acc[i][j][v] + a.bias[g * a.OCg + m], a.act), b, g * a.OCg + m, r);
+                }
+        }
+    }
+}
+
 template <int BM, int BN, int BK, int WM, int WN, int WK, int MT, int PD>
 struct ConvTiled {
     using M = Mfma<MT>;
@@ -458,98 +562,224 @@ struct ConvTiled {
         }
     }
 
-    // ---- split-K ----------------------------------------------------------------------------------------------
-    if (a.split_k > 1) {
-        if (a.counters == nullptr) {
-            // two-kernel form: store this slice's partial tile; splitk_reduce_kernel adds the slices, bias and activation
-            float *wsz = a.ws + ((size_t)z * a.groups + g) * a.OCg * (size_t)a.Npix;
-            if (wk == 0) {
-#pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const int nn = n0 + wn * WTN + j * MT + lc;
-                    if (nn >= a.Npix) continue;
-#pragma unroll
-                    for (int i = 0; i < TM; i++)
-#pragma unroll
-                        for (int v = 0; v < M::ACC; v++) {
-                            const int m = m0 + wm * WTM + i * MT + M::row(v, lane);
-                            if (m < a.OCg) wsz[(size_t)m * a.Npix + nn] = acc[i][j][v];
-                        }
-                }
-            }
-            return;
-        }
-        // one-kernel form: every slice stores its partial tile in accumulator layout ([element][thread], so a
-        // wavefront writes 256 contiguous bytes), then takes a ticket on the tile's counter; the block that
-        // draws the last ticket adds all slices in slice order (its own included, so the sum does not depend
-        // on which block came last) and runs the epilogue.  Partials and tickets move with device-scope
-        // atomics, which are coherent across the per-XCD L2s without cache-wide write-backs or invalidations;
-        // the wait on the outstanding stores before the barrier orders a block's partials before its ticket.
-        constexpr int T0 = 64 * WM * WN;
-        constexpr int E = TM * TN * M::ACC;
-        static_assert(T0 * E == BM * BN, "accumulator layout covers the tile");
-        const size_t tiles = (size_t)xcd_padded_tiles(a.tiles_m * a.tiles_n);   // (both forms size their arrays for the padded count)
-        float *slices = a.ws + (((size_t)g * tiles + tile) * a.split_k) * (size_t)(BM * BN);
-        unsigned *counter = a.counters + (size_t)g * tiles + tile;
-        int *last_flag = reinterpret_cast<int *>(smem);
-        auto exchange = [&](auto local) -> bool {   // true: this block drew the last ticket and holds the sum of all slices
-            constexpr bool LOCAL = decltype(local)::value;
-            if (wk == 0) {
-                float *mine = slices + (size_t)z * (BM * BN) + tid;
-#pragma unroll
-                for (int i = 0; i < TM; i++)
-#pragma unroll
-                    for (int j = 0; j < TN; j++)
-#pragma unroll
-                        for (int v = 0; v < M::ACC; v++) partial_store<LOCAL>(mine + ((i * TN + j) * M::ACC + v) * T0, acc[i][j][v]);
-            }
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
-            if (tid == 0) *last_flag = draw_ticket<LOCAL>(counter, a.split_k);
-            __syncthreads();
-            if (*last_flag == 0) return false;
-            if (wk == 0) {
-#pragma unroll
-                for (int i = 0; i < TM; i++)
-#pragma unroll
-                    for (int j = 0; j < TN; j++)
-#pragma unroll
-                        for (int v = 0; v < M::ACC; v++) acc[i][j][v] = 0.f;
-                for (int s = 0; s < a.split_k; s++) {
-                    const float *theirs = slices + (size_t)s * (BM * BN) + tid;
-#pragma unroll
-                    for (int i = 0; i < TM; i++)
-#pragma unroll
-                        for (int j = 0; j < TN; j++)
-#pragma unroll
-                            for (int v = 0; v < M::ACC; v++) acc[i][j][v] += partial_load<LOCAL>(theirs + ((i * TN + j) * M::ACC + v) * T0);
-                }
-            }
-            return true;
-        };
-        const bool last = a.xcd_local ? exchange(std::true_type{}) : exchange(std::false_type{});
-        if (!last) return;
-    }
+    tiled_tail<MT, BM, BN, TM, TN, WM, WN, RES>(a, smem, acc, tile, g, z, m0, n0, wm, wn, wk);
+    }   // run
+};
 
-    // ---- epilogue -------------------------------------------------------------------------------------------
-    if (wk == 0) {
+// ---- LDS-tiled kernel on the bfloat16 matrix pipe with fp32-exact operands ---------------------------------------------------
+// The fp32 matrix instructions run at 1/16 of the rate of the bfloat16 ones (measured: 149-156 against 2340 TFLOP/s).  An fp32
+// number is exactly the sum of three bfloat16 numbers (its 24 significant bits in three groups of eight: x = hi + mid + lo,
+// each term obtained by truncating the remainder to its leading eight bits, all subtractions exact), so a product of two
+// fp32 numbers is the sum of nine products of bfloat16 numbers, each exact in fp32.  This kernel adds the six largest of them
+// (hi*hi, hi*mid, mid*hi, hi*lo, mid*mid, lo*hi) on v_mfma_f32_32x32x16_bf16 with fp32 accumulation; the three that are left
+// out are below 2^-23 of the product, the size of the rounding error of an fp32 multiplication.  Six instructions of 8 passes
+// cover 16 k where the fp32 form needs eight instructions of 16 passes: 2.7 times the matrix throughput at fp32 accuracy.
+//
+// Filters are split when they are packed: three planes of bfloat16 in octets of eight consecutive k, [k / 8][plane][m][8],
+// which is the operand layout of the instruction (lane l: row l % 32, k = 8 * (l / 32) ... + 7): a wavefront reads the filter
+// operand of a 32 x 32 tile straight from global memory, one 16-byte load per lane and plane, PD K tiles ahead (the filters
+// are small and stay in the caches; the LDS, whose bandwidth bounds this kernel, carries the inputs only).  Inputs are split
+// by the thread that stages them: eight channels of one pixel, loaded PD K tiles ahead into registers, three 16-byte LDS
+// stores into [plane][octet][pixel][8 k], again the operand layout: an input operand is one conflict-free 16-byte LDS load
+// per lane and plane.  K tiles are 16 deep and lie inside one filter tap (channels padded to 16); LDS is double buffered, one
+// barrier per K tile.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// the three bfloat16 terms of an fp32 value, each in the upper half of a word (hi + mid + lo == x exactly for normal x)
+__device__ __host__ inline void split3(float x, unsigned &hi, unsigned &mid, unsigned &lo) {
+    union { float f; unsigned u; } v, r;
+    v.f = x;
+    hi = v.u & 0xffff0000u;
+    r.u = hi;
+    v.f = x - r.f;
+    mid = v.u & 0xffff0000u;
+    r.u = mid;
+    v.f = v.f - r.f;
+    lo = v.u & 0xffff0000u;
+}
+
+// three bfloat16 terms of eight fp32 values, each term as four words of two bfloat16 (lower k in the lower half)
+__device__ __forceinline__ void split_bf16x3(const float (&x)[8], uintx4 &hi, uintx4 &mid, uintx4 &lo) {
+    unsigned h[8], m[8], l[8];
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int nn = n0 + wn * WTN + j * MT + lc;
-            if (nn >= a.Npix) continue;
-            const int b = (int)fast_div((unsigned)nn, a.div_ohw);
-            const int r = nn - b * a.OHW;
-            float *yb = a.y + (long long)b * a.y_bs + (long long)g * a.OCg * a.OHW + r;
+    for (int i = 0; i < 8; i++) {
+        h[i] = __float_as_uint(x[i]) & 0xffff0000u;
+        const float r1 = x[i] - __uint_as_float(h[i]);
+        m[i] = __float_as_uint(r1) & 0xffff0000u;
+        const float r2 = r1 - __uint_as_float(m[i]);
+        l[i] = __float_as_uint(r2);
+    }
 #pragma unroll
-            for (int i = 0; i < TM; i++)
+    for (int i = 0; i < 4; i++) {   // high halves of two words side by side
+        hi[i] = __builtin_amdgcn_perm(h[2 * i + 1], h[2 * i], 0x07060302u);
+        mid[i] = __builtin_amdgcn_perm(m[2 * i + 1], m[2 * i], 0x07060302u);
+        lo[i] = __builtin_amdgcn_perm(l[2 * i + 1], l[2 * i], 0x07060302u);
+    }
+}
+
+// TMW x TNW MFMA tiles of 32 x 32 per wavefront, WM x WN wavefronts per block
+template <int TMW, int TNW, int WM, int WN, int PD>
+struct ConvSplit3 {
+    static constexpr int MT = 32, BK = 16;
+    using M = Mfma<32>;
+    static constexpr int BM = 32 * TMW * WM, BN = 32 * TNW * WN;
+    static constexpr int WAVES = WM * WN;
+    static constexpr int T = 64 * WAVES;
+    static constexpr int THREADS = T;
+    static constexpr int CPAD = BK;
+    static constexpr bool FUSABLE = false;
+    // LDS in slots of 16 bytes (eight bfloat16): per stage the input planes [3][2][BN]
+    static constexpr int STAGE = 6 * BN;
+    static constexpr int SMEM_FLOATS = 2 * STAGE * 4;
+    static constexpr int B_OCT = 2 * BN;
+    static constexpr int B_IT = (B_OCT + T - 1) / T;                   // octets a thread stages per K tile
+    static_assert(T % BN == 0, "a thread stages the same pixel in every pass");
+
+    template <bool RES = false>
+    __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *smem, int tile, int g, int z) {
+    constexpr int WTM = 32 * TMW, WTN = 32 * TNW;
+    constexpr int TM = TMW, TN = TNW;
+    uintx4 *lds = reinterpret_cast<uintx4 *>(smem);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave % WN;
+    const int wm = wave / WN;
+    const int lk = lane >> 5;   // which eight k of a K tile this lane supplies to the matrix instruction
+    const int lc = lane & 31;   // row (A) / column (B) of this lane inside an MFMA tile
+    int tm, tn;
+    xcd_tile(a, tile, tm, tn);
+    const int m0 = tm * BM;
+    const int n0 = tn * BN;
+    const int k_begin = z * a.k_chunk;
+    const int k_end = min(a.Kq, k_begin + a.k_chunk);
+    const int nkt = (k_end - k_begin) / BK;
+
+    // ---- filters: every wavefront reads the operands of its own tiles from global memory, in operand layout -------------
+    const __amdgpu_buffer_rsrc_t xr = buffer_of(a.x, a.x_bytes);
+    const __amdgpu_buffer_rsrc_t wr = buffer_of(a.wp, a.w_bytes);
+    unsigned a_off[TM];      // byte offset of this lane's slot (plane 0) inside a K tile of the packed filters, or out of range
 #pragma unroll
-                for (int v = 0; v < M::ACC; v++) {
-                    const int m = m0 + wm * WTM + i * MT + M::row(v, lane);
-                    if (m < a.OCg)
-                        yb[(long long)m * a.OHW] = add_residual<RES>(a, apply_act(acc[i][j][v] + a.bias[g * a.OCg + m], a.act), b, g * a.OCg + m, r);
-                }
+    for (int i = 0; i < TM; i++) {
+        const int m = m0 + wm * WTM + i * MT + lc;
+        // packed filters: [g][k / 8][plane][OCgP] slots of 16 bytes
+        a_off[i] = m < a.OCgP ? (unsigned)(((((size_t)g * (a.Kq >> 3) + lk) * 3) * a.OCgP + m) * 16) : kOutOfRange;
+    }
+    const unsigned a_plane = (unsigned)a.OCgP * 16u;
+    // ---- inputs: this thread's pixel and octets ----------------------------------------------------------------------------
+    const int pix = tid % BN;
+    const int n = n0 + pix;
+    const bool n_ok = n < a.Npix;
+    int ih0, iw0;
+    unsigned x_thread;
+    {
+        const int nn = n_ok ? n : 0;
+        const int b = (int)fast_div((unsigned)nn, a.div_ohw);
+        const int r = nn - b * a.OHW;
+        const int oh = (int)fast_div((unsigned)r, a.div_ow);
+        const int ow = r - oh * a.OW;
+        ih0 = oh * a.sh - a.ph;
+        iw0 = ow * a.sw - a.pw;
+        x_thread = (unsigned)(((long long)b * a.x_bs + (long long)g * a.ICg * a.HW + (long long)ih0 * a.W + iw0) * 4);
+    }
+    int b_oct[B_IT];       // which half of the K tile (channels 8 * b_oct ... + 7 of the tile) a pass of this thread stages
+#pragma unroll
+    for (int i = 0; i < B_IT; i++) b_oct[i] = (tid + i * T) / BN;
+    const unsigned b_surplus = B_OCT % T == 0 || tid < B_OCT ? 0u : kOutOfRange;   // (more threads than octets: the surplus stages nothing)
+
+    uintx4 a_reg[PD][3][TM];
+    float b_reg[PD][B_IT][8];
+    auto load_tile = [&](int kt, uintx4 (&ar)[3][TM], float (&br)[B_IT][8]) {
+        const int k0 = k_begin + kt * BK;
+        const int tap = (int)__umulhi((unsigned)k0, a.magic_icgp);
+        const int c0 = k0 - tap * a.ICgP;
+        const int kh = a.KW == 1 ? tap : (int)__umulhi((unsigned)tap, a.magic_kw);
+        const int kw = tap - kh * a.KW;
+        const unsigned tile_kill = kt < nkt ? 0u : kOutOfRange;   // tiles past the end of the K range load zeros
+        const unsigned w_tile = (unsigned)((k0 >> 3) * 3 * a.OCgP) * 16u;
+#pragma unroll
+        for (int p = 0; p < 3; p++)
+#pragma unroll
+            for (int i = 0; i < TM; i++) ar[p][i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (a_off[i] + w_tile) | tile_kill, (unsigned)p * a_plane, 0);
+        const unsigned in_h = (unsigned)(ih0 + kh) < (unsigned)a.H ? 1u : 0u;
+        const unsigned in_w = (unsigned)(iw0 + kw) < (unsigned)a.W ? 1u : 0u;
+        const unsigned kill = (((in_h & in_w & (n_ok ? 1u : 0u)) ^ 1u) << 31) | tile_kill | b_surplus;
+        const unsigned x_tile = x_thread + (unsigned)(c0 * a.HW + kh * a.W + kw) * 4u;
+        const unsigned plane = (unsigned)a.HW * 4u;
+#pragma unroll
+        for (int i = 0; i < B_IT; i++) {
+            const int c_left = a.ICg - 1 - c0 - b_oct[i] * 8;   // channels of this octet beyond c_left are padding
+            const unsigned at = (x_tile + (unsigned)(b_oct[i] * 8) * plane) | kill;
+            // (no branch around loads inside the loop: where paths that issued loads join, the compiler waits for all of them)
+#pragma unroll
+            for (int j = 0; j < 8; j++) br[i][j] = buffer_load_f32(xr, at | ((unsigned)(c_left - j) & kOutOfRange), (unsigned)j * plane);
+        }
+    };
+    const int relu_floor = a.pre_relu ? 0 : (int)0x80000000;
+    auto store_inputs = [&](int buf, const float (&br)[B_IT][8]) {
+        uintx4 *stage = lds + buf * STAGE;
+#pragma unroll
+        for (int i = 0; i < B_IT; i++) {
+            if (B_OCT % T != 0 && tid + i * T >= B_OCT) continue;
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = __int_as_float(max(__float_as_int(br[i][j]), relu_floor));   // folded ReLU of the producer
+            uintx4 hi, mid, lo;
+            split_bf16x3(v, hi, mid, lo);
+            stage[(0 + b_oct[i]) * BN + pix] = hi;
+            stage[(2 + b_oct[i]) * BN + pix] = mid;
+            stage[(4 + b_oct[i]) * BN + pix] = lo;
+        }
+    };
+
+    typename M::acc_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < M::ACC; v++) acc[i][j][v] = 0.f;
+
+    // ---- main loop ---------------------------------------------------------------------------------------------------------
+    // Register stage s holds K tile kt with kt % PD == s (filter operands of this wavefront, inputs of this thread).  Iteration
+    // kt: the matrix work of tile kt from registers (filters) and LDS stage kt & 1 (inputs), the stage's registers requested
+    // again for tile kt + PD, the inputs of tile kt + 1 split and stored into the other LDS stage, one barrier.
+#pragma unroll
+    for (int s = 0; s < PD; s++) load_tile(s, a_reg[s], b_reg[s]);
+    store_inputs(0, b_reg[0]);
+    __syncthreads();
+    for (int kt0 = 0; kt0 < nkt; kt0 += PD) {
+#pragma unroll
+        for (int s = 0; s < PD; s++) {
+            const int kt = kt0 + s;
+            const int buf = kt & 1;
+            const uintx4 *Bb = lds + buf * STAGE + lk * BN + wn * WTN + lc;
+            bf16x8 av[3][TM], bv[3][TN];
+#pragma unroll
+            for (int p = 0; p < 3; p++) {
+#pragma unroll
+                for (int i = 0; i < TM; i++) av[p][i] = __builtin_bit_cast(bf16x8, a_reg[s][p][i]);
+#pragma unroll
+                for (int j = 0; j < TN; j++) bv[p][j] = __builtin_bit_cast(bf16x8, Bb[p * 2 * BN + j * MT]);
+            }
+            // all LDS reads of the tile are requested before its first matrix instruction (left to itself the scheduler
+            // requests each operand right in front of its first use and the wavefront pays the LDS latency once per plane)
+            __builtin_amdgcn_sched_barrier(0);
+            // the six terms, smallest first; the tiles of a term are independent instructions
+            constexpr int TA[6] = {2, 0, 1, 1, 0, 0}, TB[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+            for (int t = 0; t < 6; t++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[TA[t]][i], bv[TB[t]][j], acc[i][j], 0, 0, 0);
+            store_inputs(buf ^ 1, b_reg[(s + 1) % PD]);
+            load_tile(kt + PD, a_reg[s], b_reg[s]);
+            __syncthreads();
         }
     }
+    tiled_tail<MT, BM, BN, TM, TN, WM, WN, RES>(a, smem, acc, tile, g, z, m0, n0, wm, wn, 0);
     }   // run
 };
 
@@ -1093,6 +1323,18 @@ struct ConvWsplit {
     X(86, "wq_m32n32_w1_t16_d4", 16, 2, 2, 1, 4, true, 4, 0)          \
     X(87, "wq_m64n32_w1_t16", 16, 4, 2, 1, 4, true, 2, 0)             \
     X(88, "wq_m64n64_w2_t32", 32, 2, 2, 2, 8, true, 2, 0)
-constexpr int kNumConvVariants = 89;
+// X(index, name, TMW, TNW, WM, WN, PD): the LDS-tiled kernel with operands split into three bfloat16 terms (ConvSplit3);
+// TMW x TNW tiles of 32 x 32 per wavefront, WM x WN wavefronts
+#define IOS_SPLIT3_VARIANTS(X)                     \
+    X(89, "x3_m64n128_w2x2", 1, 2, 2, 2, 2)        \
+    X(90, "x3_m64n128_w2x2_p3", 1, 2, 2, 2, 3)     \
+    X(91, "x3_m64n256_w2x4", 1, 2, 2, 4, 2)        \
+    X(92, "x3_m64n64_w2x2", 1, 1, 2, 2, 2)         \
+    X(93, "x3_m64n64_w1x1", 2, 2, 1, 1, 2)         \
+    X(94, "x3_m64n128_w1x2", 2, 2, 1, 2, 2)        \
+    X(95, "x3_m128n64_w4x1", 1, 2, 4, 1, 2)        \
+    X(96, "x3_m128n128_w4x2", 1, 2, 4, 2, 2)       \
+    X(97, "x3_m192n128_w6x2", 1, 2, 6, 2, 2)
+constexpr int kNumConvVariants = 98;
 
 }  // namespace ios

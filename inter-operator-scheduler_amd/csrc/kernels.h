@@ -53,7 +53,9 @@ struct ConvVariant {
     int threads() const { return 64 * WM * WN * WK; }
     bool fusable_;   // light enough on registers to run inside a fused stage launch
     int precision;   // PREC_FP32, or a reduced-precision mode: bfloat16 / IEEE half filters and inputs, fp32 accumulation
+    int koct = 0;    // 1: packed filters are three planes of bfloat16, [k / 8][plane][m][8] (the kernel that splits fp32 operands into three bfloat16 terms)
     bool fusable() const { return fusable_; }
+    int kvec() const { return koct ? 8 : kquad ? 4 : 1; }   // consecutive k of one output channel that lie together
 };
 
 int conv_num_variants();
@@ -80,7 +82,7 @@ bool conv_matrix_path_supported(const ConvProblem &p);
 ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only = false, int precision = PREC_FP32);
 
 // Filter packing for a kernel configuration: w[OC][ICg][KH][KW] -> packed[g][k = (kh*KW + kw)*ICgP + c][OCgP]
-// (or [g][k / 4][OCgP][k % 4] for kquad configurations), ICgP = ICg rounded up to the configuration's channel
+// (or [g][k / 4][OCgP][k % 4] for kquad configurations, three bfloat16 planes [g][k / 8][plane][OCgP][k % 8] for koct ones), ICgP = ICg rounded up to the configuration's channel
 // padding (zero rows), OCgP = OCg rounded up to 4.  16-bit configurations pack bfloat16 or half (round to nearest even), two
 // per float of the returned size.
 size_t conv_packed_floats(const ConvProblem &p, const ConvLaunch &l);

@@ -38,7 +38,14 @@ PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorV
     a.strip_rows = 0;
     a.vec_columns = 1;
     if (global) {
-        *blocks = blocks_for((long long)p.B * p.C, 4, 4096);
+        // from 2^14 planes on (a lane per plane still gives every compute unit a wavefront) the row form, else a wavefront per plane
+        const long long planes = (long long)p.B * p.C;
+        if (planes >= (1LL << 14) && p.H * p.W <= 1024) {
+            a.strip_rows = 1;
+            *blocks = blocks_for(planes, 256, 4096);
+        } else {
+            *blocks = blocks_for(planes, 4, 4096);
+        }
     } else if (p.KH == 3 && p.KW == 3 && (p.sh == 1 || p.sh == 2)) {
         // one thread per strip of output rows; the longest strip that still leaves a million threads
         int rows = kPoolStripRows;

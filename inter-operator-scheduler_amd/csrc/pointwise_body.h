@@ -227,8 +227,42 @@ __device__ __forceinline__ void pool_body(const PoolArgs &a, int block, int num_
     }
 }
 
+// window == whole map, many planes (strip_rows == 1): one lane reduces one (image, channel) plane with 16-byte loads, four
+// independent partial results, no cross-lane step; the 64 planes of a wavefront are 64 consecutive rows of H * W floats, so
+// every cache line a load touches is used up by the loads that follow, and the 64 results leave as one coalesced store.
+// (One wavefront per plane, below, spends a 64-lane load and a six-step cross-lane reduction on 256 bytes.)
+__device__ __forceinline__ void global_pool_rows_body(const PoolArgs &a, int block, int num_blocks, unsigned threads) {
+    const PoolProblem &p = a.p;
+    const unsigned planes = (unsigned)(p.B * p.C);
+    const int HW = p.H * p.W;
+    const bool is_max = p.is_max != 0;
+    for (unsigned plane = block * threads + threadIdx.x; plane < planes; plane += num_blocks * threads) {
+        const unsigned b = plane / (unsigned)p.C, c = plane - b * (unsigned)p.C;
+        const float *xc = a.x + (long long)b * a.x_bs + (long long)c * HW;
+        float best[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, sum[4] = {0.f, 0.f, 0.f, 0.f};
+        int i = 0;
+#pragma unroll 4
+        for (; i + 4 <= HW; i += 4) {
+            const pw_floatx4_u q = *reinterpret_cast<const pw_floatx4_u *>(xc + i);
+            best[0] = fmaxf(best[0], q.x); best[1] = fmaxf(best[1], q.y); best[2] = fmaxf(best[2], q.z); best[3] = fmaxf(best[3], q.w);
+            sum[0] += q.x; sum[1] += q.y; sum[2] += q.z; sum[3] += q.w;
+        }
+        for (; i < HW; i++) {
+            best[0] = fmaxf(best[0], xc[i]);
+            sum[0] += xc[i];
+        }
+        const float m = fmaxf(fmaxf(best[0], best[1]), fmaxf(best[2], best[3]));
+        const float t = (sum[0] + sum[1]) + (sum[2] + sum[3]);
+        a.y[(long long)b * a.y_bs + c] = is_max ? m : t / (float)HW;
+    }
+}
+
 // window == whole map: one wavefront reduces one (image, channel) plane
 __device__ __forceinline__ void global_pool_body(const PoolArgs &a, int block, int num_blocks, unsigned threads) {
+    if (a.strip_rows == 1) {
+        global_pool_rows_body(a, block, num_blocks, threads);
+        return;
+    }
     const PoolProblem &p = a.p;
     const int planes = p.B * p.C;
     const int HW = p.H * p.W;

@@ -266,6 +266,30 @@ def test_split_k_reduction_inside_the_kernel_equals_the_reduction_kernel(variant
         np.testing.assert_array_equal(results['xcd'], results['kernel'])
 
 
+def test_bfloat16_split_kernels_are_as_accurate_as_the_fp32_matrix_instructions():
+    """The x3_* configurations compute fp32 products as six bfloat16 products of exactly split operands: against a float64
+    reference their error must be of the size of the fp32 kernels' own (not of bfloat16's), on a long K."""
+    import torch
+    names = rt.device_info()['conv_variants']
+    in_shape, oc, batch = (256, 17, 17), 96, 2
+    graph = single_op_graph(in_shape, lambda b, v: ios.conv2d(b, [[v]], oc, (3, 3), (1, 1), (1, 1), 1, 'identity', is_exit=True))
+    x = np.random.default_rng(11).standard_normal((batch, *in_shape)).astype(np.float32)
+    conv = list(graph.conv_nodes())[0]
+    want = torch.nn.functional.conv2d(torch.from_numpy(x).double(), torch.from_numpy(conv.weight).double(),
+                                      torch.from_numpy(conv.bias).double(), padding=1).numpy()
+    scale = np.abs(want).max()
+    errors = {}
+    for name in ('wq_m32n16_w8_t16', 'm64n64k32_w2x2x1_t32', 'x3_m64n128_w2x2', 'x3_m64n64_w1x1', 'x3_m128n64_w4x1'):
+        rt.set_option('conv_variant', names.index(name))
+        got = rt.graph_inference(graph, batch, x)
+        errors[name] = np.abs(got - want).max() / scale
+    fp32 = max(errors['wq_m32n16_w8_t16'], errors['m64n64k32_w2x2x1_t32'])
+    assert fp32 < 2e-6, errors                                   # K = 2304 fp32 accumulation
+    for name, err in errors.items():
+        if name.startswith('x3_'):
+            assert err < 2.0 * fp32 + 1e-7, errors               # bfloat16 operands alone would give ~4e-3
+
+
 def test_split_k_is_repeatable_in_a_session():
     rt.set_option('conv_split_k', 4)
     graph = single_op_graph((64, 12, 12), lambda b, v: ios.conv2d(b, [[v]], 40, (3, 3), (1, 1), (1, 1), 1, 'relu', is_exit=True))

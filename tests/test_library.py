@@ -304,6 +304,26 @@ def test_xcd_local_split_k_numbering(tiles, split):
     assert blocks - len(seen) == (8 * ((tiles + 7) // 8) - tiles) * split
 
 
+def test_three_bfloat16_terms_of_an_fp32_value_are_exact():
+    """The x3_* convolution kernels multiply fp32 operands on the bfloat16 matrix pipe: x = hi + mid + lo with three bfloat16
+    terms must hold exactly (it is what makes six bfloat16 products as accurate as one fp32 product)."""
+    lib = rt.get_lib()
+    lib.ios_split_bf16x3.argtypes = [ctypes.c_float, ctypes.POINTER(ctypes.c_uint)]
+    lib.ios_split_bf16x3.restype = None
+    rng = np.random.default_rng(7)
+    values = np.concatenate([rng.standard_normal(4000).astype(np.float32) * np.float32(10.0) ** rng.integers(-20, 20, 4000).astype(np.float32),
+                             np.array([0.0, -0.0, 1.0, -1.0, 1.0 + 2.0 ** -23, 1.0 - 2.0 ** -24, 3.4028235e38, -3.4028235e38, 1.17549435e-38,
+                                       0.1, 1 / 3, 255.99998, 65535.996, 2.0 ** -100 * 1.9999999], dtype=np.float32)])
+    terms = (ctypes.c_uint * 3)()
+    for x in values:
+        lib.ios_split_bf16x3(ctypes.c_float(float(x)), terms)
+        parts = np.array(list(terms), dtype=np.uint32)
+        assert not (parts & 0xffff).any()                       # each term is a bfloat16
+        as_float = parts.view(np.float32).astype(np.float64)
+        assert as_float.sum() == np.float64(x), (x, as_float)
+        assert abs(as_float[1]) <= abs(as_float[0]) * 2.0 ** -7 + 0 and abs(as_float[2]) <= abs(as_float[0]) * 2.0 ** -15 + 0
+
+
 def test_split_k_partial_tiles_share_the_arena_like_any_other_region():
     # every convolution forced to four K slices: their partial tiles are regions with a lifetime of one stage, so they share
     # addresses with tensors that are dead by then, and must never land on one that a later operation still reads
