@@ -845,10 +845,14 @@ struct ConvWsplit {
     static constexpr bool KQUAD = QUAD;                    // packed filters are [k / 4][m][4] instead of [k][m]
     // accumulators + staged operands per lane decide whether the body fits the register budget of a fused launch
     // (the channel-padding-4 forms serve first layers, which are stages of their own: kept out of the fused launches)
-    static constexpr bool FUSABLE = CP == 0 && E + D * U * (TM + TN) <= (QUAD ? (MT == 32 ? 48 : 56) : 48);   // per-step addressing of the plain layout needs more registers, and so do the 16-register accumulator tuples of the 32 x 32 tiles
-    static constexpr int KREDUCED = RP;                    // 0: fp32 filters; 1: packed filters hold bfloat16; 2: IEEE half
+    static constexpr bool FUSABLE = RP != 3 && CP == 0 && E + D * U * (TM + TN) <= (QUAD ? (MT == 32 ? 48 : 56) : 48);   // per-step addressing of the plain layout needs more registers, and so do the 16-register accumulator tuples of the 32 x 32 tiles
+    static constexpr int KREDUCED = RP;                    // 0: fp32 filters; 1: packed filters hold bfloat16; 2: IEEE half; 3: three bfloat16 planes
+    // RP == 3: fp32 results from the bfloat16 matrix pipe, as in ConvSplit3 (operands split exactly into three bfloat16 terms,
+    // six of the nine partial products on v_mfma_f32_32x32x16_bf16): filters are split when packed, [k / 8][plane][m][8], and read
+    // as operands straight from global memory; a lane splits the eight input values it loads for a batch itself.
     static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
-    static_assert(RP >= 0 && RP <= 2 && (RP == 0 || (QUAD && MT == 16 && U == 4)), "the 16-bit paths are the 16 x 16 x 16 form of the quad layout");
+    static_assert(RP >= 0 && RP <= 3 && (RP == 0 || (RP == 3 ? QUAD && MT == 32 && U == 8 : QUAD && MT == 16 && U == 4)),
+                  "the 16-bit paths are the 16 x 16 x 16 form of the quad layout, the three-term path its 32 x 32 x 16 form");
 
     template <bool RES = false>
     __device__ static __forceinline__ void run(const ConvKernelArgs &a, float *red, int tile, int g, int z) {
@@ -897,7 +901,9 @@ struct ConvWsplit {
     for (int i = 0; i < TM; i++) {
         w_kill[i] = m0 + i * MT + lc < a.OCgP ? 0u : kOutOfRange;
         // byte offsets below 2^31 (checked on the host)
-        if (QUAD)   // [g][k / 4][m][4]: this lane's first quad of a batch is row (U / 4) * lk
+        if (RP == 3)   // [g][k / 8][plane][m] slots of 16 bytes: this lane's octet of a batch is lk
+            w_lane[i] = ((((unsigned)g * ((unsigned)a.Kq >> 3) + (unsigned)lk) * 3u) * (unsigned)a.OCgP + (unsigned)(m0 + i * MT + lc)) * 16u;
+        else if (QUAD)   // [g][k / 4][m][4]: this lane's first quad of a batch is row (U / 4) * lk
             w_lane[i] = (((unsigned)g * ((unsigned)a.Kq >> 2) + (unsigned)((U / 4) * lk)) * (unsigned)a.OCgP + (unsigned)(m0 + i * MT + lc)) * (RP != 0 ? 8u : 16u);
         else
             w_lane[i] = (((unsigned)g * (unsigned)a.Kq + (unsigned)lk) * (unsigned)a.OCgP + (unsigned)(m0 + i * MT + lc)) * 4u;
@@ -929,7 +935,10 @@ struct ConvWsplit {
     struct FilterStageBf16 {
         uintx2 v[TM];
     };
-    using FilterStage = std::conditional_t<(RP != 0), FilterStageBf16, FilterStageF32>;
+    struct FilterStageX3 {
+        uintx4 v[3][TM];
+    };
+    using FilterStage = std::conditional_t<(RP == 3), FilterStageX3, std::conditional_t<(RP != 0), FilterStageBf16, FilterStageF32>>;
     FilterStage av[D];
     float bv[D][U][TN];
 
@@ -945,7 +954,7 @@ struct ConvWsplit {
         q_cb = kb - tap * a.ICgP;
         q_kh = a.KW == 1 ? tap : (int)__umulhi((unsigned)tap, a.magic_kw);
         q_kw = tap - q_kh * a.KW;
-        q_w = (unsigned)((kb / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
+        q_w = RP == 3 ? (unsigned)((kb / 8) * 3 * a.OCgP) * 16u : (unsigned)((kb / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
     }
     // `live` (wavefront-uniform) is false for a batch beyond the wavefront's K range: its loads are still issued, against
     // descriptors of extent zero, and return zeros without touching memory.  Loads are never skipped by a branch inside
@@ -963,7 +972,13 @@ struct ConvWsplit {
             (void)s0;
             const __amdgpu_buffer_rsrc_t xr = buffer_of(a.x, live ? a.x_bytes : 0u);
             const __amdgpu_buffer_rsrc_t wr = buffer_of(a.wp, live ? a.w_bytes : 0u);
-            if constexpr (RP != 0) {
+            if constexpr (RP == 3) {
+#pragma unroll
+                for (int p = 0; p < 3; p++)
+#pragma unroll
+                    for (int i = 0; i < TM; i++)   // eight bfloat16 = the lane's eight k of this batch, one plane
+                        A.v[p][i] = __builtin_amdgcn_raw_buffer_load_b128(wr, w_lane[i] | w_kill[i], q_w + (unsigned)(p * a.OCgP) * 16u, 0);
+            } else if constexpr (RP != 0) {
 #pragma unroll
                 for (int i = 0; i < TM; i++) {   // four 16-bit values = the lane's four k of this batch
                     A.v[i] = buffer_load_u32x2(wr, w_lane[i] | w_kill[i], q_w);
@@ -1007,7 +1022,7 @@ struct ConvWsplit {
                     for (int j = 0; j < TN; j++) B[u][j] = buffer_load_f32(xr, voff[j], x_chan + (unsigned)(u * a.HW) * 4u);
             }
             // next batch (selects, not branches: the loop body stays one basic block)
-            q_w += (unsigned)((U * M::KSTEP / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
+            q_w += RP == 3 ? (unsigned)((U * M::KSTEP / 8) * 3 * a.OCgP) * 16u : (unsigned)((U * M::KSTEP / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
             q_cb += U * M::KSTEP;
             const bool next_tap = q_cb >= a.ICgP;
             q_cb = next_tap ? 0 : q_cb;
@@ -1044,7 +1059,30 @@ struct ConvWsplit {
     // folded ReLU of the producer: as integers, negative floats are below 0 and everything is above INT_MIN
     const int relu_floor = a.pre_relu ? 0 : (int)0x80000000;
     auto compute = [&](const FilterStage &A, const float(&B)[U][TN]) {
-        if constexpr (RP != 0) {
+        if constexpr (RP == 3) {
+            bf16x8 bq[3][TN];
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = __int_as_float(max(__float_as_int(B[u][j]), relu_floor));
+                uintx4 hi, mid, lo;
+                split_bf16x3(v, hi, mid, lo);
+                bq[0][j] = __builtin_bit_cast(bf16x8, hi);
+                bq[1][j] = __builtin_bit_cast(bf16x8, mid);
+                bq[2][j] = __builtin_bit_cast(bf16x8, lo);
+            }
+            // the six terms, smallest first; the tiles of a term are independent instructions
+            constexpr int TA[6] = {2, 0, 1, 1, 0, 0}, TB[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+            for (int t = 0; t < 6; t++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A.v[TA[t]][i]), bq[TB[t]][j], acc[i][j], 0, 0, 0);
+            return;
+        } else if constexpr (RP != 0) {
 #pragma unroll
             for (int j = 0; j < TN; j++) {
                 const floatx4 b32 = {__int_as_float(max(__float_as_int(B[0][j]), relu_floor)), __int_as_float(max(__float_as_int(B[1][j]), relu_floor)),
@@ -1062,16 +1100,17 @@ struct ConvWsplit {
                 }
             }
             return;
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const float bval = __int_as_float(max(__float_as_int(B[u][j]), relu_floor));   // one integer max
+                        acc[i][j] = M::run(A.v[u][i], bval, acc[i][j]);
+                    }
         }
-#pragma unroll
-        for (int u = 0; u < U; u++)
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const float bval = __int_as_float(max(__float_as_int(B[u][j]), relu_floor));   // one integer max
-                    acc[i][j] = M::run(A.v[u][i], bval, acc[i][j]);
-                }
     };
 
     const int batches = (s_end - s_begin + U - 1) / U;   // <= 0 for wavefronts beyond the end of K
@@ -1335,6 +1374,18 @@ struct ConvWsplit {
     X(95, "x3_m128n64_w4x1", 1, 2, 4, 1, 2)        \
     X(96, "x3_m128n128_w4x2", 1, 2, 4, 2, 2)       \
     X(97, "x3_m192n128_w6x2", 1, 2, 6, 2, 2)
-constexpr int kNumConvVariants = 98;
+// X(index, name, TM, TN, NW, D): wave-split configurations with operands split into three bfloat16 terms (ConvWsplit, RP = 3),
+// 32 x 32 x 16 tiles, 16 k per batch
+#define IOS_WSPLIT_X3_VARIANTS(X)            \
+    X(98, "x3w_m32n32_w8", 1, 1, 8, 2)       \
+    X(99, "x3w_m32n32_w4", 1, 1, 4, 2)       \
+    X(100, "x3w_m32n32_w16", 1, 1, 16, 2)    \
+    X(101, "x3w_m64n32_w8", 2, 1, 8, 2)      \
+    X(102, "x3w_m64n32_w4", 2, 1, 4, 2)      \
+    X(103, "x3w_m32n64_w4", 1, 2, 4, 2)      \
+    X(104, "x3w_m32n64_w8", 1, 2, 8, 2)      \
+    X(105, "x3w_m64n64_w4", 2, 2, 4, 2)      \
+    X(106, "x3w_m64n32_w2", 2, 1, 2, 2)
+constexpr int kNumConvVariants = 107;
 
 }  // namespace ios

@@ -55,10 +55,15 @@ struct VariantEntry {
      conv_kernel<ConvSplit3<TMW, TNW, WM, WN, PD>>, conv_kernel<ConvSplit3<TMW, TNW, WM, WN, PD>, true>,                                  \
      ConvSplit3<TMW, TNW, WM, WN, PD>::SMEM_FLOATS},
 
+#define IOS_WSPLIT_X3_ENTRY(IDX, NAME, TM, TN, NW, D)                                                                        \
+    {{NAME, TM * 32, TN * 32, 16, 1, 1, NW, 32, true, ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::CPAD, true, false, PREC_FP32, 1},      \
+     conv_kernel<ConvWsplit<32, TM, TN, NW, 8, true, D, 3>>, conv_kernel<ConvWsplit<32, TM, TN, NW, 8, true, D, 3>, true>,              \
+     ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::SMEM_FLOATS},
+
 static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)
                                              IOS_WSPLIT_C4_VARIANTS(IOS_WSPLIT_C4_ENTRY)
                                              IOS_WSPLIT_T32_VARIANTS(IOS_WSPLIT_ENTRY) IOS_WSPLIT_F16_VARIANTS(IOS_WSPLIT_ENTRY)
-                                             IOS_WSPLIT_LONGK_VARIANTS(IOS_WSPLIT_ENTRY) IOS_SPLIT3_VARIANTS(IOS_SPLIT3_ENTRY)};
+                                             IOS_WSPLIT_LONGK_VARIANTS(IOS_WSPLIT_ENTRY) IOS_SPLIT3_VARIANTS(IOS_SPLIT3_ENTRY) IOS_WSPLIT_X3_VARIANTS(IOS_WSPLIT_X3_ENTRY)};
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 static_assert(kNumVariants == kNumConvVariants, "variant lists and count disagree");
 
