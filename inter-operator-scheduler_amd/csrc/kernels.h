@@ -124,7 +124,9 @@ struct PoolProblem {
     int B, C, H, W, KH, KW, sh, sw, ph, pw, OH, OW;
     int is_max;  // 1: max over in-range elements, 0: sum of in-range elements / (KH*KW)
 };
-void launch_pool(const PoolProblem &p, const TensorView &x, const TensorView &y, hipStream_t stream);
+// With `bias` (one value per channel): y = act(pool(x) + bias[c]).
+void launch_pool(const PoolProblem &p, const TensorView &x, const TensorView &y, hipStream_t stream, const float *bias = nullptr,
+                 int act = ACT_NONE);
 // Window == whole map: one wavefront reduces one (n, c) plane.
 void launch_global_pool(const PoolProblem &p, const TensorView &x, const TensorView &y, hipStream_t stream);
 

@@ -63,6 +63,9 @@ struct PNode {
     Val residual_other{-1, 0, 0};
     bool residual_relu = false;
     bool made_by_conv = false;
+    // "average pool, then 1 x 1 convolution" run as "1 x 1 convolution, then average pool": on the pool the convolution, on
+    // the convolution the pool
+    int commuted_conv = -1, commuted_pool = -1;
     int references = 0;            // number of input values that name this node
 };
 
@@ -323,6 +326,7 @@ private:
         find_depthwise_sums();
         find_activated_combinations();
         find_residual_convolutions();
+        find_commuting_pools();
         for (PNode &n : nodes_) {
             if (n.type == NodeType::Identity && single_value(n)) {
                 n.parent = n.inputs[0][0].node;
@@ -498,6 +502,40 @@ private:
                 e.no_storage = holder != static_cast<int>(i);
                 break;
             }
+        }
+    }
+
+    // "Average pool that keeps the map size, then 1 x 1 convolution to no more channels, read by nobody else" (the pool branch
+    // of the reference's Inception blocks, python/ios/models/inception_v3.py:28-29,62-63,96-97; pool semantics
+    // src/ios/ios_runtime.cu:542-550, average over the padded window): both are linear and act on different axes, so W * pool(x) = pool(W * x) with the same
+    // border rule.  The launch at the pool's place in the schedule computes z = W * x (no bias, no activation), the launch at
+    // the convolution's place pools z, adds the bias and applies the activation: the pool then moves OC instead of IC
+    // channels, and the pooled input tensor is neither written nor read back.  Sums are rounded in another order than in the
+    // reference's sequence of operators (differences of a few units in the last place).
+    void find_commuting_pools() {
+        if (!planner_commute_pool_conv()) return;
+        for (size_t i = 0; i < nodes_.size(); i++) {
+            PNode &c = nodes_[i];
+            if (c.type != NodeType::Conv || !single_value(c) || c.sum_front >= 0 || c.residual_into >= 0) continue;
+            const Val &v = c.inputs[0][0];
+            PNode &pool = nodes_[v.node];
+            if (pool.type != NodeType::Pool || v.begin != 0 || v.end != pool.C || pool.references != 1 || !single_value(pool)) continue;
+            bool wrapped = false;   // the result of a Sequential can be read under the Sequential's name
+            for (const PNode &s : nodes_) wrapped = wrapped || (s.type == NodeType::Sequential && s.parent == v.node);
+            if (wrapped || pool.no_storage || pool.commuted_conv >= 0) continue;
+            const std::string pool_type = (*pool.cfg)["pool_type"].as_string();
+            if (pool_type.find("avg") == std::string::npos || pool_type.find("max") != std::string::npos ||
+                pool_type.find("global") != std::string::npos)
+                continue;
+            const PNode &x = nodes_[pool.inputs[0][0].node];
+            if (x.pre_relu_alias || x.H != pool.H || x.W != pool.W) continue;
+            const ConvProblem p = problem_of(c);
+            if (p.KH != 1 || p.KW != 1 || p.sh != 1 || p.sw != 1 || p.ph != 0 || p.pw != 0 || p.groups != 1 || p.OC > p.IC) continue;
+            if (!conv_matrix_path_supported(p) || conv_thin_applies(p)) continue;
+            pool.commuted_conv = static_cast<int>(i);
+            pool.no_storage = true;   // z lives in a temporary of the convolution's channel count
+            pool.parent = -1;
+            c.commuted_pool = v.node;
         }
     }
 
@@ -719,7 +757,7 @@ private:
     void emit(int index) {
         PNode &n = nodes_[index];
         if (n.type == NodeType::Placeholder || n.type == NodeType::Sequential) return;
-        if (n.no_storage) return;   // ReLU in front of a depth-wise convolution that reads the summed inputs itself
+        if (n.no_storage && n.commuted_conv < 0) return;   // e.g. a ReLU in front of a depth-wise convolution that reads the summed inputs itself
         if (n.made_by_conv) return;  // addition (and ReLU) of a residual unit: the convolution's epilogue wrote this tensor
         // levels count inside a schedule unit; the members of a Sequential follow each other
         if (n.unit != level_unit_) {
@@ -731,8 +769,14 @@ private:
         input_shape(n, C, H, W);
         const Json &cfg = *n.cfg;
         switch (n.type) {
-            case NodeType::Conv: emit_conv(n, cfg, C, H, W, index); break;
-            case NodeType::Pool: emit_pool(n, cfg, C, H, W, index); break;
+            case NodeType::Conv:
+                if (n.commuted_pool >= 0) emit_pool_behind_conv(n, index);
+                else emit_conv(n, cfg, C, H, W, index);
+                break;
+            case NodeType::Pool:
+                if (n.commuted_conv >= 0) emit_conv_before_pool(n, C, H, W, index);
+                else emit_pool(n, cfg, C, H, W, index);
+                break;
             case NodeType::Identity:
                 if (!single_value(n)) emit_terms(n, index, ACT_NONE, false);
                 break;
@@ -841,14 +885,13 @@ private:
         }
     }
 
-    void emit_pool(PNode &n, const Json &cfg, int C, int H, int W, int index) {
-        const ViewRef in = input_view(n, C, H, W, nullptr);
+    PoolProblem pool_problem_of(const PNode &n, int C, int H, int W) const {
+        const Json &cfg = *n.cfg;
         const std::string pool_type = cfg["pool_type"].as_string();
-        const bool global = pool_type.find("global") != std::string::npos;
         PoolProblem p;
         p.B = batch_; p.C = C; p.H = H; p.W = W;
         p.is_max = pool_type.find("max") != std::string::npos ? 1 : 0;
-        if (global) {
+        if (pool_type.find("global") != std::string::npos) {
             p.KH = H; p.KW = W; p.sh = 1; p.sw = 1; p.ph = 0; p.pw = 0;
         } else {
             p.KH = cfg["kernel"][0].as_int(); p.KW = cfg["kernel"][1].as_int();
@@ -856,6 +899,49 @@ private:
             p.ph = cfg["padding"][0].as_int(); p.pw = cfg["padding"][1].as_int();
         }
         p.OH = n.H; p.OW = n.W;
+        return p;
+    }
+
+    // the launch at the place of a commuted average pool (see find_commuting_pools): z = W * x into a temporary
+    void emit_conv_before_pool(PNode &pool, int C, int H, int W, int index) {
+        const PNode &c = nodes_[pool.commuted_conv];
+        const ViewRef in = input_view(pool, C, H, W, nullptr);
+        ConvProblem p = problem_of(c);
+        p.act = ACT_NONE;
+        const bool wide = ((unsigned long long)(batch_ - 1) * in.bstride + in.image_floats()) * 4ull >= (1ull << 31);
+        const int conv = add_plan_conv(c, p);
+        plan_.convs[conv].matrix_path = !wide;
+        plan_.convs[conv].linear = true;
+        plan_.convs[conv].zero_bias_off = reserve((size_t)p.OC);
+        const ViewRef z = dense_temp(p.OC, H, W);
+        commuted_z_[index] = z;
+        PlanOp &op = push(wide ? OpKind::ConvDirect : OpKind::ConvMfma, pool);
+        op.in = in;
+        op.out = z;
+        op.conv = conv;
+        op.flops = p.flops();
+        op.bytes = 4.0 * ((double)batch_ * C * H * W + (double)p.OC * p.K() + (double)batch_ * p.OC * H * W);
+    }
+
+    // the launch at the place of the convolution behind a commuted average pool: y = act(pool(z) + bias)
+    void emit_pool_behind_conv(PNode &c, int index) {
+        const PNode &pool = nodes_[c.commuted_pool];
+        const ViewRef z = commuted_z_.at(c.commuted_pool);
+        const PoolProblem p = pool_problem_of(pool, z.C, z.H, z.W);
+        PlanOp &op = push(OpKind::Pool, c);
+        op.in = z;
+        op.out = view_of(index);
+        op.pool = p;
+        op.bias_conv = plan_.conv_index.at(c.name);
+        op.act = act_code((*c.cfg)["act"].as_string());
+        op.flops = (double)batch_ * z.C * p.OH * p.OW * (p.KH * p.KW + 1);
+        op.bytes = 4.0 * ((double)batch_ * z.C * ((double)z.H * z.W + (double)p.OH * p.OW) + z.C);
+    }
+
+    void emit_pool(PNode &n, const Json &cfg, int C, int H, int W, int index) {
+        const ViewRef in = input_view(n, C, H, W, nullptr);
+        const bool global = cfg["pool_type"].as_string().find("global") != std::string::npos;
+        const PoolProblem p = pool_problem_of(n, C, H, W);
         PlanOp &op = push(global ? OpKind::GlobalPool : OpKind::Pool, n);
         op.in = in;
         op.out = view_of(index);
@@ -988,6 +1074,7 @@ private:
     std::vector<SeqRange> sequentials_;
     std::vector<Region> regions_;   // ascending virtual offsets
     size_t region_floats_ = 0;
+    std::map<int, ViewRef> commuted_z_;   // commuted pool node -> the temporary between the convolution and the pool
 };
 
 void json_escape(std::ostringstream &os, const std::string &s) {
@@ -1006,11 +1093,16 @@ namespace {
 bool g_arena_reuse = true;
 long long g_thin_conv_min_pixels = 1LL << 18;
 int g_host_split_k = 0;
+bool g_commute_pool_conv = true;
 }
 
 bool set_planner_option(const std::string &key, const std::string &value) {
     if (key == "arena_reuse") {
         g_arena_reuse = !(value == "0" || value == "false" || value == "off" || value.empty());
+        return true;
+    }
+    if (key == "commute_pool_conv") {
+        g_commute_pool_conv = !(value == "0" || value == "false" || value == "off" || value.empty());
         return true;
     }
     if (key == "thin_conv_min_pixels") {
@@ -1029,6 +1121,7 @@ bool set_planner_option(const std::string &key, const std::string &value) {
 bool planner_arena_reuse() { return g_arena_reuse; }
 long long planner_thin_conv_min_pixels() { return g_thin_conv_min_pixels; }
 int planner_host_split_k() { return g_host_split_k; }
+bool planner_commute_pool_conv() { return g_commute_pool_conv; }
 
 Plan build_plan(PlanMode mode, const Json &doc, const Json *extra, int batch, const LaunchChooser &chooser) {
     Planner planner(batch, chooser);
@@ -1063,6 +1156,8 @@ std::string describe_plan(const Plan &plan) {
         if (op.kind == OpKind::Nary) os << ",\"inputs\":" << op.srcs.size() << ",\"accumulate\":" << op.accumulate;
         if (op.kind == OpKind::ConvDepthwise) os << ",\"inputs\":" << (op.srcs.empty() ? 1 : op.srcs.size());
         if (op.kind == OpKind::Nary || op.kind == OpKind::Unary) os << ",\"act\":" << op.act;
+        if (op.bias_conv >= 0) os << ",\"adds_bias_of\":\"" << plan.convs[op.bias_conv].name << "\",\"act\":" << op.act;
+        if (op.conv >= 0 && plan.convs[op.conv].linear) os << ",\"linear\":true";
         if (op.has_residual) os << ",\"residual\":true,\"post_relu\":" << op.post_relu;
         os << ",\"level\":" << op.level;
         // arena extents in floats, one [begin, end) per image: what the operation writes and what it reads

@@ -51,6 +51,10 @@ struct PlanConv {
     size_t ctr_off = 0, ctr_count = 0;         // split-K ticket counters (32-bit words at float offsets), zeroed at session setup
     ConvLaunch launch;
     bool matrix_path = false;
+    // "average pool, then this convolution" run as "this convolution without bias and activation, then the pool, which adds
+    // the bias and applies the activation": the convolution's launch reads OC zeros at zero_bias_off instead of the bias
+    bool linear = false;
+    size_t zero_bias_off = 0;
     bool thin = false;   // direct path: the kernel for 3 x 3 convolutions of 3-channel images (first layers at large batches)
 };
 
@@ -64,6 +68,7 @@ struct PlanOp {
     int level = 0;
     ViewRef in, out;
     int conv = -1;        // index into Plan::convs
+    int bias_conv = -1;   // Pool behind a commuted convolution: out = act(pool(in) + bias of that convolution)
     PoolProblem pool{};
     std::vector<ViewRef> srcs;   // Nary: inputs; ConvDepthwise of a sum: the views it adds in its loader (else empty)
     int multiply = 0, accumulate = 0, act = 0;
@@ -111,10 +116,12 @@ std::string describe_plan(const Plan &plan);   // JSON array, one object per op
 
 // Planner options that need no device: "arena_reuse" = "1" (default) | "0"; "thin_conv_min_pixels" = least number of output
 // pixels (batch x OH x OW) from which a 3 x 3 convolution of a 3-channel image takes the output-bound direct kernel instead
-// of the matrix path (default 2^18; a negative value disables it).  Returns false for an unknown key.
+// of the matrix path (default 2^18; a negative value disables it); "commute_pool_conv" = "1" (default) | "0": run "average
+// pool that keeps the map size, then 1 x 1 convolution" as "convolution, then pool".  Returns false for an unknown key.
 bool set_planner_option(const std::string &key, const std::string &value);
 bool planner_arena_reuse();
 long long planner_thin_conv_min_pixels();
 int planner_host_split_k();   // option host_plan_split_k
+bool planner_commute_pool_conv();   // option commute_pool_conv (default 1): see PlanConv::linear
 
 }  // namespace ios

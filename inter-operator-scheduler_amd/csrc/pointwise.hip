@@ -23,7 +23,7 @@ static int blocks_for(long long n, int per_block, int cap) {
 }
 
 // ---- argument builders (shared with the fused stage kernel) ---------------------------------------------------------
-PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorView &y, bool global, int *blocks) {
+PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorView &y, bool global, int *blocks, const float *bias, int act) {
     if (x.C != p.C || x.H != p.H || x.W != p.W || y.C != p.C || y.H != p.OH || y.W != p.OW)
         throw std::runtime_error("pool: tensor views do not match the problem");
     if (global && (p.KH != p.H || p.KW != p.W || p.OH != 1 || p.OW != 1))
@@ -37,6 +37,8 @@ PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorV
     a.p = p;
     a.strip_rows = 0;
     a.vec_columns = 1;
+    a.bias = bias;
+    a.act = act;
     if (global) {
         // from 2^14 planes on (a lane per plane still gives every compute unit a wavefront) the row form, else a wavefront per plane
         const long long planes = (long long)p.B * p.C;
@@ -144,9 +146,9 @@ NaryKernelArgs make_nary_args(const NaryArgs &in, int multiply, int accumulate, 
 }
 
 // ---- launchers ---------------------------------------------------------------------------------------------------------
-void launch_pool(const PoolProblem &p, const TensorView &x, const TensorView &y, hipStream_t stream) {
+void launch_pool(const PoolProblem &p, const TensorView &x, const TensorView &y, hipStream_t stream, const float *bias, int act) {
     int blocks;
-    const PoolArgs a = make_pool_args(p, x, y, false, &blocks);
+    const PoolArgs a = make_pool_args(p, x, y, false, &blocks, bias, act);
     hipLaunchKernelGGL(pool_kernel, dim3(blocks), dim3(256), 0, stream, a);
 }
 

@@ -26,7 +26,15 @@ struct PoolArgs {
     PoolProblem p;
     int strip_rows;   // 3 x 3 windows: output rows per thread (see pool3x3_body); 0 selects the generic body
     int vec_columns;  // 3 x 3 windows: output columns per thread, 1 or kPoolVecColumns (see pool3x3_vec_body)
+    // the pool behind a bias-free convolution (an average pool and a 1 x 1 convolution exchanged): y = act(pool(x) + bias[c]);
+    // nullptr for a plain pool
+    const float *bias;
+    int act;
 };
+
+__device__ __forceinline__ float pool_finish(const PoolArgs &a, float v, unsigned c) {
+    return a.bias != nullptr ? act_apply(v + a.bias[c], a.act) : v;
+}
 
 __device__ __forceinline__ void pool_generic_body(const PoolArgs &a, int block, int num_blocks, unsigned threads) {
     const PoolProblem &p = a.p;
@@ -53,7 +61,7 @@ __device__ __forceinline__ void pool_generic_body(const PoolArgs &a, int block, 
                 best = fmaxf(best, v);
                 sum += v;
             }
-        a.y[(long long)b * a.y_bs + o] = p.is_max ? best : sum * inv;
+        a.y[(long long)b * a.y_bs + o] = pool_finish(a, p.is_max ? best : sum * inv, c);
     }
 }
 
@@ -97,7 +105,7 @@ __device__ __forceinline__ void pool3x3_body(const PoolArgs &a, int block, int n
             return is_max ? fmaxf(fmaxf(v0, v1), v2) : (v0 + v1) + v2;
         };
         auto combine = [&](float r0, float r1, float r2) -> float {
-            return is_max ? fmaxf(fmaxf(r0, r1), r2) : ((r0 + r1) + r2) * (1.0f / 9.0f);
+            return pool_finish(a, is_max ? fmaxf(fmaxf(r0, r1), r2) : ((r0 + r1) + r2) * (1.0f / 9.0f), c);
         };
         const int oh_begin = (int)strip * R;
         const int oh_end = min(p.OH, oh_begin + R);
@@ -176,7 +184,8 @@ __device__ __forceinline__ void pool3x3_vec_body(const PoolArgs &a, int block, i
         auto store = [&](int oh, const float (&r0)[V], const float (&r1)[V], const float (&r2)[V]) {
             float o[V];
 #pragma unroll
-            for (int k = 0; k < V; k++) o[k] = is_max ? fmaxf(fmaxf(r0[k], r1[k]), r2[k]) : ((r0[k] + r1[k]) + r2[k]) * (1.0f / 9.0f);
+            for (int k = 0; k < V; k++)
+                o[k] = pool_finish(a, is_max ? fmaxf(fmaxf(r0[k], r1[k]), r2[k]) : ((r0[k] + r1[k]) + r2[k]) * (1.0f / 9.0f), c);
             float *yr = yc + oh * p.OW;
             if (ow0 + V <= p.OW) {
                 pw_floatx4_u q;
@@ -253,7 +262,7 @@ __device__ __forceinline__ void global_pool_rows_body(const PoolArgs &a, int blo
         }
         const float m = fmaxf(fmaxf(best[0], best[1]), fmaxf(best[2], best[3]));
         const float t = (sum[0] + sum[1]) + (sum[2] + sum[3]);
-        a.y[(long long)b * a.y_bs + c] = is_max ? m : t / (float)HW;
+        a.y[(long long)b * a.y_bs + c] = pool_finish(a, is_max ? m : t / (float)HW, c);
     }
 }
 
@@ -281,7 +290,7 @@ __device__ __forceinline__ void global_pool_body(const PoolArgs &a, int block, i
             best = fmaxf(best, __shfl_xor(best, off, 64));
             sum += __shfl_xor(sum, off, 64);
         }
-        if (lane == 0) a.y[b * a.y_bs + c] = p.is_max ? best : sum / (float)HW;
+        if (lane == 0) a.y[b * a.y_bs + c] = pool_finish(a, p.is_max ? best : sum / (float)HW, (unsigned)c);
     }
 }
 

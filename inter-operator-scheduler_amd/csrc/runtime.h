@@ -164,6 +164,7 @@ private:
     void tune_convs();
     void launch_op(const PlanOp &op, int group);   // on stream `group` of the pool
     unsigned *counters_of(const PlanConv &c) const;
+    const float *bias_of(const PlanConv &c) const { return base_ + (c.linear ? c.zero_bias_off : c.bias_off); }
     void enqueue(bool stage_events);   // issue one forward pass according to the execution mode
     void enqueue_streams(bool stage_events);
     void enqueue_fused(bool stage_events);

@@ -523,6 +523,8 @@ void Session::setup() {
     hipStream_t main = ctx_.stream(0);
     if (owns_memory_) launch_fill_pattern(base_, plan_.arena_floats, 0x2468aceu, main);
     for (const PlanConv &conv : plan_.convs) {
+        // a convolution in front of the average pool it was exchanged with adds zeros; the pool adds the bias
+        if (conv.linear) launch_fill_u32(reinterpret_cast<unsigned *>(base_ + conv.zero_bias_off), (size_t)conv.problem.OC, 0u, main);
         if (!conv.matrix_path) continue;
         // the probes never upload filters: pack whatever the filter region holds so that the matrix
         // path reads initialised memory
@@ -613,7 +615,7 @@ void Session::launch_op(const PlanOp &op, int group) {
         case OpKind::ConvMfma: {
             const PlanConv &c = plan_.convs[op.conv];
             const TensorView residual = op.has_residual ? tv(op.residual) : TensorView{};
-            launch_conv_mfma(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off, tv(op.out),
+            launch_conv_mfma(c.problem, c.launch, tv(op.in), base_ + c.packed_off, bias_of(c), tv(op.out),
                              c.ws_floats ? base_ + c.ws_off : nullptr, ctx_.split_reduce(counters_of(c), group, !capturing_forks_), stream,
                              op.has_residual ? &residual : nullptr,
                              op.post_relu != 0);
@@ -623,16 +625,18 @@ void Session::launch_op(const PlanOp &op, int group) {
             const PlanConv &c = plan_.convs[op.conv];
             TensorView more[kMaxNaryInputs];
             for (size_t i = 1; i < op.srcs.size(); i++) more[i - 1] = tv(op.srcs[i]);
-            launch_dwconv(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), stream, more,
+            launch_dwconv(c.problem, tv(op.in), base_ + c.weight_off, bias_of(c), tv(op.out), stream, more,
                           op.srcs.empty() ? 0 : (int)op.srcs.size() - 1);
             break;
         }
         case OpKind::ConvDirect: {
             const PlanConv &c = plan_.convs[op.conv];
-            launch_conv_direct(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), stream, c.thin);
+            launch_conv_direct(c.problem, tv(op.in), base_ + c.weight_off, bias_of(c), tv(op.out), stream, c.thin);
             break;
         }
-        case OpKind::Pool: launch_pool(op.pool, tv(op.in), tv(op.out), stream); break;
+        case OpKind::Pool:
+            launch_pool(op.pool, tv(op.in), tv(op.out), stream, op.bias_conv >= 0 ? base_ + plan_.convs[op.bias_conv].bias_off : nullptr, op.act);
+            break;
         case OpKind::GlobalPool: launch_global_pool(op.pool, tv(op.in), tv(op.out), stream); break;
         case OpKind::Nary: {
             NaryArgs a;
@@ -744,7 +748,7 @@ void Session::build_fused() {
                     case OpKind::ConvMfma: {
                         const PlanConv &c = plan_.convs[op.conv];
                         const TensorView residual = op.has_residual ? tv(op.residual) : TensorView{};
-                        const ConvDispatch d = make_conv_dispatch(c.problem, c.launch, tv(op.in), base_ + c.packed_off, base_ + c.bias_off,
+                        const ConvDispatch d = make_conv_dispatch(c.problem, c.launch, tv(op.in), base_ + c.packed_off, bias_of(c),
                                                                   tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr, ctx_.split_reduce(counters_of(c)),
                                                                   op.has_residual ? &residual : nullptr, op.post_relu != 0);
                         pend.fusable = conv_variant(d.variant).fusable() && !op.has_residual;   // (the fused kernel holds the plain epilogue)
@@ -784,7 +788,7 @@ void Session::build_fused() {
                         const PlanConv &c = plan_.convs[op.conv];
                         pend.item.kind = op.kind == OpKind::ConvDepthwise ? WORK_DWCONV : WORK_CONV_DIRECT;
                         if (c.thin) throw std::runtime_error("internal: the thin-input convolution kernel is planned for single-group stages only");
-                        pend.item.direct = make_direct_conv_args(c.problem, tv(op.in), base_ + c.weight_off, base_ + c.bias_off, tv(op.out), &blocks);
+                        pend.item.direct = make_direct_conv_args(c.problem, tv(op.in), base_ + c.weight_off, bias_of(c), tv(op.out), &blocks);
                         if (op.kind == OpKind::ConvDepthwise && op.srcs.size() > 1) {
                             TensorView more[kMaxNaryInputs];
                             for (size_t i = 1; i < op.srcs.size(); i++) more[i - 1] = tv(op.srcs[i]);
@@ -795,7 +799,8 @@ void Session::build_fused() {
                     case OpKind::Pool:
                     case OpKind::GlobalPool:
                         pend.item.kind = op.kind == OpKind::Pool ? WORK_POOL : WORK_GLOBAL_POOL;
-                        pend.item.pool = make_pool_args(op.pool, tv(op.in), tv(op.out), op.kind == OpKind::GlobalPool, &blocks);
+                        pend.item.pool = make_pool_args(op.pool, tv(op.in), tv(op.out), op.kind == OpKind::GlobalPool, &blocks,
+                                                        op.bias_conv >= 0 ? base_ + plan_.convs[op.bias_conv].bias_off : nullptr, op.act);
                         break;
                     case OpKind::Nary:
                     case OpKind::Unary: {

@@ -640,7 +640,10 @@ def test_network_matches_oracle_under_every_schedule_and_executor(name, make, ba
                 tensor = session.tensor(node)
             except RuntimeError as error:
                 # a sum that only the ReLU behind it reads (RandWire's last stage output) is added by that ReLU's launch
-                assert 'no materialised output' in str(error) and node.type == 'identity' and name.startswith('randwire')
+                # an average pool exchanged with the 1 x 1 convolution behind it (Inception's pool branches) has no tensor either:
+                # the convolution's output, checked like every other node, covers both
+                assert 'no materialised output' in str(error)
+                assert (node.type == 'identity' and name.startswith('randwire')) or (node.type == 'pool' and name.startswith('inception'))
                 absorbed += 1
                 continue
             assert_close(tensor, want_all[node.name], f'{name}: node {node.name} ({node.type})', scaled=not strict)
@@ -662,7 +665,7 @@ def test_network_matches_oracle_under_every_schedule_and_executor(name, make, ba
             assert worst_share <= 0.02, worst_share
     assert_close(got, want, name, scaled=not strict)
     assert np.isfinite(got).all() and np.abs(got).max() > 0
-    assert absorbed == (1 if name.startswith('randwire') else 0)
+    assert absorbed == (1 if name.startswith('randwire') else 9 if name.startswith('inception') else 0)
     rt.set_option('arena_reuse', 1)      # everything below runs in the shared arena
 
     big = name.startswith(('randwire', 'nasnet'))

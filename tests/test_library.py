@@ -424,3 +424,40 @@ def test_planner_options_need_no_device_and_change_the_plan():
     finally:
         rt.set_option('thin_conv_min_pixels', 1 << 18)
         rt.set_option('arena_reuse', 1)
+
+
+def test_average_pools_change_places_with_the_pointwise_convolution_behind_them():
+    """
+    Inception's pool branches (reference python/ios/models/inception_v3.py:28-29,62-63,96-97): the launch at the pool's place
+    is the 1 x 1 convolution without bias and activation, the launch at the convolution's place pools its output and finishes
+    it; the pooled input tensor no longer exists.  Pools that change the map size, max pools and pools with other readers stay.
+    """
+    graph = ios.models.inception_v3()
+    graph.sequential_schedule()
+    by_name = {node.name: node for node in graph.nodes()}
+    try:
+        ops = rt.plan_describe(graph, 2)
+        linear = [op for op in ops if op.get('linear')]
+        finishing = [op for op in ops if 'adds_bias_of' in op]
+        assert len(linear) == len(finishing) == 9
+        for conv_op, pool_op in zip(linear, finishing):
+            pool_node, conv_node = by_name[conv_op['node']], by_name[pool_op['node']]
+            assert pool_node.type == 'pool' and conv_node.type == 'conv' and pool_op['adds_bias_of'] == conv_node.name
+            assert conv_op['kind'] == 'conv_mfma' and conv_op['conv']['act'] == 0 and pool_op['kind'] == 'pool'
+            assert conv_op['stage'] < pool_op['stage']
+            # z has the convolution's channels on the pool's input map; the pool writes the convolution's tensor
+            assert conv_op['out'] == [conv_node.out_channels, *pool_node.output_shape[1:]]
+            assert pool_op['out'] == list(conv_node.output_shape) and pool_op['act'] == 1
+            assert conv_op['writes'] == pool_op['reads']
+        assert sum(op['kind'] in ('pool', 'global_pool') for op in ops) == 14
+        _simulate(ops)
+        rt.set_option('commute_pool_conv', 0)
+        plain = rt.plan_describe(graph, 2)
+        assert not any(op.get('linear') or 'adds_bias_of' in op for op in plain)
+        assert sum(op["bytes"] for op in ops) < 0.95 * sum(op['bytes'] for op in plain)
+    finally:
+        rt.set_option('commute_pool_conv', 1)
+    # NASNet's reductions pool with stride 2 in front of 1 x 1 convolutions: the convolution would see four times the pixels
+    nasnet = ios.models.nasnet_mobile()
+    nasnet.sequential_schedule()
+    assert not any(op.get('linear') for op in rt.plan_describe(nasnet, 1))
