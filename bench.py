@@ -62,6 +62,11 @@ def network_roofline_ms(ops, parallel):
     return sum(max(groups.values()) for groups in stages.values())
 
 
+def progress(text):
+    """A line on stderr per phase: a run that takes minutes says what it is doing (stdout carries the one JSON line)."""
+    print(f'bench.py [{time.strftime("%H:%M:%S")}] {text}', file=sys.stderr, flush=True)
+
+
 def timed_latency(rt, np, graph, batch, x, steps, warmup):
     """
     Latency of a forward pass, three ways over `steps` passes after `warmup` passes, and the output:
@@ -387,6 +392,7 @@ def main():
     graph = make_graph(ios, 'inception_v3')
     x = np.random.default_rng(1).standard_normal((batch, 3, 299, 299)).astype(np.float32)
 
+    progress(f'schedule search, batch {batch}')
     # schedule search with measured stage latencies (not part of the timed steps)
     rt.set_option('autotune', 1)        # measure kernel configurations on first sight of a shape
     for item in args.option:
@@ -409,6 +415,7 @@ def main():
     graph.sequential_schedule()
 
     rt.set_option('executor', args.executor)
+    progress('timed passes')
     seq, seq_out = timed_latency(rt, np, graph, batch, x, args.steps, args.warmup)
     opt, opt_out = timed_latency(rt, np, optimized, batch, x, args.steps, args.warmup)
 
@@ -448,7 +455,7 @@ def main():
         'whole_pass': {'matrix_tflops': conv_flops / (opt['latency'] * 1e-3) / 1e12,
                        'frac_of_fp32_matrix_peak': conv_flops / (opt['latency'] * 1e-3) / 1e12 / PEAK_FP32_MATRIX_TFLOPS,
                        'algorithmic_gbs': total_bytes / (opt['latency'] * 1e-3) / 1e9},
-        'roofline': roofline_block(kernels, opt['latency'], headline=True),
+        'roofline': roofline_block(kernels, opt['latency'], headline=args.batch == 1),
         'kernels': kernels,
         'kernels_sequential_pass': seq_kernels,
         'stage_overlap': stage_overlap(ops, launches, stage_ms),
@@ -492,27 +499,43 @@ def main():
     if not args.no_sweep:
         sweep = {}
         for b in (16, 64):
+            progress(f'batch {b}: sequential and batch-1 schedules')
             xb = np.random.default_rng(1).standard_normal((b, 3, 299, 299)).astype(np.float32)
-            steps = max(10, args.steps // (b * 2))
+            steps = max(30, args.steps // b)
             s_seq, out_seq = timed_latency(rt, np, graph, b, xb, steps, 3)
             s_opt, out_opt = timed_latency(rt, np, optimized, b, xb, steps, 3)
-            # the schedule searched at this batch size (the reference's batch-size specialisation, experiments/specialization)
-            rt.set_option('executor', args.search_executor)
-            t0 = time.time()
-            optimized_b = ios.optimize(graph, batch_size=b, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
-                                       warmup=2, number=args.search_number, repeat=args.search_repeat,
-                                       max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
-            search_b = time.time() - t0
-            graph.sequential_schedule()
-            rt.set_option('executor', args.executor)
-            s_own, out_own = timed_latency(rt, np, optimized_b, b, xb, steps, 3)
+            # the schedule searched at this batch size (the reference's batch-size specialisation, experiments/specialization),
+            # once for the fused executor and once for the graph executor, whose parallel branches launch every operator by
+            # itself: there every kernel configuration competes for the parallel stages, also those too heavy on registers to
+            # share a fused launch, which pays from batch 16 on
+            searched = {}
+            for executor, search_executor in ((args.executor, args.search_executor), ('graph', 'streams')):
+                if executor in searched:
+                    continue
+                progress(f'batch {b}: schedule search for the {executor} executor')
+                rt.set_option('executor', search_executor)
+                t0 = time.time()
+                candidate = ios.optimize(graph, batch_size=b, cost_model=cost_model, opt_type='dp_parallel', compute_weight=True,
+                                         warmup=2, number=args.search_number, repeat=args.search_repeat,
+                                         max_group_size=args.max_group_size, max_num_groups=args.max_num_groups)
+                seconds = time.time() - t0
+                graph.sequential_schedule()
+                rt.set_option('executor', executor)
+                timed, out = timed_latency(rt, np, candidate, b, xb, steps, 3)
+                searched[executor] = {'schedule': candidate, 'timed': timed, 'out': out, 'search_seconds': seconds}
+            own_executor = min(searched, key=lambda e: searched[e]['timed']['latency'])
+            optimized_b, s_own, out_own = (searched[own_executor][k] for k in ('schedule', 'timed', 'out'))
+            search_b = sum(v['search_seconds'] for v in searched.values())
+            rt.set_option('executor', own_executor)
             _, _, kernels_b = launch_profile(rt, graph if s_seq['latency'] < s_own['latency'] else optimized_b, b, xb)
             ops_b = rt.plan_describe(graph, b)
             best = min(s_seq['latency'], s_opt['latency'], s_own['latency'])
             matrix_ms = sum(k['ms'] for k in kernels_b.values() if k['matrix_flops'] > 0)
             matrix_flops = sum(k['matrix_flops'] for k in kernels_b.values())
             sweep[str(b)] = {'sequential_ms': s_seq['latency'], 'dp_parallel_batch1_schedule_ms': s_opt['latency'],
-                             'dp_parallel_ms': s_own['latency'], 'search_seconds': search_b,
+                             'dp_parallel_ms': s_own['latency'], 'dp_parallel_executor': own_executor,
+                             'dp_parallel_ms_by_executor': {e: v['timed']['latency'] for e, v in searched.items()},
+                             'search_seconds': search_b,
                              'max_abs_diff_between_schedules': float(np.abs(out_seq - out_own).max()),
                              'images_per_s': b / (best * 1e-3),
                              'network_roofline_ms': network_roofline_ms(ops_b, parallel=False),
@@ -532,6 +555,7 @@ def main():
                 rt.set_option('precision', precision)
                 reduced = {}
                 for b in (1, 64):
+                    progress(f'{precision} operands, batch {b}')
                     xb = np.random.default_rng(1).standard_normal((b, 3, 299, 299)).astype(np.float32)
                     r_seq, out_b = timed_latency(rt, np, graph, b, xb, max(10, args.steps // (b * 2)), 3)
                     reduced[str(b)] = {'sequential_ms': r_seq['latency'], 'images_per_s': b / (r_seq['latency'] * 1e-3)}
@@ -544,6 +568,7 @@ def main():
     if not args.no_configs:
         configs = {}
         for name, search in (('sample_net', True), ('squeezenet_1_1', True), ('randwire_small', False), ('nasnet_mobile', False)):
+            progress(f'{name}, batch 1')
             g = make_graph(ios, name)
             xc = np.random.default_rng(1).standard_normal((1, *g.enter_node.output_shape)).astype(np.float32)
             if search or not args.greedy_big:
@@ -615,6 +640,7 @@ def main():
             result['reference_table_variants_batch1'] = variants
 
     if not args.no_cpu:
+        progress('CPU baseline and oracle comparison')
         import torch
         threads = torch.get_num_threads()
         config, weights = graph.export_config(), ios_oracle.graph_weights(graph)

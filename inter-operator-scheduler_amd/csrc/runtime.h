@@ -37,6 +37,7 @@ public:
 
     void set_option(const std::string &key, const std::string &value);
     ExecMode exec_mode() const { return exec_mode_; }
+    bool fused_executor() const { return exec_mode_ == ExecMode::Fused || exec_mode_ == ExecMode::FusedGraph; }
     bool autotune() const { return autotune_; }
     // split-K partial sums are added by a second kernel (Kernel), by the last block of a tile inside the convolution
     // kernel with the slices of a tile anywhere on the device (Inline), or the same with the slices of a tile numbered

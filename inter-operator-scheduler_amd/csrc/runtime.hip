@@ -144,7 +144,8 @@ static std::string conv_signature(const ConvProblem &p) {
 std::string DeviceContext::settings_token() const {
     std::ostringstream os;
     os << (share_cost_rule_ ? "cost" : "budget") << '/' << share_threads_per_cu_ << '/'
-       << (reduce_mode() == ReduceMode::Xcd ? "xcd" : reduce_mode() == ReduceMode::Inline ? "inline" : "kernel");
+       << (reduce_mode() == ReduceMode::Xcd ? "xcd" : reduce_mode() == ReduceMode::Inline ? "inline" : "kernel")
+       << (fused_executor() ? "" : "/own-launches");
     return os.str();
 }
 
@@ -292,11 +293,14 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     TunedConv result;
     bool found[kShareClasses];
     for (int c = 0; c < kShareClasses; c++) {
-        // class 0 is unconstrained; the others accept kernels that fit their share of the device and can run inside
-        // a fused stage launch; a budget nobody fits takes the fastest fusable configuration
+        // class 0 is unconstrained; the others accept kernels that fit their share of the device and, under the executors
+        // that put the operators of a stage into one launch, can run inside a fused stage launch (the stream and graph
+        // executors launch every operator by itself, so every configuration competes); a budget nobody fits takes the
+        // fastest such configuration
+        const bool any_kernel = !fused_executor();
         auto eligible = [&](const Candidate &cand, bool fit) {
             if (c == 0) return true;
-            return cand.fusable && (!fit || cand.footprint <= capacity / (1 << c));
+            return (cand.fusable || any_kernel) && (!fit || cand.footprint <= capacity / (1 << c));
         };
         found[c] = false;
         if (c > 0 && share_cost_rule_) {
@@ -304,7 +308,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
             auto score = [&](const Candidate &cand) { return cand.ms * (1.0 + ((1 << c) - 1) * cand.footprint / capacity); };
             std::vector<size_t> order;
             for (size_t i = 0; i < candidates.size(); i++)
-                if (candidates[i].fusable) order.push_back(i);
+                if (candidates[i].fusable || any_kernel) order.push_back(i);
             std::sort(order.begin(), order.end(), [&](size_t a, size_t b) { return score(candidates[a]) < score(candidates[b]); });
             double best = 1e300;
             for (size_t n = 0; n < order.size() && n < 3; n++) {
