@@ -58,7 +58,14 @@ PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorV
         if ((p.sw == 1 || p.sw == 2) && p.pw <= 1 && p.W >= 8) {
             const long long kVecMinThreads = 1LL << 16;   // measured: 2^16 beats the one-column form from 64x147x147 at batch 1 on, 2^14 loses
             auto quads = [&](int r) { return (long long)p.B * p.C * ((p.OH + r - 1) / r) * ((p.OW + kPoolVecColumns - 1) / kPoolVecColumns); };
+            // Tensors that give half a million threads even with the shortest strips (batch 16 and more) are bound by how many
+            // loads the device has in flight, not by the rows neighbouring strips read twice: one output row per thread for
+            // stride 2, two for stride 1 (batch 64, launched back to back: 64x147x147 stride 2 101.9 -> 89.7 us = 4.9 TB/s,
+            // 192x71x71 87.5 -> 77.3, 288x35x35 26.8 -> 22.3, 768x17x17 17.8 -> 15.9; stride 1 on 32x35x35 9.2 -> 7.5,
+            // 192x17x17 10.8 -> 9.7 us; longer strips there are 5-15 % slower, one column per thread 30-60 %)
+            const long long kShortStripThreads = 1LL << 19;
             int vrows = kPoolStripRows;
+            if (quads(1) >= kShortStripThreads) vrows = p.sh == 2 ? 1 : 2;
             while (vrows > 1 && quads(vrows) < kVecMinThreads) vrows >>= 1;
             if (quads(vrows) >= kVecMinThreads) {
                 a.vec_columns = kPoolVecColumns;
