@@ -94,7 +94,9 @@ const char *ios_last_error(void);
 /* Options (set them before sessions are created):
  *   "executor" = "fused" (default: the groups of a stage share one kernel launch per level) | "fused_graph" (fused
  *       launches inside a hipGraph) | "streams" (one HIP stream per group, event fork/join) | "graph" (the stream form
- *       captured into a hipGraph and replayed);
+ *       captured into a hipGraph and replayed).  The fused forms are the fast ones at small batches; from batch 16 on
+ *       the stream forms can be ahead, because every convolution kernel configuration may serve a parallel stage there,
+ *       also those too heavy on registers to share a fused launch;
  *   "autotune" = "1" (default) | "0": measure convolution kernel configurations on first use, like the reference's
  *       cudnnFind-based selection (src/ios/ios_runtime.cu:150-205); "clear_tuning" = anything forgets them;
  *   "split_k_reduce" = "xcd" (default: the last block of a tile adds the split-K slices inside the convolution kernel,
@@ -111,6 +113,10 @@ const char *ios_last_error(void);
  *       last stage that touches them) do not intersect share device memory; the network input and the result never do.
  *       The reference allocates every output for the lifetime of the graph (src/ios/ios_runtime.cu:1273-1285, 1318-1327).
  *       With "0" every operator output survives the pass (ios_session_get_tensor on any node); needs no device;
+ *   "commute_pool_conv" = "1" (default) | "0": an average pool that keeps the map size and the 1 x 1 convolution to no more
+ *       channels that alone reads it change places: the convolution runs first without bias and activation, the pool
+ *       then works on the convolution's channels and finishes with bias and activation (same result up to the order of
+ *       fp32 roundings; the pool operator has no tensor of its own any more); needs no device;
  *   "thin_conv_min_pixels" = count (default 262144; negative: never): a 3 x 3 convolution of a 3-channel image with at least
  *       this many output pixels (batch x OH x OW) that has its stage to itself runs on a direct kernel bound by the bytes of
  *       its output instead of the matrix path (first layers at large batches); needs no device;
