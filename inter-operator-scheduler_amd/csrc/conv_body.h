@@ -617,9 +617,20 @@ __device__ __forceinline__ void split_bf16x3(const float (&x)[8], uintx4 &hi, ui
     }
 }
 
+// eight fp32 values rounded to bfloat16 (nearest even), as four words of two (lower k in the lower half)
+typedef float floatx8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ uintx4 round_bf16x8(const float (&x)[8]) {
+    const floatx8 v = {x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]};
+    return __builtin_bit_cast(uintx4, __builtin_convertvector(v, bf16x8));
+}
+
 // TMW x TNW MFMA tiles of 32 x 32 per wavefront, WM x WN wavefronts per block
-template <int TMW, int TNW, int WM, int WN, int PD>
+// TERMS = 3: fp32 accuracy as described above.  TERMS = 1: the reduced-precision mode with bfloat16 operands (inputs and
+// filters rounded to nearest even, fp32 accumulation): one plane, one matrix instruction per tile and K tile, a sixth of the
+// matrix work and a third of the LDS traffic.
+template <int TMW, int TNW, int WM, int WN, int PD, int TERMS = 3>
 struct ConvSplit3 {
+    static_assert(TERMS == 3 || TERMS == 1, "three exact terms or one rounded term");
     static constexpr int MT = 32, BK = 16;
     using M = Mfma<32>;
     static constexpr int BM = 32 * TMW * WM, BN = 32 * TNW * WN;
@@ -628,8 +639,8 @@ struct ConvSplit3 {
     static constexpr int THREADS = T;
     static constexpr int CPAD = BK;
     static constexpr bool FUSABLE = false;
-    // LDS in slots of 16 bytes (eight bfloat16): per stage the input planes [3][2][BN]
-    static constexpr int STAGE = 6 * BN;
+    // LDS in slots of 16 bytes (eight bfloat16): per stage the input planes [TERMS][2][BN]
+    static constexpr int STAGE = 2 * TERMS * BN;
     static constexpr int SMEM_FLOATS = 2 * STAGE * 4;
     static constexpr int B_OCT = 2 * BN;
     static constexpr int B_IT = (B_OCT + T - 1) / T;                   // octets a thread stages per K tile
@@ -664,7 +675,7 @@ struct ConvSplit3 {
     for (int i = 0; i < TM; i++) {
         const int m = m0 + wm * WTM + i * MT + lc;
         // packed filters: [g][k / 8][plane][OCgP] slots of 16 bytes
-        a_off[i] = m < a.OCgP ? (unsigned)(((((size_t)g * (a.Kq >> 3) + lk) * 3) * a.OCgP + m) * 16) : kOutOfRange;
+        a_off[i] = m < a.OCgP ? (unsigned)(((((size_t)g * (a.Kq >> 3) + lk) * TERMS) * a.OCgP + m) * 16) : kOutOfRange;
     }
     const unsigned a_plane = (unsigned)a.OCgP * 16u;
     // ---- inputs: this thread's pixel and octets ----------------------------------------------------------------------------
@@ -688,18 +699,18 @@ struct ConvSplit3 {
     for (int i = 0; i < B_IT; i++) b_oct[i] = (tid + i * T) / BN;
     const unsigned b_surplus = B_OCT % T == 0 || tid < B_OCT ? 0u : kOutOfRange;   // (more threads than octets: the surplus stages nothing)
 
-    uintx4 a_reg[PD][3][TM];
+    uintx4 a_reg[PD][TERMS][TM];
     float b_reg[PD][B_IT][8];
-    auto load_tile = [&](int kt, uintx4 (&ar)[3][TM], float (&br)[B_IT][8]) {
+    auto load_tile = [&](int kt, uintx4 (&ar)[TERMS][TM], float (&br)[B_IT][8]) {
         const int k0 = k_begin + kt * BK;
         const int tap = (int)__umulhi((unsigned)k0, a.magic_icgp);
         const int c0 = k0 - tap * a.ICgP;
         const int kh = a.KW == 1 ? tap : (int)__umulhi((unsigned)tap, a.magic_kw);
         const int kw = tap - kh * a.KW;
         const unsigned tile_kill = kt < nkt ? 0u : kOutOfRange;   // tiles past the end of the K range load zeros
-        const unsigned w_tile = (unsigned)((k0 >> 3) * 3 * a.OCgP) * 16u;
+        const unsigned w_tile = (unsigned)((k0 >> 3) * TERMS * a.OCgP) * 16u;
 #pragma unroll
-        for (int p = 0; p < 3; p++)
+        for (int p = 0; p < TERMS; p++)
 #pragma unroll
             for (int i = 0; i < TM; i++) ar[p][i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (a_off[i] + w_tile) | tile_kill, (unsigned)p * a_plane, 0);
         const unsigned in_h = (unsigned)(ih0 + kh) < (unsigned)a.H ? 1u : 0u;
@@ -725,11 +736,15 @@ struct ConvSplit3 {
             float v[8];
 #pragma unroll
             for (int j = 0; j < 8; j++) v[j] = __int_as_float(max(__float_as_int(br[i][j]), relu_floor));   // folded ReLU of the producer
-            uintx4 hi, mid, lo;
-            split_bf16x3(v, hi, mid, lo);
-            stage[(0 + b_oct[i]) * BN + pix] = hi;
-            stage[(2 + b_oct[i]) * BN + pix] = mid;
-            stage[(4 + b_oct[i]) * BN + pix] = lo;
+            if constexpr (TERMS == 3) {
+                uintx4 hi, mid, lo;
+                split_bf16x3(v, hi, mid, lo);
+                stage[(0 + b_oct[i]) * BN + pix] = hi;
+                stage[(2 + b_oct[i]) * BN + pix] = mid;
+                stage[(4 + b_oct[i]) * BN + pix] = lo;
+            } else {
+                stage[b_oct[i] * BN + pix] = round_bf16x8(v);
+            }
         }
     };
 
@@ -755,9 +770,9 @@ struct ConvSplit3 {
             const int kt = kt0 + s;
             const int buf = kt & 1;
             const uintx4 *Bb = lds + buf * STAGE + lk * BN + wn * WTN + lc;
-            bf16x8 av[3][TM], bv[3][TN];
+            bf16x8 av[TERMS][TM], bv[TERMS][TN];
 #pragma unroll
-            for (int p = 0; p < 3; p++) {
+            for (int p = 0; p < TERMS; p++) {
 #pragma unroll
                 for (int i = 0; i < TM; i++) av[p][i] = __builtin_bit_cast(bf16x8, a_reg[s][p][i]);
 #pragma unroll
@@ -767,9 +782,10 @@ struct ConvSplit3 {
             // requests each operand right in front of its first use and the wavefront pays the LDS latency once per plane)
             __builtin_amdgcn_sched_barrier(0);
             // the six terms, smallest first; the tiles of a term are independent instructions
-            constexpr int TA[6] = {2, 0, 1, 1, 0, 0}, TB[6] = {0, 2, 1, 0, 1, 0};
+            constexpr int NT = TERMS == 3 ? 6 : 1;
+            constexpr int TA[6] = {TERMS == 3 ? 2 : 0, 0, 1, 1, 0, 0}, TB[6] = {0, 2, 1, 0, 1, 0};
 #pragma unroll
-            for (int t = 0; t < 6; t++)
+            for (int t = 0; t < NT; t++)
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -845,13 +861,16 @@ struct ConvWsplit {
     static constexpr bool KQUAD = QUAD;                    // packed filters are [k / 4][m][4] instead of [k][m]
     // accumulators + staged operands per lane decide whether the body fits the register budget of a fused launch
     // (the channel-padding-4 forms serve first layers, which are stages of their own: kept out of the fused launches)
-    static constexpr bool FUSABLE = RP != 3 && CP == 0 && E + D * U * (TM + TN) <= (QUAD ? (MT == 32 ? 48 : 56) : 48);   // per-step addressing of the plain layout needs more registers, and so do the 16-register accumulator tuples of the 32 x 32 tiles
-    static constexpr int KREDUCED = RP;                    // 0: fp32 filters; 1: packed filters hold bfloat16; 2: IEEE half; 3: three bfloat16 planes
+    static constexpr bool FUSABLE = RP < 3 && CP == 0 && E + D * U * (TM + TN) <= (QUAD ? (MT == 32 ? 48 : 56) : 48);   // per-step addressing of the plain layout needs more registers, and so do the 16-register accumulator tuples of the 32 x 32 tiles
+    static constexpr int KREDUCED = RP;                    // 0: fp32 filters; 1: packed filters hold bfloat16; 2: IEEE half; 3: three bfloat16 planes; 4: one
+    static constexpr int PLANES = RP == 3 ? 3 : 1;
+    // RP == 4: the reduced-precision mode on the same instruction and layout: one plane of filters rounded to bfloat16, inputs
+    // rounded after the load, one matrix instruction per tile and batch.
     // RP == 3: fp32 results from the bfloat16 matrix pipe, as in ConvSplit3 (operands split exactly into three bfloat16 terms,
     // six of the nine partial products on v_mfma_f32_32x32x16_bf16): filters are split when packed, [k / 8][plane][m][8], and read
     // as operands straight from global memory; a lane splits the eight input values it loads for a batch itself.
     static_assert(!QUAD || U % 4 == 0, "quad loads need whole groups of four k per lane");
-    static_assert(RP >= 0 && RP <= 3 && (RP == 0 || (RP == 3 ? QUAD && MT == 32 && U == 8 : QUAD && MT == 16 && U == 4)),
+    static_assert(RP >= 0 && RP <= 4 && (RP == 0 || (RP >= 3 ? QUAD && MT == 32 && U == 8 : QUAD && MT == 16 && U == 4)),
                   "the 16-bit paths are the 16 x 16 x 16 form of the quad layout, the three-term path its 32 x 32 x 16 form");
 
     template <bool RES = false>
@@ -901,8 +920,8 @@ struct ConvWsplit {
     for (int i = 0; i < TM; i++) {
         w_kill[i] = m0 + i * MT + lc < a.OCgP ? 0u : kOutOfRange;
         // byte offsets below 2^31 (checked on the host)
-        if (RP == 3)   // [g][k / 8][plane][m] slots of 16 bytes: this lane's octet of a batch is lk
-            w_lane[i] = ((((unsigned)g * ((unsigned)a.Kq >> 3) + (unsigned)lk) * 3u) * (unsigned)a.OCgP + (unsigned)(m0 + i * MT + lc)) * 16u;
+        if (RP >= 3)   // [g][k / 8][plane][m] slots of 16 bytes: this lane's octet of a batch is lk
+            w_lane[i] = ((((unsigned)g * ((unsigned)a.Kq >> 3) + (unsigned)lk) * (unsigned)PLANES) * (unsigned)a.OCgP + (unsigned)(m0 + i * MT + lc)) * 16u;
         else if (QUAD)   // [g][k / 4][m][4]: this lane's first quad of a batch is row (U / 4) * lk
             w_lane[i] = (((unsigned)g * ((unsigned)a.Kq >> 2) + (unsigned)((U / 4) * lk)) * (unsigned)a.OCgP + (unsigned)(m0 + i * MT + lc)) * (RP != 0 ? 8u : 16u);
         else
@@ -936,9 +955,9 @@ struct ConvWsplit {
         uintx2 v[TM];
     };
     struct FilterStageX3 {
-        uintx4 v[3][TM];
+        uintx4 v[PLANES][TM];
     };
-    using FilterStage = std::conditional_t<(RP == 3), FilterStageX3, std::conditional_t<(RP != 0), FilterStageBf16, FilterStageF32>>;
+    using FilterStage = std::conditional_t<(RP >= 3), FilterStageX3, std::conditional_t<(RP != 0), FilterStageBf16, FilterStageF32>>;
     FilterStage av[D];
     float bv[D][U][TN];
 
@@ -954,7 +973,7 @@ struct ConvWsplit {
         q_cb = kb - tap * a.ICgP;
         q_kh = a.KW == 1 ? tap : (int)__umulhi((unsigned)tap, a.magic_kw);
         q_kw = tap - q_kh * a.KW;
-        q_w = RP == 3 ? (unsigned)((kb / 8) * 3 * a.OCgP) * 16u : (unsigned)((kb / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
+        q_w = RP >= 3 ? (unsigned)((kb / 8) * PLANES * a.OCgP) * 16u : (unsigned)((kb / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
     }
     // `live` (wavefront-uniform) is false for a batch beyond the wavefront's K range: its loads are still issued, against
     // descriptors of extent zero, and return zeros without touching memory.  Loads are never skipped by a branch inside
@@ -972,9 +991,9 @@ struct ConvWsplit {
             (void)s0;
             const __amdgpu_buffer_rsrc_t xr = buffer_of(a.x, live ? a.x_bytes : 0u);
             const __amdgpu_buffer_rsrc_t wr = buffer_of(a.wp, live ? a.w_bytes : 0u);
-            if constexpr (RP == 3) {
+            if constexpr (RP >= 3) {
 #pragma unroll
-                for (int p = 0; p < 3; p++)
+                for (int p = 0; p < PLANES; p++)
 #pragma unroll
                     for (int i = 0; i < TM; i++)   // eight bfloat16 = the lane's eight k of this batch, one plane
                         A.v[p][i] = __builtin_amdgcn_raw_buffer_load_b128(wr, w_lane[i] | w_kill[i], q_w + (unsigned)(p * a.OCgP) * 16u, 0);
@@ -1022,7 +1041,7 @@ struct ConvWsplit {
                     for (int j = 0; j < TN; j++) B[u][j] = buffer_load_f32(xr, voff[j], x_chan + (unsigned)(u * a.HW) * 4u);
             }
             // next batch (selects, not branches: the loop body stays one basic block)
-            q_w += RP == 3 ? (unsigned)((U * M::KSTEP / 8) * 3 * a.OCgP) * 16u : (unsigned)((U * M::KSTEP / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
+            q_w += RP >= 3 ? (unsigned)((U * M::KSTEP / 8) * PLANES * a.OCgP) * 16u : (unsigned)((U * M::KSTEP / 4) * a.OCgP) * (RP != 0 ? 8u : 16u);
             q_cb += U * M::KSTEP;
             const bool next_tap = q_cb >= a.ICgP;
             q_cb = next_tap ? 0 : q_cb;
@@ -1081,6 +1100,19 @@ struct ConvWsplit {
 #pragma unroll
                     for (int j = 0; j < TN; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A.v[TA[t]][i]), bq[TB[t]][j], acc[i][j], 0, 0, 0);
+            return;
+        } else if constexpr (RP == 4) {
+            // one rounded term: the reduced-precision mode on the 32 x 32 x 16 instruction
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = __int_as_float(max(__float_as_int(B[u][j]), relu_floor));
+                const bf16x8 bq = __builtin_bit_cast(bf16x8, round_bf16x8(v));
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A.v[0][i]), bq, acc[i][j], 0, 0, 0);
+            }
             return;
         } else if constexpr (RP != 0) {
 #pragma unroll
@@ -1386,6 +1418,22 @@ struct ConvWsplit {
     X(104, "x3w_m32n64_w8", 1, 2, 8, 2)      \
     X(105, "x3w_m64n64_w4", 2, 2, 4, 2)      \
     X(106, "x3w_m64n32_w2", 2, 1, 2, 2)
-constexpr int kNumConvVariants = 107;
+// X(index, name, TMW, TNW, WM, WN, PD): ConvSplit3 with one rounded term (option precision=bf16), up to 64 x 64 per wavefront
+#define IOS_SPLIT1_VARIANTS(X)                      \
+    X(107, "wb_x1_m64n128_w2x2", 1, 2, 2, 2, 2)     \
+    X(108, "wb_x1_m128n128_w2x2", 2, 2, 2, 2, 2)    \
+    X(109, "wb_x1_m128n256_w2x4", 2, 2, 2, 4, 2)    \
+    X(110, "wb_x1_m64n128_w1x2", 2, 2, 1, 2, 2)     \
+    X(111, "wb_x1_m128n64_w4x1", 1, 2, 4, 1, 2)     \
+    X(112, "wb_x1_m64n256_w2x4", 1, 2, 2, 4, 2)
+// X(index, name, TM, TN, NW, D): the wave-split kernel with one rounded term (ConvWsplit, RP = 4)
+#define IOS_WSPLIT_X1_VARIANTS(X)              \
+    X(113, "wb_x1w_m32n32_w4", 1, 1, 4, 2)     \
+    X(114, "wb_x1w_m64n32_w4", 2, 1, 4, 2)     \
+    X(115, "wb_x1w_m32n64_w4", 1, 2, 4, 2)     \
+    X(116, "wb_x1w_m64n64_w4", 2, 2, 4, 2)     \
+    X(117, "wb_x1w_m32n32_w8", 1, 1, 8, 2)     \
+    X(118, "wb_x1w_m64n64_w2", 2, 2, 2, 2)
+constexpr int kNumConvVariants = 119;
 
 }  // namespace ios

@@ -51,19 +51,31 @@ struct VariantEntry {
 
 #define IOS_SPLIT3_ENTRY(IDX, NAME, TMW, TNW, WM, WN, PD)                                                                              \
     {{NAME, ConvSplit3<TMW, TNW, WM, WN, PD>::BM, ConvSplit3<TMW, TNW, WM, WN, PD>::BN, 16, WM, WN, 1, 32, false,                         \
-      ConvSplit3<TMW, TNW, WM, WN, PD>::CPAD, false, false, PREC_FP32, 1},                                                                \
+      ConvSplit3<TMW, TNW, WM, WN, PD>::CPAD, false, false, PREC_FP32, 3},                                                                \
      conv_kernel<ConvSplit3<TMW, TNW, WM, WN, PD>>, conv_kernel<ConvSplit3<TMW, TNW, WM, WN, PD>, true>,                                  \
      ConvSplit3<TMW, TNW, WM, WN, PD>::SMEM_FLOATS},
 
 #define IOS_WSPLIT_X3_ENTRY(IDX, NAME, TM, TN, NW, D)                                                                        \
-    {{NAME, TM * 32, TN * 32, 16, 1, 1, NW, 32, true, ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::CPAD, true, false, PREC_FP32, 1},      \
+    {{NAME, TM * 32, TN * 32, 16, 1, 1, NW, 32, true, ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::CPAD, true, false, PREC_FP32, 3},      \
      conv_kernel<ConvWsplit<32, TM, TN, NW, 8, true, D, 3>>, conv_kernel<ConvWsplit<32, TM, TN, NW, 8, true, D, 3>, true>,              \
      ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::SMEM_FLOATS},
+
+#define IOS_SPLIT1_ENTRY(IDX, NAME, TMW, TNW, WM, WN, PD)                                                                              \
+    {{NAME, ConvSplit3<TMW, TNW, WM, WN, PD, 1>::BM, ConvSplit3<TMW, TNW, WM, WN, PD, 1>::BN, 16, WM, WN, 1, 32, false,                   \
+      ConvSplit3<TMW, TNW, WM, WN, PD, 1>::CPAD, false, false, PREC_BF16, 1},                                                             \
+     conv_kernel<ConvSplit3<TMW, TNW, WM, WN, PD, 1>>, conv_kernel<ConvSplit3<TMW, TNW, WM, WN, PD, 1>, true>,                            \
+     ConvSplit3<TMW, TNW, WM, WN, PD, 1>::SMEM_FLOATS},
+
+#define IOS_WSPLIT_X1_ENTRY(IDX, NAME, TM, TN, NW, D)                                                                        \
+    {{NAME, TM * 32, TN * 32, 16, 1, 1, NW, 32, true, ConvWsplit<32, TM, TN, NW, 8, true, D, 4>::CPAD, true, false, PREC_BF16, 1},      \
+     conv_kernel<ConvWsplit<32, TM, TN, NW, 8, true, D, 4>>, conv_kernel<ConvWsplit<32, TM, TN, NW, 8, true, D, 4>, true>,              \
+     ConvWsplit<32, TM, TN, NW, 8, true, D, 4>::SMEM_FLOATS},
 
 static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)
                                              IOS_WSPLIT_C4_VARIANTS(IOS_WSPLIT_C4_ENTRY)
                                              IOS_WSPLIT_T32_VARIANTS(IOS_WSPLIT_ENTRY) IOS_WSPLIT_F16_VARIANTS(IOS_WSPLIT_ENTRY)
-                                             IOS_WSPLIT_LONGK_VARIANTS(IOS_WSPLIT_ENTRY) IOS_SPLIT3_VARIANTS(IOS_SPLIT3_ENTRY) IOS_WSPLIT_X3_VARIANTS(IOS_WSPLIT_X3_ENTRY)};
+                                             IOS_WSPLIT_LONGK_VARIANTS(IOS_WSPLIT_ENTRY) IOS_SPLIT3_VARIANTS(IOS_SPLIT3_ENTRY) IOS_WSPLIT_X3_VARIANTS(IOS_WSPLIT_X3_ENTRY)
+                                             IOS_SPLIT1_VARIANTS(IOS_SPLIT1_ENTRY) IOS_WSPLIT_X1_VARIANTS(IOS_WSPLIT_X1_ENTRY)};
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 static_assert(kNumVariants == kNumConvVariants, "variant lists and count disagree");
 
@@ -215,7 +227,7 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     a.HW = p.H * p.W; a.OHW = p.OH * p.OW; a.groups = p.groups;
     a.x_bs = x.bstride; a.y_bs = y.bstride;
     const unsigned long long x_bytes = ((unsigned long long)(p.B - 1) * x.bstride + (unsigned long long)p.IC * p.H * p.W) * 4ull;
-    const unsigned long long w_bytes = (unsigned long long)p.groups * p.Kq(e.v.cpad) * p.OCgP() * (e.v.koct ? 6ull : e.v.precision != PREC_FP32 ? 2ull : 4ull);
+    const unsigned long long w_bytes = (unsigned long long)p.groups * p.Kq(e.v.cpad) * p.OCgP() * (e.v.koct ? 2ull * e.v.koct : e.v.precision != PREC_FP32 ? 2ull : 4ull);
     if (x_bytes >= (1ull << 31) || w_bytes >= (1ull << 31)) throw std::runtime_error("conv: tensor too large for 31-bit buffer offsets");
     a.x_bytes = (unsigned)x_bytes;
     a.w_bytes = (unsigned)w_bytes;
@@ -317,10 +329,11 @@ void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorVie
 
 // ---- filter packing ------------------------------------------------------------------------
 __global__ void pack_filters_kernel(const float *w, float *packed, int OCg, int OCgP, int ICg, int ICgP, int taps, int groups, int kvec,
-                                    int precision) {
+                                    int precision, int planes) {
     // packed[g][k][m] = w[g * OCg + m][c][tap] with k = tap * ICgP + c;  rows with c >= ICg and columns with m >= OCg are zero.
     // kvec = 4: packed[g][k / 4][m][k % 4] instead (ICgP is a multiple of 4)
-    // kvec = 8: three planes of bfloat16, packed[g][k / 8][plane][m][k % 8], the exact three-term split of every filter value
+    // kvec = 8: planes of bfloat16, packed[g][k / 8][plane][m][k % 8]: three planes with the exact three-term split of every filter
+    // value, or one plane with the value rounded to nearest even (the reduced-precision mode)
     const size_t total = (size_t)groups * taps * ICgP * OCgP;
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         int m;
@@ -339,14 +352,18 @@ __global__ void pack_filters_kernel(const float *w, float *packed, int OCg, int 
         const int g = (int)(gt / taps);
         const float value = (m < OCg && c < ICg) ? w[(((size_t)g * OCg + m) * ICg + c) * taps + tap] : 0.f;
         if (kvec == 8) {
-            unsigned hi, mid, lo;
-            split3(value, hi, mid, lo);
-            unsigned short *planes = reinterpret_cast<unsigned short *>(packed);
             const size_t octet = gk / 8;                         // (g, k / 8)
-            const size_t at = (octet * 3 * OCgP + m) * 8 + (gk % 8);
-            planes[at] = (unsigned short)(hi >> 16);
-            planes[at + (size_t)OCgP * 8] = (unsigned short)(mid >> 16);
-            planes[at + (size_t)OCgP * 16] = (unsigned short)(lo >> 16);
+            const size_t at = (octet * planes * OCgP + m) * 8 + (gk % 8);
+            if (planes == 3) {
+                unsigned hi, mid, lo;
+                split3(value, hi, mid, lo);
+                unsigned short *out = reinterpret_cast<unsigned short *>(packed);
+                out[at] = (unsigned short)(hi >> 16);
+                out[at + (size_t)OCgP * 8] = (unsigned short)(mid >> 16);
+                out[at + (size_t)OCgP * 16] = (unsigned short)(lo >> 16);
+            } else {
+                reinterpret_cast<__bf16 *>(packed)[at] = (__bf16)value;   // round to nearest even
+            }
         } else if (precision == PREC_BF16) reinterpret_cast<__bf16 *>(packed)[i] = (__bf16)value;   // round to nearest even
         else if (precision == PREC_FP16) reinterpret_cast<_Float16 *>(packed)[i] = (_Float16)value;   // round to nearest even
         else packed[i] = value;
@@ -356,7 +373,7 @@ __global__ void pack_filters_kernel(const float *w, float *packed, int OCg, int 
 size_t conv_packed_floats(const ConvProblem &p, const ConvLaunch &l) {
     if (l.variant < 0 || l.variant >= kNumVariants) throw std::runtime_error("conv: bad variant");
     const size_t elements = (size_t)p.groups * p.Kq(kVariants[l.variant].v.cpad) * p.OCgP();
-    if (kVariants[l.variant].v.koct) return elements + (elements + 1) / 2;   // three planes of bfloat16
+    if (kVariants[l.variant].v.koct) return (elements * kVariants[l.variant].v.koct + 1) / 2;   // planes of bfloat16
     return kVariants[l.variant].v.precision != PREC_FP32 ? (elements + 1) / 2 : elements;
 }
 
@@ -364,7 +381,7 @@ size_t conv_packed_floats_max(const ConvProblem &p) {
     size_t most = 0;
     for (const VariantEntry &e : kVariants) {
         const size_t elements = (size_t)p.groups * p.Kq(e.v.cpad) * p.OCgP();
-        most = std::max(most, e.v.koct ? elements + (elements + 1) / 2 : elements);
+        most = std::max(most, e.v.koct ? (elements * e.v.koct + 1) / 2 : elements);
     }
     return most;
 }
@@ -374,7 +391,7 @@ void launch_pack_filters(const ConvProblem &p, const ConvLaunch &l, const float 
     const size_t total = (size_t)p.groups * p.Kq(cpad) * p.OCgP();   // elements
     const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 65535);
     hipLaunchKernelGGL(pack_filters_kernel, dim3(blocks), dim3(256), 0, stream, w, packed, p.OCg(), p.OCgP(), p.ICg(), p.ICgP(cpad),
-                       p.KH * p.KW, p.groups, kVariants[l.variant].v.kvec(), kVariants[l.variant].v.precision);
+                       p.KH * p.KW, p.groups, kVariants[l.variant].v.kvec(), kVariants[l.variant].v.precision, kVariants[l.variant].v.koct);
 }
 
 }  // namespace ios

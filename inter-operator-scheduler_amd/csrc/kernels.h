@@ -53,7 +53,9 @@ struct ConvVariant {
     int threads() const { return 64 * WM * WN * WK; }
     bool fusable_;   // light enough on registers to run inside a fused stage launch
     int precision;   // PREC_FP32, or a reduced-precision mode: bfloat16 / IEEE half filters and inputs, fp32 accumulation
-    int koct = 0;    // 1: packed filters are three planes of bfloat16, [k / 8][plane][m][8] (the kernel that splits fp32 operands into three bfloat16 terms)
+    // packed filters as planes of bfloat16, [k / 8][plane][m][8]: 3 = the exact three-term split of fp32 values (fp32 results from
+    // the bfloat16 matrix pipe), 1 = one plane rounded to nearest even (the reduced-precision mode on the same kernels), 0 = neither
+    int koct = 0;
     bool fusable() const { return fusable_; }
     int kvec() const { return koct ? 8 : kquad ? 4 : 1; }   // consecutive k of one output channel that lie together
 };
