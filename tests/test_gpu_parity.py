@@ -320,6 +320,73 @@ POOLS = [
 ]
 
 
+COMMUTED = [
+    # in_shape, out_channels, act, pool kernel / stride / padding, batch, executor: average pools that keep the map size in
+    # front of a 1 x 1 convolution to no more channels (every pool body: one column, four columns, generic window)
+    ((48, 17, 17), 24, 'relu', (3, 3), (1, 1), (1, 1), 3, 'streams'),
+    ((64, 35, 35), 64, 'identity', (3, 3), (1, 1), (1, 1), 16, 'fused'),        # four output columns per thread
+    ((20, 9, 11), 7, 'tanh', (5, 5), (1, 1), (2, 2), 2, 'streams'),              # generic window, odd channel count
+    ((96, 8, 8), 32, 'sigmoid', (3, 3), (1, 1), (1, 1), 1, 'fused_graph'),
+]
+
+
+@pytest.mark.parametrize('case', COMMUTED, ids=[f'{c[0][0]}x{c[0][1]}x{c[0][2]}-{c[1]}-{c[2]}' for c in COMMUTED])
+def test_average_pool_exchanged_with_its_pointwise_convolution_matches_oracle(case):
+    """
+    y = act(W * avgpool(x) + b) computed as act(avgpool(W * x) + b): the border elements, where the window counts padding
+    (the divisor stays KH * KW, reference src/ios/ios_runtime.cu:542-550), bias and activation included.  A second reader of
+    the pool, a max pool, a pool that changes the map size and a 3 x 3 convolution keep the reference's order.
+    """
+    in_shape, oc, act, kernel, stride, padding, batch, executor = case
+
+    def build(b, v):
+        pooled = ios.pool2d(b, [[v]], 'avg', kernel, stride, padding)
+        ios.conv2d(b, [[pooled]], oc, (1, 1), (1, 1), (0, 0), 1, act, is_exit=True)
+
+    graph = single_op_graph(in_shape, build)
+    rt.set_option('executor', executor)
+    try:
+        ops = rt.plan_describe(graph, batch)
+        assert [bool(op.get('linear')) for op in ops] == [True, False] and ops[1]['kind'] == 'pool' and 'adds_bias_of' in ops[1]
+        got, want = run_both(graph, batch)
+        assert_close(got, want, f'exchanged pool {case}')
+        # border rows and columns on their own: a wrong divisor or a bias added before the pool shows there first
+        for border in (got[:, :, 0, :] - want[:, :, 0, :], got[:, :, :, -1] - want[:, :, :, -1]):
+            assert np.abs(border).max() <= 1e-4 + 1e-3 * np.abs(want).max()
+        rt.set_option('commute_pool_conv', 0)
+        plain = rt.graph_inference(graph, batch, np.random.default_rng(1).standard_normal((batch, *in_shape)).astype(np.float32))
+        assert_close(plain, want, f'reference order {case}')
+        assert not any(op.get('linear') for op in rt.plan_describe(graph, batch))
+    finally:
+        rt.set_option('commute_pool_conv', 1)
+        rt.set_option('executor', 'streams')
+
+
+def test_pools_that_must_keep_their_place():
+    def two_readers(b, v):
+        pooled = ios.pool2d(b, [[v]], 'avg', (3, 3), (1, 1), (1, 1))
+        c = ios.conv2d(b, [[pooled]], 16, (1, 1), (1, 1), (0, 0), 1, 'relu')
+        ios.identity(b, [[c], [pooled]], is_exit=True)
+
+    def max_pool(b, v):
+        ios.conv2d(b, [[ios.pool2d(b, [[v]], 'max', (3, 3), (1, 1), (1, 1))]], 16, (1, 1), (1, 1), (0, 0), 1, 'relu', is_exit=True)
+
+    def shrinking(b, v):
+        ios.conv2d(b, [[ios.pool2d(b, [[v]], 'avg', (3, 3), (2, 2), (1, 1))]], 16, (1, 1), (1, 1), (0, 0), 1, 'relu', is_exit=True)
+
+    def wide_window(b, v):
+        ios.conv2d(b, [[ios.pool2d(b, [[v]], 'avg', (3, 3), (1, 1), (1, 1))]], 16, (3, 3), (1, 1), (1, 1), 1, 'relu', is_exit=True)
+
+    def more_channels(b, v):
+        ios.conv2d(b, [[ios.pool2d(b, [[v]], 'avg', (3, 3), (1, 1), (1, 1))]], 64, (1, 1), (1, 1), (0, 0), 1, 'relu', is_exit=True)
+
+    for build in (two_readers, max_pool, shrinking, wide_window, more_channels):
+        graph = single_op_graph((24, 14, 14), build)
+        assert not any(op.get('linear') for op in rt.plan_describe(graph, 2)), build.__name__
+        got, want = run_both(graph, 2)
+        assert_close(got, want, build.__name__)
+
+
 @pytest.mark.parametrize('case', POOLS)
 def test_pool_matches_oracle(case):
     in_shape, kind, k, s, p, batch = case
