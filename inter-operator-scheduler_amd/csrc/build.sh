@@ -12,7 +12,7 @@ FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclan
 # two forms spill or slow the memory-bound bodies down with it (NASNet +0.8 %), so they keep the default.
 declare -A FILE_FLAGS=([conv_mfma.hip]="-mllvm -amdgpu-sched-strategy=max-ilp" [fused_512.hip]="-mllvm -amdgpu-sched-strategy=max-ilp")
 pids=()
-for src in conv_mfma.hip pointwise.hip fused.hip fused_512.hip runtime.hip c_api.hip; do
+for src in conv_mfma.hip pointwise.hip fused.hip fused_512.hip fused_wide.hip runtime.hip c_api.hip; do
     # the resource remarks go to a log: a kernel that spills registers to scratch memory is reported below
     hipcc $FLAGS ${FILE_FLAGS[$src]:-} -Rpass-analysis=kernel-resource-usage -c "$src" -o "build/${src%.hip}.o" 2> "build/${src%.hip}.log" &
     pids+=($!)
@@ -29,5 +29,5 @@ if grep -h "ScratchSize \[bytes/lane\]: [1-9]" build/*.log > /dev/null; then
     echo "warning: kernels spilling to scratch memory:" >&2
     grep -h -B4 "ScratchSize \[bytes/lane\]: [1-9]" build/*.log | grep "Function Name" | sed 's/.*Function Name: /  /; s/ \[-R.*//' >&2
 fi
-hipcc --offload-arch=gfx950 -shared -fPIC -o build/libios_runtime.so build/conv_mfma.o build/pointwise.o build/fused.o build/fused_512.o build/runtime.o build/c_api.o build/plan.o
+hipcc --offload-arch=gfx950 -shared -fPIC -o build/libios_runtime.so build/conv_mfma.o build/pointwise.o build/fused.o build/fused_512.o build/fused_wide.o build/runtime.o build/c_api.o build/plan.o
 echo "built $(pwd)/build/libios_runtime.so"

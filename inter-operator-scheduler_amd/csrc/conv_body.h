@@ -862,6 +862,9 @@ struct ConvWsplit {
     // accumulators + staged operands per lane decide whether the body fits the register budget of a fused launch
     // (the channel-padding-4 forms serve first layers, which are stages of their own: kept out of the fused launches)
     static constexpr bool FUSABLE = RP < 3 && CP == 0 && E + D * U * (TM + TN) <= (QUAD ? (MT == 32 ? 48 : 56) : 48);   // per-step addressing of the plain layout needs more registers, and so do the 16-register accumulator tuples of the 32 x 32 tiles
+    // the three-term bodies of up to two 32 x 32 tiles per wavefront (100-155 registers) run inside fused launches of the
+    // wide-register kernel family (fused_kernel_wide)
+    static constexpr bool FUSABLE_WIDE = RP == 3 && NW <= 8 && TM * TN <= 2;
     static constexpr int KREDUCED = RP;                    // 0: fp32 filters; 1: packed filters hold bfloat16; 2: IEEE half; 3: three bfloat16 planes; 4: one
     static constexpr int PLANES = RP == 3 ? 3 : 1;
     // RP == 4: the reduced-precision mode on the same instruction and layout: one plane of filters rounded to bfloat16, inputs

@@ -56,7 +56,8 @@ struct VariantEntry {
      ConvSplit3<TMW, TNW, WM, WN, PD>::SMEM_FLOATS},
 
 #define IOS_WSPLIT_X3_ENTRY(IDX, NAME, TM, TN, NW, D)                                                                        \
-    {{NAME, TM * 32, TN * 32, 16, 1, 1, NW, 32, true, ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::CPAD, true, false, PREC_FP32, 3},      \
+    {{NAME, TM * 32, TN * 32, 16, 1, 1, NW, 32, true, ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::CPAD, true, false, PREC_FP32, 3, \
+      ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::FUSABLE_WIDE},      \
      conv_kernel<ConvWsplit<32, TM, TN, NW, 8, true, D, 3>>, conv_kernel<ConvWsplit<32, TM, TN, NW, 8, true, D, 3>, true>,              \
      ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::SMEM_FLOATS},
 

@@ -49,7 +49,8 @@ constexpr int kFusedThreadClasses[] = {256, 512, 1024};
 // kernel-argument segment instead (fused_kernel.h); `num_cus`: compute units of the device.
 // The form of the fused kernel a launch of these items (host copies) takes: the items in a table in device memory, or in the
 // kernel-argument segment, where one kernel holds the matrix-path convolution bodies and another the depth-wise / direct ones.
-enum class FusedForm { Table, InlineMatrix, InlineDirect };
+// Wide: a convolution item needs the kernel family without a register cap (ConvVariant::needs_wide): items in the table.
+enum class FusedForm { Table, InlineMatrix, InlineDirect, Wide };
 FusedForm fused_launch_form(const WorkItem *host_items, int num_items, int threads, int total_blocks, int num_cus);
 const char *fused_kernel_name(FusedForm form);   // without the block size
 void launch_fused(int threads, const WorkItem *device_items, const WorkItem *host_items, const FusedHeader &header, int total_blocks, int smem_bytes, int num_cus, hipStream_t stream);

@@ -8,6 +8,9 @@
 namespace ios {
 
 FusedForm fused_launch_form(const WorkItem *host_items, int num_items, int threads, int total_blocks, int num_cus) {
+    if (host_items)
+        for (int i = 0; i < num_items; i++)
+            if (host_items[i].kind == WORK_CONV && conv_variant(host_items[i].variant).needs_wide()) return FusedForm::Wide;
     if (!host_items || num_items > kInlineItems) return FusedForm::Table;
     bool matrix = false, direct = false;
     for (int i = 0; i < num_items; i++) {
@@ -21,7 +24,8 @@ FusedForm fused_launch_form(const WorkItem *host_items, int num_items, int threa
 }
 
 const char *fused_kernel_name(FusedForm form) {
-    return form == FusedForm::Table ? "fused_kernel" : form == FusedForm::InlineMatrix ? "fused_kernel_inline" : "fused_kernel_inline_direct";
+    return form == FusedForm::Table ? "fused_kernel" : form == FusedForm::InlineMatrix ? "fused_kernel_inline"
+           : form == FusedForm::InlineDirect ? "fused_kernel_inline_direct" : "fused_kernel_wide";
 }
 
 void launch_fused(int threads, const WorkItem *device_items, const WorkItem *host_items, const FusedHeader &header, int total_blocks, int smem_bytes, int num_cus, hipStream_t stream) {
@@ -31,6 +35,10 @@ void launch_fused(int threads, const WorkItem *device_items, const WorkItem *hos
     int b[kFusedHeaderItems];
     for (int i = 0; i < kFusedHeaderItems; i++) b[i] = i < header.num_items ? header.first_block[i] : INT_MAX;
     const FusedForm form = fused_launch_form(host_items, header.num_items, threads, total_blocks, num_cus);
+    if (form == FusedForm::Wide) {
+        launch_fused_wide(threads, device_items, header.num_items, b, total_blocks, smem_bytes, stream);
+        return;
+    }
     if (form == FusedForm::Table) host_items = nullptr;
     if (host_items && threads != 512) {
         InlineItems inl{};

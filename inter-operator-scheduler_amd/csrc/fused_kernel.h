@@ -8,7 +8,8 @@ namespace ios {
 
 // One block of a fused launch: the body of `item`.  MATRIX / DIRECT: the matrix-path convolution bodies / the depth-wise and
 // direct convolution bodies are part of the kernel.
-template <int T, bool MATRIX = true, bool DIRECT = true>
+// WIDE: the kernel also holds the three-term wave-split bodies (fused_kernel_wide, no cap on registers).
+template <int T, bool MATRIX = true, bool DIRECT = true, bool WIDE = false>
 __device__ __forceinline__ void fused_item(const WorkItem &item, const int bid, float *smem) {
     // An item spans five 64-byte lines of the scalar cache, and the bodies read its fields in two or three dependent steps
     // (kind, then configuration, then arguments): one word of every line is requested together with the first step, so
@@ -57,6 +58,13 @@ __device__ __forceinline__ void fused_item(const WorkItem &item, const int bid, 
         if constexpr (64 * NW <= T && ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::FUSABLE)           \
             ConvWsplit<MT, TM, TN, NW, U, QUAD, D, BF16, 4>::run(a, smem, tile, g, z);                    \
         break;
+#define IOS_CASE_X3(IDX, NAME, TM, TN, NW, D)                                                         \
+    case IDX:                                                                                      \
+        if constexpr (WIDE && 64 * NW <= T && ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::FUSABLE_WIDE)   \
+            ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::run(a, smem, tile, g, z);                   \
+        break;
+                IOS_WSPLIT_X3_VARIANTS(IOS_CASE_X3)
+#undef IOS_CASE_X3
                 IOS_TILED_VARIANTS(IOS_CASE_TILED)
                 IOS_WSPLIT_VARIANTS(IOS_CASE_WSPLIT)
                 IOS_WSPLIT_C4_VARIANTS(IOS_CASE_WSPLIT_C4)
@@ -175,6 +183,22 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(4))) void fus
                                                                                                           int b6, int b7, const InlineItems inl) {
     fused_inline_block<T, false>(b1, b2, b3, b4, b5, b6, b7);
 }
+
+// The family with room for the three-term wave-split bodies: no cap on registers (its heaviest body takes ~155, three
+// wavefronts per SIMD), every other body as well, items in the table.  For parallel stages at batch 16 and more, where those
+// bodies are the fastest convolution kernels and the launches run long enough for the lower occupancy not to matter.
+template <int T>
+__global__ __launch_bounds__(T) void fused_kernel_wide(const WorkItem *__restrict__ items, int num_items, int b1, int b2, int b3, int b4, int b5, int b6,
+                                                        int b7) {
+    extern __shared__ floatx4 fused_smem[];
+    float *smem = reinterpret_cast<float *>(fused_smem);
+    const int bid = blockIdx.x;
+    const int index = fused_item_index<T>(items, bid, num_items, b1, b2, b3, b4, b5, b6, b7);
+    fused_item<T, true, true, true>(items[index], bid, smem);
+}
+
+// fused_wide.hip (256 and 512 threads)
+void launch_fused_wide(int threads, const WorkItem *device_items, int num_items, const int *first_blocks, int total_blocks, int smem_bytes, hipStream_t stream);
 
 // fused_512.hip
 void launch_fused_512(const WorkItem *device_items, const WorkItem *host_items, int num_items, const int *first_blocks, int total_blocks, int smem_bytes, hipStream_t stream);

@@ -56,7 +56,10 @@ struct ConvVariant {
     // packed filters as planes of bfloat16, [k / 8][plane][m][8]: 3 = the exact three-term split of fp32 values (fp32 results from
     // the bfloat16 matrix pipe), 1 = one plane rounded to nearest even (the reduced-precision mode on the same kernels), 0 = neither
     int koct = 0;
-    bool fusable() const { return fusable_; }
+    // fits a fused stage launch of the wide-register kernel family only (the three-term wave-split configurations)
+    bool fusable_wide_ = false;
+    bool fusable() const { return fusable_ || fusable_wide_; }
+    bool needs_wide() const { return fusable_wide_ && !fusable_; }
     int kvec() const { return koct ? 8 : kquad ? 4 : 1; }   // consecutive k of one output channel that lie together
 };
 

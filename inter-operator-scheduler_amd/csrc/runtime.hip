@@ -298,8 +298,16 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
         // executors launch every operator by itself, so every configuration competes); a budget nobody fits takes the
         // fastest such configuration
         const bool any_kernel = !fused_executor();
+        // A configuration of the wide-register fused family (three wavefronts per SIMD, items fetched from the table) only
+        // competes when it runs for 12 us or more by itself: below that the family's slower start costs more than the
+        // kernel gains (Inception-v3 at batch 1, same device: 0.379-0.385 ms with it against 0.375-0.377 ms without).
+        constexpr float kWideMinMs = 0.012f;
+        auto wide_too_short = [&](const Candidate &cand) {
+            return !any_kernel && conv_variant(cand.launch.variant).needs_wide() && cand.ms < kWideMinMs;
+        };
         auto eligible = [&](const Candidate &cand, bool fit) {
             if (c == 0) return true;
+            if (wide_too_short(cand)) return false;
             return (cand.fusable || any_kernel) && (!fit || cand.footprint <= capacity / (1 << c));
         };
         found[c] = false;
@@ -308,7 +316,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
             auto score = [&](const Candidate &cand) { return cand.ms * (1.0 + ((1 << c) - 1) * cand.footprint / capacity); };
             std::vector<size_t> order;
             for (size_t i = 0; i < candidates.size(); i++)
-                if (candidates[i].fusable || any_kernel) order.push_back(i);
+                if ((candidates[i].fusable || any_kernel) && !wide_too_short(candidates[i])) order.push_back(i);
             std::sort(order.begin(), order.end(), [&](size_t a, size_t b) { return score(candidates[a]) < score(candidates[b]); });
             double best = 1e300;
             for (size_t n = 0; n < order.size() && n < 3; n++) {
@@ -844,6 +852,17 @@ void Session::build_fused() {
                         all_fusable = all_fusable && pend.fusable;
                     }
             if (here.empty()) continue;
+            // a configuration of the wide-register family beside a 1024-thread body: that family has no such form, the
+            // operators of the level are launched one after the other instead (they are independent of each other)
+            bool needs_wide = false;
+            for (Pending *pend : here)
+                needs_wide = needs_wide || (pend->item.kind == WORK_CONV && conv_variant(pend->item.variant).needs_wide());
+            if (needs_wide && widest > 512 && all_fusable) {
+                for (Pending *pend : here)
+                    if (pend->item.kind != WORK_REDUCE)   // (a stand-alone split-K launch brings its own reduction)
+                        fused_stages_[s].push_back(FusedLaunch{0, 0, 0, 0, 0, pend->op, {}, {pend->op}});
+                continue;
+            }
             if (solo && (here.size() == 1 || !all_fusable)) {
                 for (Pending *pend : here) fused_stages_[s].push_back(FusedLaunch{0, 0, 0, 0, 0, pend->op, {}, {pend->op}});
                 continue;

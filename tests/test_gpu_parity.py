@@ -807,6 +807,38 @@ def test_network_with_measured_kernel_configurations_matches_oracle(name, make):
         rt.set_option('autotune', 0)
 
 
+@pytest.mark.parametrize('variant_name', ['x3w_m64n32_w4', 'x3w_m32n64_w4', 'x3w_m32n32_w8', 'x3w_m64n32_w2'])
+def test_three_term_configurations_inside_fused_stage_launches(variant_name):
+    """
+    The three-term wave-split bodies are too heavy on registers for the fused stage kernels with six wavefronts per SIMD and run
+    in a family of their own (256 and 512 threads, items in the table): parallel stages of Inception-v3 at batch 4 with one such
+    configuration pinned for every convolution, against the oracle and bit for bit against the stream executor.
+    """
+    graph = ios.models.inception_v3(init_seed=0, init_scheme='he_normal_bias')
+    graph.sequential_schedule()
+    x = np.random.default_rng(2).standard_normal((4, *graph.enter_node.output_shape)).astype(np.float32)
+    want = ios_oracle.run(graph, x)
+    graph.greedy_schedule(8)
+    rt.set_option('conv_variant', rt.device_info()['conv_variants'].index(variant_name))
+    rt.set_option('conv_split_k', 1)
+    outs = {}
+    for executor in ('streams', 'fused', 'fused_graph'):
+        rt.set_option('executor', executor)
+        with rt.Session(graph, 4) as session:
+            session.load_weights()
+            session.set_input(x)
+            for _ in range(2):
+                session.run()
+            outs[executor] = session.output()
+            if executor == 'fused':
+                kernels = {launch['kernel'] for launch in session.launches() if len(launch['ops']) > 1}
+                threads = 512 if variant_name.endswith('w8') else 256
+                assert f'fused_kernel_wide<{threads}>' in kernels, kernels
+    assert_close(outs['streams'], want, variant_name)
+    for executor in ('fused', 'fused_graph'):
+        np.testing.assert_array_equal(outs[executor], outs['streams'], err_msg=executor)
+
+
 # The rest of the reference's model zoo (python/ios/models/{alexnet,vgg,resnet}.py): chains, and residual networks whose
 # additions are the two-operand `element` operator.  (id, constructor, batch, operators without a tensor of their own: the
 # last convolution of a residual unit writes the sum, and the addition in front of a ReLU is part of that launch too)
