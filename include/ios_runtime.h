@@ -94,9 +94,9 @@ const char *ios_last_error(void);
 /* Options (set them before sessions are created):
  *   "executor" = "fused" (default: the groups of a stage share one kernel launch per level) | "fused_graph" (fused
  *       launches inside a hipGraph) | "streams" (one HIP stream per group, event fork/join) | "graph" (the stream form
- *       captured into a hipGraph and replayed).  The fused forms are the fast ones at small batches; from batch 16 on
- *       the stream forms can be ahead, because every convolution kernel configuration may serve a parallel stage there,
- *       also those too heavy on registers to share a fused launch;
+ *       captured into a hipGraph and replayed).  The fused forms are the fast ones at small batches; at large ones
+ *       (batch 64) the stream forms can be ahead by a little, because every convolution kernel configuration may serve a
+ *       parallel stage there, also the few too heavy on registers or LDS to share any fused launch;
  *   "autotune" = "1" (default) | "0": measure convolution kernel configurations on first use, like the reference's
  *       cudnnFind-based selection (src/ios/ios_runtime.cu:150-205); "clear_tuning" = anything forgets them;
  *   "split_k_reduce" = "xcd" (default: the last block of a tile adds the split-K slices inside the convolution kernel,
