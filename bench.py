@@ -239,6 +239,32 @@ def probe(args, np, ios, rt):
                           'write_bytes_per_launch': nbytes, 'ms_per_launch': ms,
                           'gbs': 2 * nbytes / (ms * 1e-3) / 1e9}))
         return
+    if args.probe == 'layer':
+        # one convolution with one pinned kernel configuration, a few launches: for counter runs on a single kernel
+        ic, h, w, oc, kh, kw, stride, ph, pw = (int(v) for v in args.layer.split(','))
+        rt.set_option('autotune', 0)
+        rt.set_option('executor', 'streams')
+        rt.set_option('conv_variant', rt.device_info()['conv_variants'].index(args.variant))
+        rt.set_option('conv_split_k', args.split_k)
+        ios.reset_name()
+        v = ios.placeholder((ic, h, w))
+        block = ios.Block(v.node)
+        ios.conv2d(block, [[v]], oc, (kh, kw), (stride, stride), (ph, pw), 1, 'relu', is_exit=True)
+        graph = ios.Graph('layer', v.node, [block])
+        graph.init_weights(0, 'he_normal_bias')
+        graph.sequential_schedule()
+        x = np.random.default_rng(0).standard_normal((args.batch, ic, h, w)).astype(np.float32)
+        with rt.Session(graph, args.batch) as session:
+            session.load_weights()
+            session.set_input(x)
+            for _ in range(args.passes):
+                session.run()
+            ms = session.profile_ops(2, 10)[0]
+            op = session.describe()[0]
+        print(json.dumps({'probe': 'layer', 'layer': args.layer, 'batch': args.batch, 'variant': op.get('variant'), 'split_k': op.get('split_k'),
+                          'us_per_launch': ms * 1e3, 'flops': op['flops'], 'bytes': op['bytes'],
+                          'tflops': op['flops'] / (ms * 1e-3) / 1e12, 'gbs': op['bytes'] / (ms * 1e-3) / 1e9}))
+        return
     if args.probe == 'floor':
         # what a launch costs when it does next to nothing: a chain of dependent tanh activations on one 8 x 8 x 8 tensor and a
         # chain of dependent 1x1 convolutions (8 -> 8 channels on 8 x 8 pixels), one launch each, under every executor
@@ -364,7 +390,10 @@ def main():
                              "with bypass, the chains and residual networks of its zoo) under sequential, greedy and searched schedules "
                              "(about three more minutes; not part of the metric)")
     parser.add_argument('--option', action='append', default=[], metavar='KEY=VALUE', help='extra runtime option (repeatable)')
-    parser.add_argument('--probe', choices=['copy', 'search', 'pass', 'floor'], help='run a profiler probe instead of the benchmark')
+    parser.add_argument('--probe', choices=['copy', 'search', 'pass', 'floor', 'layer'], help='run a profiler probe instead of the benchmark')
+    parser.add_argument('--layer', default='80,73,73,192,3,3,1,0,0', help='probe layer: IC,H,W,OC,KH,KW,stride,pad_h,pad_w of the convolution')
+    parser.add_argument('--variant', default='x3_m64n128_w2x2', help='probe layer: kernel configuration name')
+    parser.add_argument('--split-k', type=int, default=1, help='probe layer: K slices')
     parser.add_argument('--model', default='inception_v3', choices=sorted(CONFIG_MODELS), help='network of the search / pass probes')
     parser.add_argument('--schedule-file', help='probe search: where to write the schedule; probe pass: schedule to run (default: sequential)')
     parser.add_argument('--passes', type=int, default=3, help='forward passes of the pass probe')
