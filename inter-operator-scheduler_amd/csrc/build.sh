@@ -26,8 +26,9 @@ if [ "$status" -ne 0 ]; then
     exit 1
 fi
 if grep -h "ScratchSize \[bytes/lane\]: [1-9]" build/*.log > /dev/null; then
-    echo "warning: kernels spilling to scratch memory:" >&2
-    grep -h -B4 "ScratchSize \[bytes/lane\]: [1-9]" build/*.log | grep "Function Name" | sed 's/.*Function Name: /  /; s/ \[-R.*//' >&2
+    echo "warning: kernels spilling to scratch memory (bytes per lane):" >&2
+    awk '/Function Name:/ { name = $0; sub(/.*Function Name: /, "", name); sub(/ \[-R.*/, "", name) }
+         /ScratchSize \[bytes\/lane\]: [1-9]/ { size = $0; sub(/.*lane\]: /, "", size); sub(/ .*/, "", size); print "  " size "  " name }' build/*.log >&2
 fi
 hipcc --offload-arch=gfx950 -shared -fPIC -o build/libios_runtime.so build/conv_mfma.o build/pointwise.o build/fused.o build/fused_512.o build/fused_wide.o build/runtime.o build/c_api.o build/plan.o
 echo "built $(pwd)/build/libios_runtime.so"
