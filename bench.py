@@ -349,7 +349,7 @@ def probe(args, np, ios, rt):
                       'executor': args.executor, 'kernels': kernels,
                       'launches': [{'stage': l['stage'], 'kernel': l['kernel'], 'blocks': l['blocks'], 'flops': l['flops'],
                                     'bytes': l['bytes'],
-                                    'ops': [{'node': ops[i]['node'], 'kind': ops[i]['kind'], 'conv': ops[i].get('conv'), 'depthwise': ops[i].get('depthwise'),
+                                    'ops': [{'node': ops[i]['node'], 'kind': ops[i]['kind'], 'conv': ops[i].get('conv'),
                                              'out': ops[i]['out'], 'variant': ops[i].get('variant'), 'flops': ops[i]['flops'],
                                              'bytes': ops[i]['bytes']} for i in l['ops']]} for l in launches]}))
 

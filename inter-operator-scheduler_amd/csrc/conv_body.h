@@ -29,7 +29,6 @@
 #pragma once
 
 #include "kernels.h"
-#include "pointwise_body.h"
 
 #include <type_traits>
 
@@ -60,9 +59,6 @@ __device__ __forceinline__ unsigned fast_div(unsigned n, const FastDiv &f) {
 }
 
 struct ConvKernelArgs {
-    // separable pair (configurations with SEP): the 1 x 1 convolution reads the depth-wise result from LDS and none of the fields
-    // that describe its input (x, x_bs, x_bytes, H, W, strides, padding); x then holds the address of the depth-wise half's
-    // argument block in device memory, see sep()
     const float *x;
     const float *wp;
     const float *bias;
@@ -78,7 +74,6 @@ struct ConvKernelArgs {
     unsigned x_bytes, w_bytes;        // extents of the input view and of the packed filters, both < 2^31
     int Npix;
     int act, pre_relu;
-    __host__ __device__ const DirectConvArgs *sep() const { return reinterpret_cast<const DirectConvArgs *>(x); }
     int split_k, k_chunk;
     int steps_total, steps_chunk, steps_per_wave;   // wave-split kernels: MFMA k-steps in K, in a grid slice, in a wavefront's share of a full slice
     int tiles_m, tiles_n;
@@ -834,93 +829,6 @@ __device__ __forceinline__ void splitk_reduce_body(const ReduceArgs &a, int bloc
 }
 
 
-// Separable pair, depth-wise half of one wavefront (see ConvWsplit, SEP): results of the channels [c_lo, c_hi) x the BN pixels
-// from n0 on into stage[channel * BN + pixel].  A lane takes EU elements per round; the K * K taps of all of them are
-// independent buffer loads issued together (taps outside the image, and elements that only pad the tile, carry the
-// out-of-range bit and read zero), then the same for every further summed input in turn (SUM; the values are added in input
-// order, then the folded ReLU, as in the depth-wise kernel), then bias + taps in (kh, kw) order.  Nothing in a round
-// branches, so its loads overlap.
-template <int K, int BN, bool SUM>
-__device__ __forceinline__ void sep_stage_n(const DirectConvArgs &dw, const ConvKernelArgs &a, float *stage, int c_lo, int c_hi, int n0, int lane) {
-    constexpr int EU = K == 3 ? 4 : K == 5 ? 2 : 1;
-    constexpr int T = K * K;
-    const ConvProblem &p = dw.p;
-    const int relu_floor = p.pre_relu ? 0 : (int)0x80000000;   // folded ReLU as an integer max
-    const int count = (c_hi - c_lo) * BN;   // <= 0 for a wavefront beyond the end of K
-    const int plane = p.H * p.W;
-    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(dw.x), 0, dw.x_bytes, 0x00020000);
-    for (int e0 = lane; e0 < count; e0 += 64 * EU) {
-        unsigned inside[EU];   // offset of the window's first tap inside an image, in bytes (may be "negative": wraps)
-        unsigned image[EU];    // image index
-        unsigned kill[EU][T];
-        const float *wc[EU];
-        float acc[EU], v[EU][T];
-        bool real[EU];
-#pragma unroll
-        for (int q = 0; q < EU; q++) {
-            const int e = e0 + q * 64;
-            const int c = c_lo + e / BN;
-            const int n = n0 + e % BN;
-            real[q] = e < count && c < a.ICg && n < a.Npix;
-            const int cc = min(c, a.ICg - 1);
-            const int nn = real[q] ? n : 0;
-            const int b = (int)fast_div((unsigned)nn, a.div_ohw);
-            const int rem = nn - __mul24(b, a.OHW);
-            const int oh = (int)fast_div((unsigned)rem, a.div_ow);
-            const int ow = rem - __mul24(oh, a.OW);
-            const int h0 = oh * p.sh - p.ph, w0 = ow * p.sw - p.pw;
-            image[q] = (unsigned)b;
-            inside[q] = (unsigned)(cc * plane + h0 * p.W + w0) * 4u;
-            wc[q] = dw.w + cc * T;
-            acc[q] = dw.bias[cc];
-            const unsigned dead = real[q] ? 0u : 0x80000000u;
-#pragma unroll
-            for (int i = 0; i < K; i++) {
-                const unsigned row_kill = (unsigned)(h0 + i) < (unsigned)p.H ? dead : 0x80000000u;
-#pragma unroll
-                for (int j = 0; j < K; j++) kill[q][i * K + j] = (unsigned)(w0 + j) < (unsigned)p.W ? row_kill : 0x80000000u;
-            }
-        }
-#pragma unroll
-        for (int q = 0; q < EU; q++) {
-            const unsigned base = image[q] * (unsigned)dw.x_bs * 4u + inside[q];
-#pragma unroll
-            for (int i = 0; i < K; i++)
-#pragma unroll
-                for (int j = 0; j < K; j++) v[q][i * K + j] = pw_buffer_load(xr, (base + (unsigned)(i * p.W + j) * 4u) | kill[q][i * K + j]);
-        }
-        float w[EU][T];
-#pragma unroll
-        for (int q = 0; q < EU; q++)
-#pragma unroll
-            for (int t = 0; t < T; t++) w[q][t] = wc[q][t];
-        if constexpr (SUM) {
-            for (int s = 0; s < dw.nmore; s++) {
-                const __amdgpu_buffer_rsrc_t sr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(dw.more[s]), 0, dw.more_bytes[s], 0x00020000);
-                float u[EU][T];
-#pragma unroll
-                for (int q = 0; q < EU; q++) {
-                    const unsigned base = image[q] * (unsigned)dw.more_bs[s] * 4u + inside[q];
-#pragma unroll
-                    for (int i = 0; i < K; i++)
-#pragma unroll
-                        for (int j = 0; j < K; j++) u[q][i * K + j] = pw_buffer_load(sr, (base + (unsigned)(i * p.W + j) * 4u) | kill[q][i * K + j]);
-                }
-#pragma unroll
-                for (int q = 0; q < EU; q++)
-#pragma unroll
-                    for (int t = 0; t < T; t++) v[q][t] += u[q][t];
-            }
-        }
-#pragma unroll
-        for (int q = 0; q < EU; q++) {
-#pragma unroll
-            for (int t = 0; t < T; t++) acc[q] = fmaf(__int_as_float(max(__float_as_int(v[q][t]), relu_floor)), w[q][t], acc[q]);
-            if (e0 + q * 64 < count) stage[c_lo * BN + e0 + q * 64] = real[q] ? act_apply(acc[q], p.act) : 0.f;
-        }
-    }
-}
-
 // ---- wave-split variant: no LDS staging, K divided among the wavefronts of a block ---------------------------------------
 // For batch-1 layers (tens to hundreds of pixels, K in the thousands) the LDS-tiled kernel is bound by the chain
 // load -> LDS -> barrier per K tile, and slicing K over blocks costs a second kernel.  Here every wavefront of a
@@ -941,23 +849,13 @@ __device__ __forceinline__ void sep_stage_n(const DirectConvArgs &dw, const Conv
 //
 // CP: channel padding of the packed filters when it should differ from the default (8, or the batch with QUAD); 4 serves
 // layers with a handful of input channels (the first layer of an image network), whose K would otherwise be mostly padding.
-//
-// SEP (separable pair, fp32 QUAD forms with two batches in flight): the input of this 1 x 1 convolution is the result of a
-// depth-wise convolution that nobody else reads.  A wavefront only needs the channels of its own K range, so before its K loop
-// it computes the depth-wise result of those channels for the BN pixels of the block's tile (the element function of the
-// depth-wise kernel, a few elements per lane with all their taps in flight) into its own part of an LDS stage [channel][pixel]
-// behind the reduction area; the K loop then takes its input operand from there (one conflict-free LDS read per value) instead
-// of global memory.  No barrier: a wavefront reads what it wrote itself.  The depth-wise tensor never exists in memory and its
-// launch disappears; every block of a pixel tile (one per BM output channels and K slice) repeats the depth-wise work of the
-// channels it needs.
-template <int MT, int TM, int TN, int NW, int U, bool QUAD = false, int D = 2, int RP = 0, int CP = 0, bool SEP = false>
+template <int MT, int TM, int TN, int NW, int U, bool QUAD = false, int D = 2, int RP = 0, int CP = 0>
 struct ConvWsplit {
     using M = Mfma<MT>;
     static constexpr int BM = TM * MT, BN = TN * MT;
     static constexpr int E = TM * TN * M::ACC;
     static constexpr int THREADS = 64 * NW;
-    static constexpr int SMEM_FLOATS = NW * E * 64;   // SEP: the stage of ICgP * BN floats follows (the launcher adds it)
-    static_assert(!SEP || (QUAD && D == 2 && RP == 0 && CP == 0), "separable pairs: fp32 quad layout, two batches in flight");
+    static constexpr int SMEM_FLOATS = NW * E * 64;
     static constexpr int CPAD = CP ? CP : (QUAD ? U * M::KSTEP : 8);   // channel padding of the packed filters this kernel expects
     static_assert(CP == 0 || (!QUAD && CP % M::KSTEP == 0), "a k-step must lie inside one filter tap");
     static constexpr bool KQUAD = QUAD;                    // packed filters are [k / 4][m][4] instead of [k][m]
@@ -1044,32 +942,6 @@ struct ConvWsplit {
         const int m = m0 + (e / (M::ACC * TN)) * MT + M::row(e % M::ACC, lane);
         bias_pre[t] = a.bias[g * a.OCg + min(m, a.OCg - 1)];
     }
-    float *stage = red + SMEM_FLOATS;
-    if constexpr (SEP) {
-        // depth-wise results of this wavefront's channels (k = channel for a 1 x 1 convolution) x the tile's pixels; channels
-        // beyond the real ones (padding of the last batch) and pixels beyond the last one are staged as zeros
-        // (read through the constant address space: the block is never written while kernels run, so its fields are scalar
-        // loads that need no repeating behind the LDS stores of the stage)
-        typedef const DirectConvArgs __attribute__((address_space(4))) *ConstantBlock;
-        unsigned long long block_address = (unsigned long long)a.sep();
-        asm volatile("" : "+s"(block_address));
-        const DirectConvArgs &dw = *(const DirectConvArgs *)(ConstantBlock)block_address;
-        const int c_lo = s_begin * M::KSTEP;
-        const int c_hi = min(s_end * M::KSTEP, a.ICgP);
-        const bool sums = dw.nmore > 0;   // wavefront-uniform
-        if (dw.p.KH == 3) {
-            if (sums) sep_stage_n<3, BN, true>(dw, a, stage, c_lo, c_hi, n0, lane);
-            else sep_stage_n<3, BN, false>(dw, a, stage, c_lo, c_hi, n0, lane);
-        } else if (dw.p.KH == 5) {
-            if (sums) sep_stage_n<5, BN, true>(dw, a, stage, c_lo, c_hi, n0, lane);
-            else sep_stage_n<5, BN, false>(dw, a, stage, c_lo, c_hi, n0, lane);
-        } else {
-            sep_stage_n<7, BN, false>(dw, a, stage, c_lo, c_hi, n0, lane);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
     typename M::acc_t acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
@@ -1144,17 +1016,6 @@ struct ConvWsplit {
                         A.v[q * 4 + 2][i] = w4.z;
                         A.v[q * 4 + 3][i] = w4.w;
                     }
-            }
-            if constexpr (SEP) {
-                // the lane's U channels of this batch x its pixel of every tile, from this wavefront's part of the stage
-                const float *mine = stage + (q_cb + U * lk) * BN + lc;
-#pragma unroll
-                for (int u = 0; u < U; u++)
-#pragma unroll
-                    for (int j = 0; j < TN; j++) B[u][j] = mine[u * BN + j * MT];
-                q_w += (unsigned)((U * M::KSTEP / 4) * a.OCgP) * 16u;
-                q_cb += U * M::KSTEP;
-                return;
             }
             const unsigned x_tap = (unsigned)(q_kh * a.W + q_kw) * 4u;
             const unsigned x_chan = (unsigned)(q_cb * a.HW) * 4u;
@@ -1344,9 +1205,7 @@ struct ConvWsplit {
                 if (b + st < batches) compute(av[st], bv[st]);
         }
     };
-    if constexpr (SEP) {
-        k_loop(std::false_type{});   // padding channels are zeros in the stage
-    } else if constexpr (QUAD) {
+    if constexpr (QUAD) {
         if ((a.ICg & (U - 1)) == 0) k_loop(std::false_type{});
         else k_loop(std::true_type{});
     } else {
@@ -1578,18 +1437,6 @@ struct ConvWsplit {
     X(116, "wb_x1w_m64n64_w4", 2, 2, 4, 2)     \
     X(117, "wb_x1w_m32n32_w8", 1, 1, 8, 2)     \
     X(118, "wb_x1w_m64n64_w2", 2, 2, 2, 2)
-// X(index, name, MT, TM, TN, NW, U): separable pairs (ConvWsplit with SEP), the fp32 quad configurations that the 1 x 1 layers
-// behind depth-wise convolutions take at batch 1 (at most eight wavefronts: the depth-wise windows need more registers than a
-// 1024-thread block leaves a lane)
-#define IOS_WSPLIT_SEP_VARIANTS(X)              \
-    X(119, "sq_m16n16_w8", 16, 1, 1, 8, 4)      \
-    X(120, "sq_m32n16_w8", 16, 2, 1, 8, 4)      \
-    X(121, "sq_m64n16_w8", 16, 4, 1, 8, 4)      \
-    X(122, "sq_m32n32_w8", 16, 2, 2, 8, 4)      \
-    X(123, "sq_m32n32_w8_t32", 32, 1, 1, 8, 4)  \
-    X(124, "sq_m32n32_w4_t32", 32, 1, 1, 4, 8)  \
-    X(125, "sq_m16n16_w4", 16, 1, 1, 4, 4)      \
-    X(126, "sq_m32n16_w4", 16, 2, 1, 4, 4)
-constexpr int kNumConvVariants = 127;
+constexpr int kNumConvVariants = 119;
 
 }  // namespace ios

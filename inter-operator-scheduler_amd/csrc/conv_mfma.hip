@@ -3,7 +3,6 @@
 #include "launch_internal.h"
 
 #include <algorithm>
-#include <cstring>
 #include <stdexcept>
 #include <string>
 
@@ -73,18 +72,11 @@ struct VariantEntry {
      conv_kernel<ConvWsplit<32, TM, TN, NW, 8, true, D, 4>>, conv_kernel<ConvWsplit<32, TM, TN, NW, 8, true, D, 4>, true>,              \
      ConvWsplit<32, TM, TN, NW, 8, true, D, 4>::SMEM_FLOATS},
 
-#define IOS_WSPLIT_SEP_ENTRY(IDX, NAME, MT, TM, TN, NW, U)                                                                     \
-    {{NAME, TM * MT, TN * MT, U *(MT == 32 ? 2 : 4), 1, 1, NW, MT, true, ConvWsplit<MT, TM, TN, NW, U, true, 2, 0, 0, true>::CPAD, true, \
-      false, PREC_FP32, 0, true, true},                                                                                          \
-     conv_kernel<ConvWsplit<MT, TM, TN, NW, U, true, 2, 0, 0, true>>, conv_kernel<ConvWsplit<MT, TM, TN, NW, U, true, 2, 0, 0, true>>, \
-     ConvWsplit<MT, TM, TN, NW, U, true, 2, 0, 0, true>::SMEM_FLOATS},
-
 static const VariantEntry kVariants[] = {IOS_TILED_VARIANTS(IOS_TILED_ENTRY) IOS_WSPLIT_VARIANTS(IOS_WSPLIT_ENTRY)
                                              IOS_WSPLIT_C4_VARIANTS(IOS_WSPLIT_C4_ENTRY)
                                              IOS_WSPLIT_T32_VARIANTS(IOS_WSPLIT_ENTRY) IOS_WSPLIT_F16_VARIANTS(IOS_WSPLIT_ENTRY)
                                              IOS_WSPLIT_LONGK_VARIANTS(IOS_WSPLIT_ENTRY) IOS_SPLIT3_VARIANTS(IOS_SPLIT3_ENTRY) IOS_WSPLIT_X3_VARIANTS(IOS_WSPLIT_X3_ENTRY)
-                                             IOS_SPLIT1_VARIANTS(IOS_SPLIT1_ENTRY) IOS_WSPLIT_X1_VARIANTS(IOS_WSPLIT_X1_ENTRY)
-                                             IOS_WSPLIT_SEP_VARIANTS(IOS_WSPLIT_SEP_ENTRY)};
+                                             IOS_SPLIT1_VARIANTS(IOS_SPLIT1_ENTRY) IOS_WSPLIT_X1_VARIANTS(IOS_WSPLIT_X1_ENTRY)};
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 static_assert(kNumVariants == kNumConvVariants, "variant lists and count disagree");
 
@@ -146,17 +138,6 @@ ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only
         return (long long)ceil_div(M, v.BM) * ceil_div(N, v.BN) * p.groups;
     };
     ConvLaunch best;
-    if (p.separable()) {
-        // separable pairs (batch-1 sized by the planner's rule): the largest tile that still offers a block per compute unit
-        static const int sep_large_to_small[] = {variant_by_name("sq_m64n16_w8"), variant_by_name("sq_m32n16_w8"), variant_by_name("sq_m16n16_w8")};
-        for (int idx : sep_large_to_small)
-            if (blocks_of(idx) >= num_cus) {
-                best.variant = idx;
-                return best;
-            }
-        best.variant = variant_by_name("sq_m16n16_w8");
-        return best;
-    }
     if (precision != PREC_FP32) {
         // reduced precision: wave-split configurations only, the largest tile that offers two blocks per compute unit
         static const int bf16_large_to_small[] = {variant_by_name("wb_m64n64_w4"), variant_by_name("wb_m64n32_w8"),
@@ -212,42 +193,6 @@ ConvLaunch conv_pick_launch(const ConvProblem &p, int num_cus, bool fusable_only
     return best;
 }
 
-// Separable pairs: windows the staging code is instantiated for, summed inputs only where the depth-wise kernel adds them,
-// a stage (channels padded to 32 x the widest pixel tile) that leaves LDS for two blocks per compute unit, and input tensors
-// within 31-bit byte offsets (the caller checks the views' real extents).
-bool conv_separable_supported(const ConvProblem &p) {
-    if (!p.separable()) return false;
-    if (p.KH != 1 || p.KW != 1 || p.sh != 1 || p.sw != 1 || p.ph != 0 || p.pw != 0 || p.groups != 1 || p.pre_relu) return false;
-    if (p.dw_k != 3 && p.dw_k != 5 && p.dw_k != 7) return false;
-    if (p.dw_nsrc < 1 || p.dw_nsrc > kMaxNaryInputs || (p.dw_nsrc > 1 && p.dw_k == 7)) return false;
-    if ((long long)p.ICgP(32) * 32 * 4 > 48 * 1024) return false;
-    return (unsigned long long)p.B * p.IC * p.dw_h * p.dw_w * 4ull < (1ull << 30);
-}
-
-int conv_separable_lds_bytes(const ConvProblem &p, int variant) {
-    const VariantEntry &e = kVariants[variant];
-    return (e.smem_floats + p.ICgP(e.v.cpad) * e.v.BN) * (int)sizeof(float);
-}
-
-size_t conv_depthwise_args_floats() { return (sizeof(DirectConvArgs) + 3) / 4; }
-
-void fill_conv_depthwise_args(const ConvProblem &p, const TensorView &x, const TensorView *more, int nmore, const float *w, const float *bias,
-                              int pre_relu, int act, void *host_block) {
-    if (!conv_separable_supported(p) || nmore + 1 != p.dw_nsrc) throw std::runtime_error("conv: not a separable pair this library fuses");
-    ConvProblem d{};
-    d.B = p.B; d.IC = p.IC; d.OC = p.IC; d.groups = p.IC;
-    d.H = p.dw_h; d.W = p.dw_w; d.OH = p.H; d.OW = p.W;
-    d.KH = d.KW = p.dw_k; d.sh = d.sw = p.dw_s; d.ph = d.pw = p.dw_p;
-    d.act = act; d.pre_relu = pre_relu;
-    TensorView none{};   // the depth-wise result has no tensor
-    none.C = d.OC; none.H = d.OH; none.W = d.OW;
-    int blocks = 0;
-    DirectConvArgs a = make_direct_conv_args(d, x, w, bias, none, &blocks);
-    if (nmore > 0) add_dwconv_sources(a, more, nmore);
-    if (a.x_bytes == 0) throw std::runtime_error("conv: separable pair with an input view beyond 31-bit byte offsets");
-    memcpy(host_block, &a, sizeof(a));
-}
-
 bool conv_matrix_path_supported(const ConvProblem &p) {
     // packed filter rows are indexed with 16 bits, input and filter byte offsets with 31 bits
     const unsigned long long x_bytes = (unsigned long long)p.B * p.IC * p.H * p.W * 4ull;
@@ -259,13 +204,11 @@ bool conv_matrix_path_supported(const ConvProblem &p) {
 
 ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
                                 const float *bias, const TensorView &y, float *workspace, const SplitKReduce &reduce,
-                                const TensorView *residual, bool post_relu, const DirectConvArgs *depthwise) {
+                                const TensorView *residual, bool post_relu) {
     if (l.variant < 0 || l.variant >= kNumVariants) throw std::runtime_error("conv: bad variant");
     const VariantEntry &e = kVariants[l.variant];
-    if (x.C != p.IC || x.H != (p.separable() ? p.dw_h : p.H) || x.W != (p.separable() ? p.dw_w : p.W) || y.C != p.OC || y.H != p.OH || y.W != p.OW)
+    if (x.C != p.IC || x.H != p.H || x.W != p.W || y.C != p.OC || y.H != p.OH || y.W != p.OW)
         throw std::runtime_error("conv: tensor views do not match the problem");
-    if (e.v.separable != p.separable() || (p.separable() && (depthwise == nullptr || residual != nullptr || !conv_separable_supported(p))))
-        throw std::runtime_error("conv: separable pairs and the configurations for them go together");
     if (p.IC % p.groups != 0 || p.OC % p.groups != 0) throw std::runtime_error("conv: channels not divisible by groups");
     if (!conv_matrix_path_supported(p)) throw std::runtime_error("conv: problem too large for the matrix path");
     ConvDispatch d;
@@ -310,7 +253,6 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     a.div_tile = make_fast_div((unsigned)a.tile_div);
     a.div_ohw = make_fast_div((unsigned)a.OHW);
     a.div_ow = make_fast_div((unsigned)a.OW);
-    if (e.v.separable) a.x = reinterpret_cast<const float *>(depthwise);   // see ConvKernelArgs::sep()
     a.res = nullptr;
     a.res_bs = 0;
     a.post_relu = post_relu ? 1 : 0;
@@ -328,10 +270,6 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
     d.variant = l.variant;
     d.threads = e.v.threads();
     d.smem_bytes = e.smem_floats * (int)sizeof(float);
-    if (e.v.separable) {
-        d.smem_bytes = conv_separable_lds_bytes(p, l.variant);   // the stage of depth-wise results behind the reduction area
-        if (d.smem_bytes > 64 * 1024) throw std::runtime_error(std::string("conv: separable pair too wide for configuration ") + e.v.name);
-    }
     d.tiles = a.tiles_m * a.tiles_n;
     d.groups = p.groups;
     d.slices = a.split_k;
@@ -372,8 +310,8 @@ ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const
 
 void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
                       const float *bias, const TensorView &y, float *workspace, const SplitKReduce &reduce, hipStream_t stream,
-                      const TensorView *residual, bool post_relu, const DirectConvArgs *depthwise) {
-    const ConvDispatch d = make_conv_dispatch(p, l, x, packed, bias, y, workspace, reduce, residual, post_relu, depthwise);
+                      const TensorView *residual, bool post_relu) {
+    const ConvDispatch d = make_conv_dispatch(p, l, x, packed, bias, y, workspace, reduce, residual, post_relu);
     const VariantEntry &e = kVariants[d.variant];
     const dim3 grid = d.xcd_blocks > 0 ? dim3((unsigned)d.xcd_blocks) : dim3((unsigned)d.tiles, (unsigned)d.groups, (unsigned)d.slices);
     const ConvKernelFn kernel = !d.args.xcd_local && d.args.res != nullptr ? e.kernel_residual : e.kernel;

@@ -9,8 +9,6 @@ namespace ios {
 // One block of a fused launch: the body of `item`.  MATRIX / DIRECT: the matrix-path convolution bodies / the depth-wise and
 // direct convolution bodies are part of the kernel.
 // WIDE: the kernel also holds the three-term wave-split bodies (fused_kernel_wide, no cap on registers).
-// It also holds the bodies of the separable pairs, whose depth-wise windows (up to 49 taps in flight per element) do not fit
-// the register caps of the other kernels either.
 template <int T, bool MATRIX = true, bool DIRECT = true, bool WIDE = false>
 __device__ __forceinline__ void fused_item(const WorkItem &item, const int bid, float *smem) {
     // An item spans five 64-byte lines of the scalar cache, and the bodies read its fields in two or three dependent steps
@@ -65,13 +63,7 @@ __device__ __forceinline__ void fused_item(const WorkItem &item, const int bid, 
         if constexpr (WIDE && 64 * NW <= T && ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::FUSABLE_WIDE)   \
             ConvWsplit<32, TM, TN, NW, 8, true, D, 3>::run(a, smem, tile, g, z);                   \
         break;
-#define IOS_CASE_SEP(IDX, NAME, MT, TM, TN, NW, U)                                                    \
-    case IDX:                                                                                      \
-        if constexpr (WIDE && 64 * NW <= T) ConvWsplit<MT, TM, TN, NW, U, true, 2, 0, 0, true>::run(a, smem, tile, g, z); \
-        break;
                 IOS_WSPLIT_X3_VARIANTS(IOS_CASE_X3)
-                IOS_WSPLIT_SEP_VARIANTS(IOS_CASE_SEP)
-#undef IOS_CASE_SEP
 #undef IOS_CASE_X3
                 IOS_TILED_VARIANTS(IOS_CASE_TILED)
                 IOS_WSPLIT_VARIANTS(IOS_CASE_WSPLIT)

@@ -16,7 +16,6 @@ enum Act : int { ACT_NONE = 0, ACT_RELU = 1, ACT_TANH = 2, ACT_SIGMOID = 3 };
 enum Precision : int { PREC_FP32 = 0, PREC_BF16 = 1, PREC_FP16 = 2 };   // operand type of the matrix-path convolutions
 
 constexpr int kMaxNaryInputs = 8;   // views one launch adds (or multiplies)
-struct DirectConvArgs;   // argument block of the depth-wise / direct convolution kernels (pointwise_body.h)
 
 struct TensorView {
     float *ptr = nullptr;  // element (0, 0, 0, 0)
@@ -30,11 +29,6 @@ struct ConvProblem {
     int OH, OW;
     int act;       // Act applied after bias
     int pre_relu;  // apply max(x, 0) to the input while loading it
-    // Separable pair (dw_k > 0): this 1 x 1 convolution reads the result of a depth-wise dw_k x dw_k convolution (stride dw_s,
-    // padding dw_p) of dw_nsrc summed tensors of IC x dw_h x dw_w, which its launch computes itself; H x W is the depth-wise
-    // result.  dw_k == 0: an ordinary convolution.
-    int dw_k, dw_s, dw_p, dw_h, dw_w, dw_nsrc;
-    bool separable() const { return dw_k > 0; }
     int ICg() const { return IC / groups; }
     int OCg() const { return OC / groups; }
     int K() const { return ICg() * KH * KW; }
@@ -62,12 +56,8 @@ struct ConvVariant {
     // packed filters as planes of bfloat16, [k / 8][plane][m][8]: 3 = the exact three-term split of fp32 values (fp32 results from
     // the bfloat16 matrix pipe), 1 = one plane rounded to nearest even (the reduced-precision mode on the same kernels), 0 = neither
     int koct = 0;
-    // fits a fused stage launch of the wide-register kernel family only (the three-term wave-split configurations and those for
-    // separable pairs)
+    // fits a fused stage launch of the wide-register kernel family only (the three-term wave-split configurations)
     bool fusable_wide_ = false;
-    // computes the depth-wise convolution of a separable pair in front of its own 1 x 1 convolution (ConvProblem::dw_k); such
-    // configurations serve those problems and no others
-    bool separable = false;
     bool fusable() const { return fusable_ || fusable_wide_; }
     bool needs_wide() const { return fusable_wide_ && !fusable_; }
     int kvec() const { return koct ? 8 : kquad ? 4 : 1; }   // consecutive k of one output channel that lie together
@@ -119,15 +109,7 @@ struct SplitKReduce {
 // partial outputs (conv_workspace_floats).
 void launch_conv_mfma(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
                       const float *bias, const TensorView &y, float *workspace, const SplitKReduce &reduce, hipStream_t stream,
-                      const TensorView *residual = nullptr, bool post_relu = false, const struct DirectConvArgs *depthwise = nullptr);
-// Separable pair: the argument block of the depth-wise half (the launch reads it from device memory: `depthwise` above points
-// to a copy there).  x: the first summed input; more: the others; w, bias: the depth-wise filters [C][dw_k][dw_k] and bias.
-size_t conv_depthwise_args_floats();
-void fill_conv_depthwise_args(const ConvProblem &p, const TensorView &x, const TensorView *more, int nmore, const float *w, const float *bias,
-                              int pre_relu, int act, void *host_block);
-// largest depth-wise input (channels x pixels of a block tile) a separable configuration stages in LDS
-bool conv_separable_supported(const ConvProblem &p);
-int conv_separable_lds_bytes(const ConvProblem &p, int variant);   // LDS of a separable configuration on this problem (at most 64 KiB may be used)
+                      const TensorView *residual = nullptr, bool post_relu = false);
 
 // Depth-wise convolution (groups == IC == OC), filters in their original [C][1][KH][KW] layout.  With `more`, the input is
 // x + more[0] + ... + more[nmore - 1] (at most kMaxNaryInputs views in all, added left to right before the folded ReLU).

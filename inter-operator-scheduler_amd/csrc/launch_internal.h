@@ -20,7 +20,7 @@ struct ConvDispatch {
 
 ConvDispatch make_conv_dispatch(const ConvProblem &p, const ConvLaunch &l, const TensorView &x, const float *packed,
                                 const float *bias, const TensorView &y, float *workspace, const SplitKReduce &reduce,
-                                const TensorView *residual = nullptr, bool post_relu = false, const DirectConvArgs *depthwise = nullptr);
+                                const TensorView *residual = nullptr, bool post_relu = false);
 PoolArgs make_pool_args(const PoolProblem &p, const TensorView &x, const TensorView &y, bool global, int *blocks,
                         const float *bias = nullptr, int act = ACT_NONE);
 DirectConvArgs make_direct_conv_args(const ConvProblem &p, const TensorView &x, const float *w, const float *bias,

@@ -66,8 +66,6 @@ struct PNode {
     // "average pool, then 1 x 1 convolution" run as "1 x 1 convolution, then average pool": on the pool the convolution, on
     // the convolution the pool
     int commuted_conv = -1, commuted_pool = -1;
-    // separable pair: on the depth-wise convolution the 1 x 1 convolution whose launch computes it, and the other way round
-    int sep_pw = -1, sep_dw = -1;
     int references = 0;            // number of input values that name this node
 };
 
@@ -326,7 +324,6 @@ private:
             }
         }
         find_depthwise_sums();
-        find_separable_pairs();
         find_activated_combinations();
         find_residual_convolutions();
         find_commuting_pools();
@@ -374,7 +371,6 @@ private:
         p.groups = cfg["groups"].as_int();
         p.act = act_code(cfg["act"].as_string());
         p.pre_relu = 0;
-        p.dw_k = p.dw_s = p.dw_p = p.dw_h = p.dw_w = p.dw_nsrc = 0;
         return p;
     }
 
@@ -413,48 +409,6 @@ private:
                     r.no_storage = true;   // the convolution reads the ReLU's inputs itself
                     r.parent = -1;
                 }
-            }
-        }
-    }
-
-    // The 1 x 1 convolution of a separable pair as a problem of its own kind: the depth-wise half's geometry rides along.
-    ConvProblem separable_problem(const PNode &dw, const PNode &pw) const {
-        const ConvProblem pd = problem_of(dw);
-        ConvProblem p = problem_of(pw);
-        p.dw_k = pd.KH; p.dw_s = pd.sh; p.dw_p = pd.ph; p.dw_h = pd.H; p.dw_w = pd.W;
-        p.dw_nsrc = dw.sum_front >= 0 ? (int)nodes_[dw.sum_front].inputs[0].size() : 1;
-        return p;
-    }
-
-    // Sequential children [..., depth-wise K x K convolution, 1 x 1 convolution, ...] (the separable convolution of the reference's
-    // python/ios/models/common.py:365-395, which the reference runs as two cuDNN calls, src/ios/ios_runtime.cu:1059-1084): when
-    // nobody else reads the depth-wise result and the pair is small (option separable_max_pixels; at batch 1 such a pair is bound
-    // by the two launches, not by its arithmetic), the launch of the 1 x 1 convolution computes the depth-wise values it needs
-    // itself (ConvWsplit, SEP): the depth-wise launch and its tensor disappear.  The chooser may decline (a reduced-precision
-    // mode, a pinned kernel configuration): then the pair stays two launches.
-    void find_separable_pairs() {
-        if (planner_separable_max_pixels() <= 0) return;
-        for (const auto &seq : sequentials_) {
-            for (int i = seq.first; i < seq.second; i++) {
-                PNode &dw = nodes_[i];
-                PNode &pw = nodes_[i + 1];
-                if (dw.type != NodeType::Conv || pw.type != NodeType::Conv || dw.references != 1 || !single_value(pw)) continue;
-                const Val &v = pw.inputs[0][0];
-                if (v.node != i || v.begin != 0 || v.end != dw.C) continue;
-                if (dw.sum_front < 0 && !single_value(dw)) continue;   // (a concatenating depth-wise convolution keeps its launch)
-                const ConvProblem pd = problem_of(dw);
-                if (!pd.is_depthwise() || pd.KH != pd.KW || pd.sh != pd.sw || pd.ph != pd.pw) continue;
-                const ConvProblem p = separable_problem(dw, pw);
-                if (!conv_separable_supported(p) || !conv_matrix_path_supported(p) || p.Npix() > planner_separable_max_pixels()) continue;
-                // every summed input is addressed with 31-bit byte offsets wherever it will live (as in find_depthwise_sums)
-                unsigned long long widest = 0;
-                for (const PNode &n : nodes_) widest = std::max(widest, (unsigned long long)n.C * n.H * n.W);
-                if (((unsigned long long)(batch_ - 1) * widest + (unsigned long long)pd.IC * pd.H * pd.W) * 4ull >= (1ull << 31)) continue;
-                if (chooser_(p, 1).variant < 0) continue;
-                dw.sep_pw = i + 1;
-                pw.sep_dw = i;
-                dw.no_storage = true;   // the depth-wise result only exists in the LDS of the 1 x 1 convolution's blocks
-                dw.parent = -1;
             }
         }
     }
@@ -876,10 +830,6 @@ private:
             for (const Val &v : nodes_[n.sum_front].inputs[0]) sum_srcs.push_back(view_of(v.node).window(v.begin, v.end));
             pre_relu = n.sum_relu;
         }
-        if (n.sep_dw >= 0) {
-            emit_separable(n, index);
-            return;
-        }
         const ViewRef in = n.sum_front >= 0 ? sum_srcs[0] : input_view(n, C, H, W, &pre_relu);
         ConvProblem p = problem_of(n);
         p.pre_relu = pre_relu ? 1 : 0;
@@ -933,36 +883,6 @@ private:
                 level_top_ = std::max(level_top_, sum.level + 1);
             }
         }
-    }
-
-    // the one launch of a separable pair (see find_separable_pairs): at the place of the 1 x 1 convolution
-    void emit_separable(PNode &pw, int index) {
-        PNode &dw = nodes_[pw.sep_dw];
-        int C, H, W;
-        input_shape(dw, C, H, W);
-        bool pre_relu = false;
-        std::vector<ViewRef> sum_srcs;
-        if (dw.sum_front >= 0) {
-            for (const Val &v : nodes_[dw.sum_front].inputs[0]) sum_srcs.push_back(view_of(v.node).window(v.begin, v.end));
-            pre_relu = dw.sum_relu;
-        }
-        const ViewRef in = dw.sum_front >= 0 ? sum_srcs[0] : input_view(dw, C, H, W, &pre_relu);
-        ConvProblem pd = problem_of(dw);
-        pd.pre_relu = pre_relu ? 1 : 0;
-        const int dw_conv = add_plan_conv(dw, pd);   // filters and bias of the depth-wise half; no operation of its own
-        const ConvProblem p = separable_problem(dw, pw);
-        const int conv = add_plan_conv(pw, p);
-        plan_.convs[conv].matrix_path = true;
-        plan_.convs[conv].sep_dw = dw_conv;
-        plan_.convs[conv].sep_args_off = reserve(conv_depthwise_args_floats());
-        PlanOp &op = push(OpKind::ConvMfma, pw);
-        op.in = in;
-        op.out = view_of(index);
-        op.conv = conv;
-        op.srcs = sum_srcs;
-        const double k = sum_srcs.empty() ? 1.0 : (double)sum_srcs.size();
-        op.flops = pd.flops() + (k - 1.0) * (double)batch_ * C * H * W + p.flops();
-        op.bytes = 4.0 * (k * (double)batch_ * C * H * W + (double)pd.OC * pd.K() + pd.OC + (double)p.OC * p.K() + p.OC + (double)batch_ * p.OC * p.OH * p.OW);
     }
 
     PoolProblem pool_problem_of(const PNode &n, int C, int H, int W) const {
@@ -1174,16 +1094,11 @@ bool g_arena_reuse = true;
 long long g_thin_conv_min_pixels = 1LL << 18;
 int g_host_split_k = 0;
 bool g_commute_pool_conv = true;
-long long g_separable_max_pixels = 4096;
 }
 
 bool set_planner_option(const std::string &key, const std::string &value) {
     if (key == "arena_reuse") {
         g_arena_reuse = !(value == "0" || value == "false" || value == "off" || value.empty());
-        return true;
-    }
-    if (key == "separable_max_pixels") {
-        g_separable_max_pixels = atoll(value.c_str());
         return true;
     }
     if (key == "commute_pool_conv") {
@@ -1207,7 +1122,6 @@ bool planner_arena_reuse() { return g_arena_reuse; }
 long long planner_thin_conv_min_pixels() { return g_thin_conv_min_pixels; }
 int planner_host_split_k() { return g_host_split_k; }
 bool planner_commute_pool_conv() { return g_commute_pool_conv; }
-long long planner_separable_max_pixels() { return g_separable_max_pixels; }
 
 Plan build_plan(PlanMode mode, const Json &doc, const Json *extra, int batch, const LaunchChooser &chooser) {
     Planner planner(batch, chooser);
@@ -1238,14 +1152,6 @@ std::string describe_plan(const Plan &plan) {
                 os << ",\"variant\":\"" << conv_variant(c.launch.variant).name << "\",\"split_k\":" << c.launch.split_k
                    << ",\"fusable\":" << (conv_variant(c.launch.variant).fusable() ? "true" : "false");
             }
-        }
-        if (op.conv >= 0 && plan.convs[op.conv].sep_dw >= 0) {
-            const PlanConv &c = plan.convs[op.conv], &dw = plan.convs[c.sep_dw];
-            os << ",\"depthwise\":{\"name\":";
-            json_escape(os, dw.name);
-            os << ",\"h\":" << c.problem.dw_h << ",\"w\":" << c.problem.dw_w << ",\"k\":" << c.problem.dw_k << ",\"s\":" << c.problem.dw_s
-               << ",\"p\":" << c.problem.dw_p << ",\"inputs\":" << c.problem.dw_nsrc << ",\"act\":" << dw.problem.act
-               << ",\"pre_relu\":" << dw.problem.pre_relu << "}";
         }
         if (op.kind == OpKind::Nary) os << ",\"inputs\":" << op.srcs.size() << ",\"accumulate\":" << op.accumulate;
         if (op.kind == OpKind::ConvDepthwise) os << ",\"inputs\":" << (op.srcs.empty() ? 1 : op.srcs.size());

@@ -56,11 +56,6 @@ struct PlanConv {
     bool linear = false;
     size_t zero_bias_off = 0;
     bool thin = false;   // direct path: the kernel for 3 x 3 convolutions of 3-channel images (first layers at large batches)
-    // separable pair (problem.separable()): the depth-wise convolution whose result this 1 x 1 convolution's launch computes
-    // itself (its filters and bias live under that entry; it has no operation of its own), and the argument block of the
-    // depth-wise half in the arena (conv_depthwise_args_floats() floats, written at session setup)
-    int sep_dw = -1;
-    size_t sep_args_off = 0;
 };
 
 struct PlanOp {
@@ -75,9 +70,7 @@ struct PlanOp {
     int conv = -1;        // index into Plan::convs
     int bias_conv = -1;   // Pool behind a commuted convolution: out = act(pool(in) + bias of that convolution)
     PoolProblem pool{};
-    // Nary: inputs; ConvDepthwise of a sum: the views it adds in its loader (else empty); ConvMfma of a separable pair: the same
-    // for its depth-wise half (`in` is the depth-wise input)
-    std::vector<ViewRef> srcs;
+    std::vector<ViewRef> srcs;   // Nary: inputs; ConvDepthwise of a sum: the views it adds in its loader (else empty)
     int multiply = 0, accumulate = 0, act = 0;
     // ConvMfma of a residual unit: out = residual + act(conv + bias), then max(., 0) when post_relu
     bool has_residual = false;
@@ -130,8 +123,5 @@ bool planner_arena_reuse();
 long long planner_thin_conv_min_pixels();
 int planner_host_split_k();   // option host_plan_split_k
 bool planner_commute_pool_conv();   // option commute_pool_conv (default 1): see PlanConv::linear
-// option separable_max_pixels (default 4096): "depth-wise convolution, then 1 x 1 convolution" inside one Sequential become one
-// launch (PlanConv::sep_dw) when the pair has at most this many output pixels (batch x OH x OW); 0 disables it
-long long planner_separable_max_pixels();
 
 }  // namespace ios

@@ -98,7 +98,7 @@ DirectConvArgs make_direct_conv_args(const ConvProblem &p, const TensorView &x, 
     a.nmore = 0;
     for (int s = 0; s < kMaxNaryInputs - 1; s++) {
         a.more[s] = x.ptr;
-        a.more_bs[s] = 0;
+        a.more_bs[s] = x.bstride;
         a.more_bytes[s] = 0;
     }
     *blocks = blocks_for((long long)p.B * p.OC * p.OH * p.OW, 256, 8192);
@@ -124,7 +124,7 @@ void add_dwconv_sources(DirectConvArgs &a, const TensorView *more, int count) {
         const unsigned long long bytes = ((unsigned long long)(p.B - 1) * more[s].bstride + (unsigned long long)p.IC * p.H * p.W) * 4ull;
         if (bytes >= (1ull << 31) || a.x_bytes == 0) throw std::runtime_error("dwconv: summed inputs beyond 31-bit offsets");
         a.more[s] = more[s].ptr;
-        a.more_bs[s] = p.B > 1 ? (int)more[s].bstride : 0;   // (one image: the stride is never used)
+        a.more_bs[s] = more[s].bstride;
         a.more_bytes[s] = (unsigned)bytes;
     }
     a.nmore = count;

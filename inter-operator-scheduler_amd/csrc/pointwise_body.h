@@ -306,7 +306,7 @@ struct DirectConvArgs {
     // depth-wise convolution of a sum: the input is x + more[0] + ... + more[nmore - 1] (added left to right, then the
     // folded ReLU), every view of the shape of x; the reference adds them with a kernel of its own (src/ios/ops.cu:26-48)
     const float *more[kMaxNaryInputs - 1];
-    int more_bs[kMaxNaryInputs - 1];   // batch strides in elements (below 2^29: the views fit 31-bit byte offsets)
+    long long more_bs[kMaxNaryInputs - 1];
     unsigned more_bytes[kMaxNaryInputs - 1];
     int nmore;
 };

@@ -97,8 +97,8 @@ private:
     int share_threads_per_cu_ = 1024;   // resident threads per compute unit the share-class budgets assume (four wavefronts per SIMD)
     void load_tune_cache();
     std::string settings_token() const;
-    float *tune_buf_[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
-    size_t tune_floats_[5] = {0, 0, 0, 0, 0};
+    float *tune_buf_[4] = {nullptr, nullptr, nullptr, nullptr};
+    size_t tune_floats_[4] = {0, 0, 0, 0};
     std::string tune_cache_path_;
     int num_cus_ = 0;
     std::string name_, arch_;
@@ -166,10 +166,6 @@ private:
     void launch_op(const PlanOp &op, int group);   // on stream `group` of the pool
     unsigned *counters_of(const PlanConv &c) const;
     const float *bias_of(const PlanConv &c) const { return base_ + (c.linear ? c.zero_bias_off : c.bias_off); }
-    // separable pair: the argument block of the depth-wise half (in the arena); null for an ordinary convolution
-    const struct DirectConvArgs *depthwise_of(const PlanConv &c) const {
-        return c.sep_dw >= 0 ? reinterpret_cast<const struct DirectConvArgs *>(base_ + c.sep_args_off) : nullptr;
-    }
     void enqueue(bool stage_events);   // issue one forward pass according to the execution mode
     void enqueue_streams(bool stage_events);
     void enqueue_fused(bool stage_events);

@@ -137,7 +137,6 @@ static std::string conv_signature(const ConvProblem &p) {
     std::ostringstream os;
     os << p.B << ' ' << p.IC << ' ' << p.H << ' ' << p.W << ' ' << p.OC << ' ' << p.KH << ' ' << p.KW << ' ' << p.sh << ' ' << p.sw
        << ' ' << p.ph << ' ' << p.pw << ' ' << p.groups;
-    if (p.separable()) os << " dw" << p.dw_k << '/' << p.dw_s << '/' << p.dw_p << '/' << p.dw_h << 'x' << p.dw_w << '/' << p.dw_nsrc;
     return os.str();
 }
 
@@ -224,26 +223,13 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
     const size_t kMaxWorkspace = size_t(96) << 20;   // floats
     TensorView x, y;
-    x.C = p.IC; x.H = p.separable() ? p.dw_h : p.H; x.W = p.separable() ? p.dw_w : p.W; x.bstride = (long long)p.IC * x.H * x.W;
+    x.C = p.IC; x.H = p.H; x.W = p.W; x.bstride = (long long)p.IC * p.H * p.W;
     y.C = p.OC; y.H = p.OH; y.W = p.OW; y.bstride = (long long)p.OC * p.OH * p.OW;
     x.ptr = tuning_buffer(0, (size_t)p.B * x.bstride);
     y.ptr = tuning_buffer(1, (size_t)p.B * y.bstride);
     float *packed = tuning_buffer(2, conv_packed_floats_max(p) + p.OC);
     float *bias = packed + conv_packed_floats_max(p);
     hipStream_t stream = streams_[0];
-    // separable pair: depth-wise filters, bias and the argument block of the depth-wise half (all summed inputs read x)
-    const DirectConvArgs *depthwise = nullptr;
-    if (p.separable()) {
-        const size_t dw_floats = (size_t)p.IC * p.dw_k * p.dw_k + p.IC;
-        float *block = tuning_buffer(4, conv_depthwise_args_floats() + dw_floats);
-        float *dw_w = block + conv_depthwise_args_floats();
-        TensorView more[kMaxNaryInputs];
-        for (int i = 0; i + 1 < p.dw_nsrc; i++) more[i] = x;
-        std::vector<float> host(conv_depthwise_args_floats());
-        fill_conv_depthwise_args(p, x, more, p.dw_nsrc - 1, dw_w, dw_w + (size_t)p.IC * p.dw_k * p.dw_k, 1, ACT_NONE, host.data());
-        IOS_HIP(hipMemcpy(block, host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice));
-        depthwise = reinterpret_cast<const DirectConvArgs *>(block);
-    }
     struct EventPair {   // destroyed on every way out, a failing launch included
         hipEvent_t start = nullptr, stop = nullptr;
         ~EventPair() {
@@ -267,9 +253,9 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
         const size_t ws = conv_workspace_floats(p, l);
         float *workspace = ws ? tuning_buffer(3, ws) : nullptr;
         const SplitKReduce counters = split_reduce(tuning_counters(conv_counter_count(p, l)));
-        launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream, nullptr, false, depthwise);   // warm-up
+        launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream);   // warm-up
         IOS_HIP(hipEventRecord(start, stream));
-        for (int r = 0; r < reps; r++) launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream, nullptr, false, depthwise);
+        for (int r = 0; r < reps; r++) launch_conv_mfma(p, l, x, packed, bias, y, workspace, counters, stream);
         IOS_HIP(hipEventRecord(stop, stream));
         IOS_HIP(hipEventSynchronize(stop));
         float ms = 0.f;
@@ -281,9 +267,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
     float fastest = 1e30f;
     for (int v = 0; v < conv_num_variants(); v++) {
         const ConvVariant &cv = conv_variant(v);
-        if (cv.separable != p.separable()) continue;   // separable pairs have configurations of their own
-        if (cv.precision != (p.separable() ? PREC_FP32 : precision_)) continue;   // the precision mode decides which family of configurations competes
-        if (cv.separable && conv_separable_lds_bytes(p, v) > 64 * 1024) continue;
+        if (cv.precision != precision_) continue;   // the precision mode decides which family of configurations competes
         // tiles more than twice as tall / wide as the problem only waste lanes
         if (cv.BM >= 2 * p.OCg() + 32 || cv.BN >= 2 * p.Npix() + 32) continue;
         int last_effective = -1;
@@ -319,8 +303,7 @@ DeviceContext::TunedConv DeviceContext::tune_conv(const ConvProblem &p) {
         // kernel gains (Inception-v3 at batch 1, same device: 0.379-0.385 ms with it against 0.375-0.377 ms without).
         constexpr float kWideMinMs = 0.012f;
         auto wide_too_short = [&](const Candidate &cand) {
-            // (separable pairs have no other configurations: theirs always compete)
-            return !any_kernel && conv_variant(cand.launch.variant).needs_wide() && !conv_variant(cand.launch.variant).separable && cand.ms < kWideMinMs;
+            return !any_kernel && conv_variant(cand.launch.variant).needs_wide() && cand.ms < kWideMinMs;
         };
         auto eligible = [&](const Candidate &cand, bool fit) {
             if (c == 0) return true;
@@ -384,22 +367,6 @@ ConvLaunch DeviceContext::choose_launch(const ConvProblem &p, int share, bool al
     int cls = 0;
     while (cls + 1 < kShareClasses && (1 << (cls + 1)) <= share) cls++;   // floor(log2(share)), capped
     ConvLaunch launch;
-    // A pinned configuration (option conv_variant) for separable pairs applies to them and to nothing else; any other pinned
-    // configuration or K split, and the reduced-precision modes, make the planner keep the two convolutions of a pair apart
-    // (variant -1 declines: the fused form computes in fp32 and has configurations of its own).
-    const bool pinned_pair = forced_variant_ >= 0 && conv_variant(forced_variant_).separable;
-    if (p.separable()) {
-        if (precision_ != PREC_FP32 || ((forced_variant_ >= 0 || forced_split_k_ > 0) && !pinned_pair) ||
-            (pinned_pair && conv_separable_lds_bytes(p, forced_variant_) > 64 * 1024)) {
-            launch.variant = -1;
-            return launch;
-        }
-        if (pinned_pair) {
-            launch.variant = forced_variant_;
-            launch.split_k = std::max(1, forced_split_k_);
-            return launch;
-        }
-    }
     bool chosen = false;
     if (autotune_) {
         const std::string key = conv_signature(p) + " " + settings_token() + (precision_ == PREC_BF16 ? " bf16" : precision_ == PREC_FP16 ? " fp16" : "");
@@ -413,8 +380,8 @@ ConvLaunch DeviceContext::choose_launch(const ConvProblem &p, int share, bool al
     if (!chosen) {
         launch = conv_pick_launch(p, std::max(1, num_cus_ >> cls), cls > 0, precision_);
     }
-    if (forced_variant_ >= 0 && !pinned_pair) launch.variant = forced_variant_;
-    if (forced_split_k_ > 0 && !pinned_pair) launch.split_k = forced_split_k_;
+    if (forced_variant_ >= 0) launch.variant = forced_variant_;
+    if (forced_split_k_ > 0) launch.split_k = forced_split_k_;
     return launch;
 }
 
@@ -577,18 +544,6 @@ void Session::setup() {
         // split-K tickets start at zero; every launch leaves them at zero again
         if (conv.ctr_count > 0) launch_fill_u32(reinterpret_cast<unsigned *>(base_ + conv.ctr_off), conv.ctr_count, 0u, main);
     }
-    // separable pairs: the argument blocks of the depth-wise halves
-    for (const PlanOp &op : plan_.ops) {
-        if (op.kind != OpKind::ConvMfma || plan_.convs[op.conv].sep_dw < 0) continue;
-        const PlanConv &c = plan_.convs[op.conv], &dw = plan_.convs[c.sep_dw];
-        TensorView more[kMaxNaryInputs];
-        for (size_t i = 1; i < op.srcs.size(); i++) more[i - 1] = tv(op.srcs[i]);
-        std::vector<float> host(conv_depthwise_args_floats());
-        fill_conv_depthwise_args(c.problem, tv(op.in), more, op.srcs.empty() ? 0 : (int)op.srcs.size() - 1, base_ + dw.weight_off, base_ + dw.bias_off,
-                                 dw.problem.pre_relu, dw.problem.act, host.data());
-        IOS_HIP(hipMemcpyAsync(base_ + c.sep_args_off, host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice, main));
-        IOS_HIP(hipStreamSynchronize(main));   // (the copy reads `host`)
-    }
     const size_t num_stages = plan_.stages.size();
     if (static_) {   // no events: everything is issued on the main stream and the host waits for the stream
         IOS_HIP(hipStreamSynchronize(main));
@@ -675,7 +630,7 @@ void Session::launch_op(const PlanOp &op, int group) {
             launch_conv_mfma(c.problem, c.launch, tv(op.in), base_ + c.packed_off, bias_of(c), tv(op.out),
                              c.ws_floats ? base_ + c.ws_off : nullptr, ctx_.split_reduce(counters_of(c), group, !capturing_forks_), stream,
                              op.has_residual ? &residual : nullptr,
-                             op.post_relu != 0, depthwise_of(c));
+                             op.post_relu != 0);
             break;
         }
         case OpKind::ConvDepthwise: {
@@ -807,7 +762,7 @@ void Session::build_fused() {
                         const TensorView residual = op.has_residual ? tv(op.residual) : TensorView{};
                         const ConvDispatch d = make_conv_dispatch(c.problem, c.launch, tv(op.in), base_ + c.packed_off, bias_of(c),
                                                                   tv(op.out), c.ws_floats ? base_ + c.ws_off : nullptr, ctx_.split_reduce(counters_of(c)),
-                                                                  op.has_residual ? &residual : nullptr, op.post_relu != 0, depthwise_of(c));
+                                                                  op.has_residual ? &residual : nullptr, op.post_relu != 0);
                         pend.fusable = conv_variant(d.variant).fusable() && !op.has_residual;   // (the fused kernel holds the plain epilogue)
                         if (!pend.fusable && !solo)
                             throw std::runtime_error(op.has_residual ? std::string("internal: a residual convolution is planned for single-group stages only")
@@ -899,7 +854,6 @@ void Session::build_fused() {
             if (here.empty()) continue;
             // a configuration of the wide-register family beside a 1024-thread body: that family has no such form, the
             // operators of the level are launched one after the other instead (they are independent of each other)
-            // (separable pairs belong to that family too)
             bool needs_wide = false;
             for (Pending *pend : here)
                 needs_wide = needs_wide || (pend->item.kind == WORK_CONV && conv_variant(pend->item.variant).needs_wide());

@@ -42,11 +42,9 @@ def default_options():
     rt.set_option('precision', 'fp32')
     rt.set_option('arena_reuse', 1)
     rt.set_option('thin_conv_min_pixels', 1 << 18)
-    rt.set_option('separable_max_pixels', 4096)
     yield
     rt.set_option('arena_reuse', 1)
     rt.set_option('thin_conv_min_pixels', 1 << 18)
-    rt.set_option('separable_max_pixels', 4096)
     rt.set_option('precision', 'fp32')
     rt.set_option('autotune', 0)
     rt.set_option('conv_variant', -1)
@@ -589,90 +587,8 @@ def separable_graph(in_shape, inputs, relu, oc, window, stride):
     return single_op_graph(in_shape, build)
 
 
-SEPARABLE_CASES = [((312, 7, 7), 8, True, 312, 3, 1, 1), ((200, 9, 9), 3, True, 64, 3, 2, 2), ((78, 28, 28), 2, True, 78, 3, 1, 2),
-                   ((21, 9, 9), 2, False, 33, 3, 2, 3), ((176, 7, 7), 2, False, 176, 5, 1, 1), ((96, 8, 8), 5, True, 96, 5, 1, 3),
-                   ((3, 6, 6), 7, True, 5, 5, 2, 1), ((64, 10, 10), 2, True, 64, 7, 1, 1), ((44, 28, 28), 1, True, 44, 5, 1, 1),
-                   ((11, 31, 31), 1, True, 22, 7, 2, 2), ((88, 14, 14), 1, False, 88, 3, 1, 1), ((156, 14, 14), 4, True, 156, 3, 1, 1)]
-
-
-def test_separable_pairs_run_as_one_launch():
-    """(sum of k values,) (ReLU,) depth-wise convolution, 1 x 1 convolution: one launch, whose blocks compute the depth-wise
-    values they need (windows 3, 5, 7; sums for 3 and 5; the last channels and pixels of a tile are padding)."""
-    for in_shape, inputs, relu, oc, window, stride, batch in SEPARABLE_CASES:
-        graph = separable_graph(in_shape, inputs, relu, oc, window, stride)
-        ops = rt.plan_describe(graph, batch)
-        kinds = [op['kind'] for op in ops]
-        pairs = [op for op in ops if 'depthwise' in op]
-        assert 'conv_depthwise' not in kinds and len(pairs) == 1, (in_shape, kinds)
-        pair = pairs[0]
-        assert pair['variant'].startswith('sq_') and pair['depthwise']['k'] == window and pair['depthwise']['s'] == stride
-        summed_apart = window > 5 and inputs > 1      # 7 x 7 windows keep the summing launch, which then applies the ReLU as well
-        assert pair['depthwise']['inputs'] == (1 if summed_apart else inputs) and pair['depthwise']['pre_relu'] == int(relu and not summed_apart)
-        assert kinds.count('nary') == (1 if window > 5 and inputs > 1 else 0)      # 7 x 7 windows keep the summing launch
-        x = np.random.default_rng(15).standard_normal((batch, *in_shape)).astype(np.float32)
-        want = ios_oracle.run(graph, x)
-        outs = {}
-        for executor in ('streams', 'fused', 'fused_graph', 'graph'):
-            rt.set_option('executor', executor)
-            outs[executor] = rt.graph_inference(graph, batch, x)
-            assert_close(outs[executor], want, f'separable pair {in_shape} k={inputs} {window}x{window} {executor}')
-            np.testing.assert_array_equal(outs[executor], outs['streams'])
-
-
-def test_every_configuration_for_separable_pairs_matches_oracle():
-    """Option conv_variant pinned to a configuration for separable pairs applies to the pairs only; K slices in every form."""
-    names = rt.device_info()['conv_variants']
-    pair_variants = [n for n in names if n.startswith('sq_')]
-    assert len(pair_variants) == 8
-    cases = [SEPARABLE_CASES[i] for i in (0, 1, 5, 7, 8, 11)]
-    graphs = [(separable_graph(*case[:6]), case) for case in cases]
-    for name in pair_variants:
-        for split, reduce in ((1, 'xcd'), (2, 'xcd'), (3, 'inline'), (2, 'kernel')):
-            rt.set_option('conv_variant', names.index(name))
-            rt.set_option('conv_split_k', split)
-            rt.set_option('split_k_reduce', reduce)
-            for graph, case in graphs:
-                in_shape, batch = case[0], case[6]
-                x = np.random.default_rng(17).standard_normal((batch, *in_shape)).astype(np.float32)
-                want = ios_oracle.run(graph, x)
-                outs = {}
-                for executor in ('streams', 'fused'):
-                    rt.set_option('executor', executor)
-                    with rt.Session(graph, batch) as session:
-                        session.load_weights()
-                        pair = [op for op in session.describe() if 'depthwise' in op]
-                        if not pair:      # too wide for this configuration's LDS stage: the pair stays two launches
-                            assert in_shape[0] * int(name.split('n')[1][:2]) * 4 > 30 * 1024, (name, in_shape)
-                            continue
-                        assert pair[0]['variant'] == name and all(op['variant'] != name for op in session.describe() if 'variant' in op and 'depthwise' not in op)
-                        session.set_input(x)
-                        session.run()
-                        outs[executor] = session.output()
-                    assert_close(outs[executor], want, f'{name} split {split} {reduce} {in_shape} {executor}')
-                if len(outs) == 2:
-                    np.testing.assert_array_equal(outs['fused'], outs['streams'])
-
-
-def test_separable_pairs_stay_apart_when_asked_or_large():
-    graph = separable_graph((78, 28, 28), 2, True, 78, 3, 1)
-    assert [op['kind'] for op in rt.plan_describe(graph, 1)].count('conv_depthwise') == 0
-    assert [op['kind'] for op in rt.plan_describe(graph, 16)].count('conv_depthwise') == 1      # 16 x 28 x 28 pixels > 4096
-    rt.set_option('separable_max_pixels', 0)
-    assert [op['kind'] for op in rt.plan_describe(graph, 1)].count('conv_depthwise') == 1
-    rt.set_option('separable_max_pixels', 4096)
-    rt.set_option('precision', 'bf16')      # the fused form computes in fp32: the reduced-precision modes keep two launches
-    x = np.random.default_rng(16).standard_normal((1, 78, 28, 28)).astype(np.float32)
-    with rt.Session(graph, 1) as session:
-        assert [op['kind'] for op in session.describe()].count('conv_depthwise') == 1
-    rt.set_option('precision', 'fp32')
-    rt.set_option('conv_variant', rt.device_info()['conv_variants'].index('wq_m16n16_w16_t16'))      # a pinned configuration too
-    with rt.Session(graph, 1) as session:
-        assert [op['kind'] for op in session.describe()].count('conv_depthwise') == 1
-
-
 def test_depthwise_kernel_adds_up_to_eight_inputs_in_its_loader():
     """(sum of k values,) (ReLU,) depth-wise convolution: no summing launch, no sum tensor (3 x 3 and 5 x 5 windows)."""
-    rt.set_option('separable_max_pixels', 0)      # the depth-wise kernel itself: the pair stays two launches
     for in_shape, inputs, relu, oc, window, stride, batch in [((312, 7, 7), 8, True, 312, 3, 1, 1), ((200, 9, 9), 3, True, 64, 3, 2, 2),
                                                               ((78, 28, 28), 2, True, 78, 3, 1, 2), ((21, 9, 9), 2, False, 33, 3, 2, 3),
                                                               ((176, 7, 7), 2, False, 176, 5, 1, 1), ((96, 8, 8), 5, True, 96, 5, 1, 3),
@@ -711,18 +627,16 @@ def test_depthwise_sums_share_fused_launches_with_other_operators():
     graph = single_op_graph((20, 14, 14), build)
     names = [n.name for n in graph.blocks[0].inner_nodes]
     graph.blocks[0].stages = [[[names[0]], [names[1]]], [[n] for n in names[2:8]], [[graph.blocks[0].exit_node.name]]]
-    for separable in (0, 4096):      # the pairs as two launches each, then as one
-        rt.set_option('separable_max_pixels', separable)
-        for batch in (1, 2):
-            x = np.random.default_rng(13).standard_normal((batch, 20, 14, 14)).astype(np.float32)
-            want = ios_oracle.run(graph, x)
-            outs = {}
-            for executor in ('streams', 'fused', 'fused_graph', 'graph'):
-                rt.set_option('executor', executor)
-                outs[executor] = rt.graph_inference(graph, batch, x)
-                assert_close(outs[executor], want, f'{executor} batch {batch} separable {separable}')
-            for executor in ('fused', 'fused_graph', 'graph'):
-                np.testing.assert_array_equal(outs[executor], outs['streams'])
+    for batch in (1, 2):
+        x = np.random.default_rng(13).standard_normal((batch, 20, 14, 14)).astype(np.float32)
+        want = ios_oracle.run(graph, x)
+        outs = {}
+        for executor in ('streams', 'fused', 'fused_graph', 'graph'):
+            rt.set_option('executor', executor)
+            outs[executor] = rt.graph_inference(graph, batch, x)
+            assert_close(outs[executor], want, f'{executor} batch {batch}')
+        for executor in ('fused', 'fused_graph', 'graph'):
+            np.testing.assert_array_equal(outs[executor], outs['streams'])
 
 
 def test_passes_queued_back_to_back_give_the_result_of_a_single_pass():
